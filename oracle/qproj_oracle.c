@@ -1,0 +1,863 @@
+/*
+ * CPU oracle for the quantized projection path -- see qproj_oracle.h for scope,
+ * provenance and pin status.  TEST INFRASTRUCTURE ONLY.
+ *
+ * Upstream functions restated here live in llama.cpp @ 0b1bad14 (absent from
+ * /root/reference; pinned by /root/reference/inference/native-pin.toml:11-14):
+ *   ggml/src/ggml-common.h      block_q8_0, block_q4_K, block_q6_K, block_q8_K
+ *   ggml/src/ggml-quants.c      quantize_row_*_ref, dequantize_row_*, make_qkx2_quants,
+ *                               make_qx_quants, nearest_int, get_scale_min_k4
+ *   ggml/src/ggml-cpu/quants.c  ggml_vec_dot_*_generic, quantize_row_q8_K
+ *   ggml/src/ggml-cpu/ggml-cpu.c ggml_compute_forward_mul_mat{,_id}
+ *   src/llama-graph.cpp         build_moe_ffn
+ *
+ * Build with -ffp-contract=off: "d*q - m" must stay a multiply followed by a
+ * subtract so that bit-exact dequantization has one meaning.
+ */
+#include "qproj_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#include <time.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+#if defined(__F16C__)
+#include <immintrin.h>
+#endif
+
+/* ---------------------------------------------------------------- sizes */
+
+size_t orc_sizeof_block(int type) {
+    switch (type) {
+    case ORC_TYPE_Q8_0: return sizeof(orc_block_q8_0);
+    case ORC_TYPE_Q4_K: return sizeof(orc_block_q4_K);
+    case ORC_TYPE_Q6_K: return sizeof(orc_block_q6_K);
+    default: return 0;
+    }
+}
+
+int orc_block_elems(int type) {
+    switch (type) {
+    case ORC_TYPE_Q8_0: return ORC_QK8_0;
+    case ORC_TYPE_Q4_K:
+    case ORC_TYPE_Q6_K: return ORC_QK_K;
+    default: return 0;
+    }
+}
+
+size_t orc_row_bytes(int type, int64_t k) {
+    int be = orc_block_elems(type);
+    if (be == 0 || k % be != 0) return 0;
+    return (size_t)(k / be) * orc_sizeof_block(type);
+}
+
+_Static_assert(sizeof(orc_block_q8_0) == 34, "block_q8_0 is 34 bytes");
+_Static_assert(sizeof(orc_block_q4_K) == 144, "block_q4_K is 144 bytes");
+_Static_assert(sizeof(orc_block_q6_K) == 210, "block_q6_K is 210 bytes");
+_Static_assert(sizeof(orc_block_q8_K) == 292, "block_q8_K is 292 bytes");
+
+/* ---------------------------------------------------------------- fp16 */
+
+/* IEEE binary16 -> binary32, exact, subnormals included (ggml GGML_FP16_TO_FP32). */
+float orc_fp16_to_fp32(orc_half h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else { /* subnormal: normalise */
+            int e = -1;
+            do {
+                man <<= 1;
+                e++;
+            } while ((man & 0x400u) == 0);
+            man &= 0x3ffu;
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7f800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+/* binary32 -> binary16, round to nearest even (ggml GGML_FP32_TO_FP16). */
+orc_half orc_fp32_to_fp16(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint32_t sign = (x >> 16) & 0x8000u;
+    uint32_t ax = x & 0x7fffffffu;
+    if (ax >= 0x7f800000u) { /* inf / nan */
+        return (orc_half)(sign | 0x7c00u | ((ax > 0x7f800000u) ? (0x200u | ((ax >> 13) & 0x3ffu)) : 0));
+    }
+    int32_t e = (int32_t)(ax >> 23) - 127 + 15;
+    uint32_t man = ax & 0x7fffffu;
+    if (e >= 31) return (orc_half)(sign | 0x7c00u); /* overflow -> inf */
+    if (e <= 0) {
+        if (e < -10) return (orc_half)sign; /* underflow -> 0 */
+        man |= 0x800000u;
+        uint32_t shift = (uint32_t)(14 - e);
+        uint32_t half = man >> shift;
+        uint32_t rem = man & ((1u << shift) - 1u);
+        uint32_t mid = 1u << (shift - 1);
+        if (rem > mid || (rem == mid && (half & 1u))) half++;
+        return (orc_half)(sign | half);
+    }
+    uint32_t half = ((uint32_t)e << 10) | (man >> 13);
+    uint32_t rem = man & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (half & 1u))) half++; /* may carry into exponent: correct */
+    return (orc_half)(sign | half);
+}
+
+float orc_fp16_to_fp32_f16c(orc_half h) {
+#if defined(__F16C__)
+    return _cvtsh_ss(h);
+#else
+    return orc_fp16_to_fp32(h);
+#endif
+}
+
+orc_half orc_fp32_to_fp16_f16c(float f) {
+#if defined(__F16C__)
+    return (orc_half)_cvtss_sh(f, 0);
+#else
+    return orc_fp32_to_fp16(f);
+#endif
+}
+
+/* ---------------------------------------------------------------- 6-bit scales */
+
+/* ggml-quants.c get_scale_min_k4: sub-block j of a Q4_K super-block keeps a
+ * 6-bit scale and a 6-bit min inside 12 bytes. */
+void orc_get_scale_min_k4(int j, const uint8_t *q, uint8_t *sc, uint8_t *m) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((q[j + 4] & 0x0f) | ((q[j - 4] >> 6) << 4));
+        *m = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+/* inverse of the above, as written by quantize_row_q4_K_ref */
+void orc_pack_scale_min_k4(const uint8_t sc[8], const uint8_t mn[8], uint8_t out[12]) {
+    memset(out, 0, 12);
+    for (int j = 0; j < 8; ++j) {
+        uint8_t ls = sc[j] & 63, lm = mn[j] & 63;
+        if (j < 4) {
+            out[j] |= ls;
+            out[j + 4] |= lm;
+        } else {
+            out[j + 4] = (uint8_t)((ls & 0x0f) | ((lm & 0x0f) << 4));
+            out[j - 4] |= (uint8_t)((ls >> 4) << 6);
+            out[j] |= (uint8_t)((lm >> 4) << 6);
+        }
+    }
+}
+
+/* ---------------------------------------------------------------- dequantize */
+
+/* ggml-quants.c dequantize_row_q8_0: y = q * d */
+void orc_dequantize_row_q8_0(const orc_block_q8_0 *x, float *y, int64_t k) {
+    const int64_t nb = k / ORC_QK8_0;
+    for (int64_t i = 0; i < nb; ++i) {
+        const float d = orc_fp16_to_fp32(x[i].d);
+        for (int j = 0; j < ORC_QK8_0; ++j) y[i * ORC_QK8_0 + j] = x[i].qs[j] * d;
+    }
+}
+
+/* ggml-quants.c dequantize_row_q4_K: y = (d*sc)*q - (dmin*m), multiply then subtract */
+void orc_dequantize_row_q4_K(const orc_block_q4_K *x, float *y, int64_t k) {
+    const int64_t nb = k / ORC_QK_K;
+    for (int64_t i = 0; i < nb; ++i) {
+        const uint8_t *q = x[i].qs;
+        const float d = orc_fp16_to_fp32(x[i].d);
+        const float min = orc_fp16_to_fp32(x[i].dmin);
+        int is = 0;
+        for (int j = 0; j < ORC_QK_K; j += 64) {
+            uint8_t sc, m;
+            orc_get_scale_min_k4(is + 0, x[i].scales, &sc, &m);
+            const float d1 = d * sc;
+            const float m1 = min * m;
+            orc_get_scale_min_k4(is + 1, x[i].scales, &sc, &m);
+            const float d2 = d * sc;
+            const float m2 = min * m;
+            for (int l = 0; l < 32; ++l) *y++ = d1 * (q[l] & 0xF) - m1;
+            for (int l = 0; l < 32; ++l) *y++ = d2 * (q[l] >> 4) - m2;
+            q += 32;
+            is += 2;
+        }
+    }
+}
+
+/* ggml-quants.c dequantize_row_q6_K: y = (d*sc)*(q-32) */
+void orc_dequantize_row_q6_K(const orc_block_q6_K *x, float *y, int64_t k) {
+    const int64_t nb = k / ORC_QK_K;
+    for (int64_t i = 0; i < nb; ++i) {
+        const float d = orc_fp16_to_fp32(x[i].d);
+        const uint8_t *ql = x[i].ql;
+        const uint8_t *qh = x[i].qh;
+        const int8_t *sc = x[i].scales;
+        for (int n = 0; n < ORC_QK_K; n += 128) {
+            for (int l = 0; l < 32; ++l) {
+                const int is = l / 16;
+                const int8_t q1 = (int8_t)((ql[l + 0] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+                const int8_t q2 = (int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                const int8_t q3 = (int8_t)((ql[l + 0] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                const int8_t q4 = (int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+                y[l + 0] = d * sc[is + 0] * q1;
+                y[l + 32] = d * sc[is + 2] * q2;
+                y[l + 64] = d * sc[is + 4] * q3;
+                y[l + 96] = d * sc[is + 6] * q4;
+            }
+            y += 128;
+            ql += 64;
+            qh += 32;
+            sc += 8;
+        }
+    }
+}
+
+void orc_dequantize_row(int type, const void *blocks, float *y, int64_t k) {
+    switch (type) {
+    case ORC_TYPE_Q8_0: orc_dequantize_row_q8_0((const orc_block_q8_0 *)blocks, y, k); break;
+    case ORC_TYPE_Q4_K: orc_dequantize_row_q4_K((const orc_block_q4_K *)blocks, y, k); break;
+    case ORC_TYPE_Q6_K: orc_dequantize_row_q6_K((const orc_block_q6_K *)blocks, y, k); break;
+    default: break;
+    }
+}
+
+/* ---------------------------------------------------------------- quantize */
+
+/* ggml-quants.c nearest_int: round half to even through the 2^23+2^22 trick */
+static inline int nearest_int(float fval) {
+    float val = fval + 12582912.f;
+    int i;
+    memcpy(&i, &val, sizeof(int));
+    return (i & 0x007fffff) - 0x00400000;
+}
+
+#define ORC_MAX(a, b) ((a) > (b) ? (a) : (b))
+#define ORC_MIN(a, b) ((a) < (b) ? (a) : (b))
+#define ORC_GROUP_MAX_EPS 1e-15f
+
+/* ggml-quants.c quantize_row_q8_0_ref: d = amax/127, q = roundf(x * (1/d)) */
+void orc_quantize_row_q8_0(const float *x, orc_block_q8_0 *y, int64_t k) {
+    const int64_t nb = k / ORC_QK8_0;
+    for (int64_t i = 0; i < nb; ++i) {
+        float amax = 0.0f;
+        for (int j = 0; j < ORC_QK8_0; ++j) {
+            const float v = fabsf(x[i * ORC_QK8_0 + j]);
+            amax = ORC_MAX(amax, v);
+        }
+        const float d = amax / ((1 << 7) - 1);
+        const float id = d ? 1.0f / d : 0.0f;
+        y[i].d = orc_fp32_to_fp16(d);
+        for (int j = 0; j < ORC_QK8_0; ++j) {
+            const float x0 = x[i * ORC_QK8_0 + j] * id;
+            y[i].qs[j] = (int8_t)roundf(x0);
+        }
+    }
+}
+
+/* per-32 activation block of the prefill path: like q8_0 but the scale stays
+ * fp32 and the integer sum of the quants is kept for the Q4_K min term. */
+void orc_quantize_row_q8x32(const float *x, orc_block_q8x32 *y, int64_t k) {
+    const int64_t nb = k / 32;
+    for (int64_t i = 0; i < nb; ++i) {
+        float amax = 0.0f;
+        for (int j = 0; j < 32; ++j) {
+            const float v = fabsf(x[i * 32 + j]);
+            amax = ORC_MAX(amax, v);
+        }
+        const float d = amax / 127.0f;
+        const float id = d ? 1.0f / d : 0.0f;
+        int32_t s = 0;
+        for (int j = 0; j < 32; ++j) {
+            const int q = (int)roundf(x[i * 32 + j] * id);
+            y[i].qs[j] = (int8_t)q;
+            s += q;
+        }
+        y[i].d = d;
+        y[i].isum = s;
+    }
+}
+
+/* ggml-cpu/quants.c quantize_row_q8_K (== quantize_row_q8_K_ref) */
+void orc_quantize_row_q8_K(const float *x, orc_block_q8_K *y, int64_t k) {
+    const int64_t nb = k / ORC_QK_K;
+    for (int64_t i = 0; i < nb; ++i) {
+        float max = 0, amax = 0;
+        for (int j = 0; j < ORC_QK_K; ++j) {
+            const float ax = fabsf(x[j]);
+            if (ax > amax) {
+                amax = ax;
+                max = x[j];
+            }
+        }
+        if (!amax) {
+            memset(&y[i], 0, sizeof(y[i]));
+            x += ORC_QK_K;
+            continue;
+        }
+        const float iscale = -127.f / max;
+        for (int j = 0; j < ORC_QK_K; ++j) {
+            const int v = nearest_int(iscale * x[j]);
+            y[i].qs[j] = (int8_t)ORC_MIN(127, v);
+        }
+        for (int j = 0; j < ORC_QK_K / 16; ++j) {
+            int sum = 0;
+            for (int ii = 0; ii < 16; ++ii) sum += y[i].qs[j * 16 + ii];
+            y[i].bsums[j] = (int16_t)sum;
+        }
+        y[i].d = 1 / iscale;
+        x += ORC_QK_K;
+    }
+}
+
+/* ggml-quants.c make_qkx2_quants: weighted affine fit (scale, min<=0) of n
+ * values onto 0..nmax, refined over nstep+1 candidate inverse scales. */
+static float fit_affine_qkx2(int n, int nmax, const float *x, const float *w, uint8_t *L,
+                             float *the_min, uint8_t *Laux, float rmin, float rdelta, int nstep) {
+    float lo = x[0], hi = x[0];
+    float sum_w = w[0];
+    float sum_x = sum_w * x[0];
+    for (int i = 1; i < n; ++i) {
+        if (x[i] < lo) lo = x[i];
+        if (x[i] > hi) hi = x[i];
+        sum_w += w[i];
+        sum_x += w[i] * x[i];
+    }
+    if (lo > 0) lo = 0;
+    if (hi == lo) {
+        for (int i = 0; i < n; ++i) L[i] = 0;
+        *the_min = -lo;
+        return 0.f;
+    }
+    float iscale = nmax / (hi - lo);
+    float scale = 1 / iscale;
+    float best = 0;
+    for (int i = 0; i < n; ++i) {
+        int l = nearest_int(iscale * (x[i] - lo));
+        L[i] = (uint8_t)ORC_MAX(0, ORC_MIN(nmax, l));
+        float diff = scale * L[i] + lo - x[i];
+        best += w[i] * (diff * diff);
+    }
+    for (int is = 0; is <= nstep; ++is) {
+        iscale = (rmin + rdelta * is + nmax) / (hi - lo);
+        float sum_l = 0, sum_l2 = 0, sum_xl = 0;
+        for (int i = 0; i < n; ++i) {
+            int l = nearest_int(iscale * (x[i] - lo));
+            l = ORC_MAX(0, ORC_MIN(nmax, l));
+            Laux[i] = (uint8_t)l;
+            sum_l += w[i] * l;
+            sum_l2 += w[i] * l * l;
+            sum_xl += w[i] * l * x[i];
+        }
+        const float D = sum_w * sum_l2 - sum_l * sum_l;
+        if (D > 0) {
+            float this_scale = (sum_w * sum_xl - sum_x * sum_l) / D;
+            float this_min = (sum_l2 * sum_x - sum_l * sum_xl) / D;
+            if (this_min > 0) {
+                this_min = 0;
+                this_scale = sum_xl / sum_l2;
+            }
+            float err = 0;
+            for (int i = 0; i < n; ++i) {
+                float diff = this_scale * Laux[i] + this_min - x[i];
+                err += w[i] * (diff * diff);
+            }
+            if (err < best) {
+                for (int i = 0; i < n; ++i) L[i] = Laux[i];
+                best = err;
+                scale = this_scale;
+                lo = this_min;
+            }
+        }
+    }
+    *the_min = -lo;
+    return scale;
+}
+
+/* ggml-quants.c quantize_row_q4_K_ref */
+void orc_quantize_row_q4_K(const float *x, orc_block_q4_K *y, int64_t k) {
+    const int64_t nb = k / ORC_QK_K;
+    uint8_t L[ORC_QK_K], Laux[32];
+    float weights[32], mins[8], scales[8];
+    for (int64_t i = 0; i < nb; ++i) {
+        float max_scale = 0, max_min = 0;
+        for (int j = 0; j < 8; ++j) {
+            float sum_x2 = 0;
+            for (int l = 0; l < 32; ++l) sum_x2 += x[32 * j + l] * x[32 * j + l];
+            const float av_x = sqrtf(sum_x2 / 32);
+            for (int l = 0; l < 32; ++l) weights[l] = av_x + fabsf(x[32 * j + l]);
+            scales[j] = fit_affine_qkx2(32, 15, x + 32 * j, weights, L + 32 * j, &mins[j], Laux, -1.f,
+                                        0.1f, 20);
+            if (scales[j] > max_scale) max_scale = scales[j];
+            if (mins[j] > max_min) max_min = mins[j];
+        }
+        const float inv_scale = max_scale > 0 ? 63.f / max_scale : 0.f;
+        const float inv_min = max_min > 0 ? 63.f / max_min : 0.f;
+        uint8_t ls8[8], lm8[8];
+        for (int j = 0; j < 8; ++j) {
+            int ls = nearest_int(inv_scale * scales[j]);
+            int lm = nearest_int(inv_min * mins[j]);
+            ls8[j] = (uint8_t)ORC_MIN(63, ls);
+            lm8[j] = (uint8_t)ORC_MIN(63, lm);
+        }
+        orc_pack_scale_min_k4(ls8, lm8, y[i].scales);
+        y[i].d = orc_fp32_to_fp16(max_scale / 63.f);
+        y[i].dmin = orc_fp32_to_fp16(max_min / 63.f);
+        for (int j = 0; j < 8; ++j) {
+            uint8_t sc, m;
+            orc_get_scale_min_k4(j, y[i].scales, &sc, &m);
+            const float d = orc_fp16_to_fp32(y[i].d) * sc;
+            if (!d) continue;
+            const float dm = orc_fp16_to_fp32(y[i].dmin) * m;
+            for (int ii = 0; ii < 32; ++ii) {
+                int l = nearest_int((x[32 * j + ii] + dm) / d);
+                l = ORC_MAX(0, ORC_MIN(15, l));
+                L[32 * j + ii] = (uint8_t)l;
+            }
+        }
+        uint8_t *q = y[i].qs;
+        for (int j = 0; j < ORC_QK_K; j += 64) {
+            for (int l = 0; l < 32; ++l) q[l] = (uint8_t)(L[j + l] | (L[j + l + 32] << 4));
+            q += 32;
+        }
+        x += ORC_QK_K;
+    }
+}
+
+/* ggml-quants.c make_qx_quants with rmse_type = 1 (weights x^2), no external weights */
+static float fit_symmetric_qx(int n, int nmax, const float *x, int8_t *L) {
+    float max = 0, amax = 0;
+    for (int i = 0; i < n; ++i) {
+        float ax = fabsf(x[i]);
+        if (ax > amax) {
+            amax = ax;
+            max = x[i];
+        }
+    }
+    if (amax < ORC_GROUP_MAX_EPS) {
+        for (int i = 0; i < n; ++i) L[i] = 0;
+        return 0.f;
+    }
+    float iscale = -nmax / max;
+    float sumlx = 0, suml2 = 0;
+    for (int i = 0; i < n; ++i) {
+        int l = nearest_int(iscale * x[i]);
+        l = ORC_MAX(-nmax, ORC_MIN(nmax - 1, l));
+        L[i] = (int8_t)(l + nmax);
+        float w = x[i] * x[i];
+        sumlx += w * x[i] * l;
+        suml2 += w * l * l;
+    }
+    float scale = suml2 ? sumlx / suml2 : 0.0f;
+    float best = scale * sumlx;
+    for (int is = -9; is <= 9; ++is) {
+        if (is == 0) continue;
+        iscale = -(nmax + 0.1f * is) / max;
+        sumlx = suml2 = 0;
+        for (int i = 0; i < n; ++i) {
+            int l = nearest_int(iscale * x[i]);
+            l = ORC_MAX(-nmax, ORC_MIN(nmax - 1, l));
+            float w = x[i] * x[i];
+            sumlx += w * x[i] * l;
+            suml2 += w * l * l;
+        }
+        if (suml2 > 0 && sumlx * sumlx > best * suml2) {
+            for (int i = 0; i < n; ++i) {
+                int l = nearest_int(iscale * x[i]);
+                L[i] = (int8_t)(nmax + ORC_MAX(-nmax, ORC_MIN(nmax - 1, l)));
+            }
+            scale = sumlx / suml2;
+            best = scale * sumlx;
+        }
+    }
+    return scale;
+}
+
+/* ggml-quants.c quantize_row_q6_K_ref */
+void orc_quantize_row_q6_K(const float *x, orc_block_q6_K *y, int64_t k) {
+    const int64_t nb = k / ORC_QK_K;
+    int8_t L[ORC_QK_K];
+    float scales[16];
+    for (int64_t i = 0; i < nb; ++i) {
+        float max_scale = 0, max_abs_scale = 0;
+        for (int ib = 0; ib < 16; ++ib) {
+            const float scale = fit_symmetric_qx(16, 32, x + 16 * ib, L + 16 * ib);
+            scales[ib] = scale;
+            const float a = fabsf(scale);
+            if (a > max_abs_scale) {
+                max_abs_scale = a;
+                max_scale = scale;
+            }
+        }
+        if (max_abs_scale < ORC_GROUP_MAX_EPS) {
+            memset(&y[i], 0, sizeof(y[i]));
+            x += ORC_QK_K;
+            continue;
+        }
+        const float iscale = -128.f / max_scale;
+        y[i].d = orc_fp32_to_fp16(1 / iscale);
+        for (int ib = 0; ib < 16; ++ib)
+            y[i].scales[ib] = (int8_t)ORC_MIN(127, nearest_int(iscale * scales[ib]));
+        for (int j = 0; j < 16; ++j) {
+            const float d = orc_fp16_to_fp32(y[i].d) * y[i].scales[j];
+            if (!d) continue;
+            for (int ii = 0; ii < 16; ++ii) {
+                int l = nearest_int(x[16 * j + ii] / d);
+                l = ORC_MAX(-32, ORC_MIN(31, l));
+                L[16 * j + ii] = (int8_t)(l + 32);
+            }
+        }
+        uint8_t *ql = y[i].ql;
+        uint8_t *qh = y[i].qh;
+        for (int j = 0; j < ORC_QK_K; j += 128) {
+            for (int l = 0; l < 32; ++l) {
+                const uint8_t q1 = L[j + l + 0] & 0xF;
+                const uint8_t q2 = L[j + l + 32] & 0xF;
+                const uint8_t q3 = L[j + l + 64] & 0xF;
+                const uint8_t q4 = L[j + l + 96] & 0xF;
+                ql[l + 0] = (uint8_t)(q1 | (q3 << 4));
+                ql[l + 32] = (uint8_t)(q2 | (q4 << 4));
+                qh[l] = (uint8_t)((L[j + l] >> 4) | ((L[j + l + 32] >> 4) << 2) |
+                                  ((L[j + l + 64] >> 4) << 4) | ((L[j + l + 96] >> 4) << 6));
+            }
+            ql += 64;
+            qh += 32;
+        }
+        x += ORC_QK_K;
+    }
+}
+
+void orc_quantize_row(int type, const float *x, void *blocks, int64_t k) {
+    switch (type) {
+    case ORC_TYPE_Q8_0: orc_quantize_row_q8_0(x, (orc_block_q8_0 *)blocks, k); break;
+    case ORC_TYPE_Q4_K: orc_quantize_row_q4_K(x, (orc_block_q4_K *)blocks, k); break;
+    case ORC_TYPE_Q6_K: orc_quantize_row_q6_K(x, (orc_block_q6_K *)blocks, k); break;
+    default: break;
+    }
+}
+
+void orc_quantize_rows(int type, const float *x, void *blocks, int64_t k, int64_t nrows, int nthreads) {
+    const size_t rb = orc_row_bytes(type, k);
+    if (nthreads < 1) nthreads = 1;
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+    for (int64_t r = 0; r < nrows; ++r)
+        orc_quantize_row(type, x + r * k, (char *)blocks + (size_t)r * rb, k);
+}
+
+/* ---------------------------------------------------------------- dot products */
+
+/* ggml-cpu/quants.c ggml_vec_dot_q8_0_q8_0_generic */
+float orc_vec_dot_q8_0_q8_0(int64_t k, const orc_block_q8_0 *w, const orc_block_q8_0 *a) {
+    const int64_t nb = k / ORC_QK8_0;
+    float sumf = 0;
+    for (int64_t ib = 0; ib < nb; ++ib) {
+        int sumi = 0;
+        for (int j = 0; j < ORC_QK8_0; ++j) sumi += w[ib].qs[j] * a[ib].qs[j];
+        sumf += sumi * (orc_fp16_to_fp32(w[ib].d) * orc_fp16_to_fp32(a[ib].d));
+    }
+    return sumf;
+}
+
+/* ggml-cpu/quants.c ggml_vec_dot_q4_K_q8_K_generic.  Eight interleaved int32
+ * lanes (element index mod 8) carry scale*(q4*q8); each lane is scaled by
+ * d*y.d per super-block into its own fp32 sum; the min term is one fp32
+ * accumulator; the lanes are added to it at the end. */
+float orc_vec_dot_q4_K_q8_K(int64_t k, const orc_block_q4_K *w, const orc_block_q8_K *a) {
+    const int64_t nb = k / ORC_QK_K;
+    float lane_sum[8] = {0};
+    float sumf = 0;
+    for (int64_t i = 0; i < nb; ++i) {
+        int8_t q[ORC_QK_K];
+        const uint8_t *q4 = w[i].qs;
+        for (int c = 0; c < 4; ++c) {
+            for (int l = 0; l < 32; ++l) q[64 * c + l] = (int8_t)(q4[32 * c + l] & 0xF);
+            for (int l = 0; l < 32; ++l) q[64 * c + 32 + l] = (int8_t)(q4[32 * c + l] >> 4);
+        }
+        uint8_t sc[8], mn[8];
+        for (int j = 0; j < 8; ++j) orc_get_scale_min_k4(j, w[i].scales, &sc[j], &mn[j]);
+        int sumi = 0;
+        for (int j = 0; j < 16; ++j) sumi += a[i].bsums[j] * mn[j / 2];
+        int32_t lane[8] = {0};
+        for (int j = 0; j < 8; ++j) {
+            const int32_t scale = sc[j];
+            for (int l = 0; l < 32; ++l) {
+                const int16_t p = (int16_t)(a[i].qs[32 * j + l] * q[32 * j + l]);
+                lane[l & 7] += scale * p;
+            }
+        }
+        const float d = orc_fp16_to_fp32(w[i].d) * a[i].d;
+        for (int l = 0; l < 8; ++l) lane_sum[l] += d * lane[l];
+        const float dmin = orc_fp16_to_fp32(w[i].dmin) * a[i].d;
+        sumf -= dmin * sumi;
+    }
+    for (int l = 0; l < 8; ++l) sumf += lane_sum[l];
+    return sumf;
+}
+
+/* ggml-cpu/quants.c ggml_vec_dot_q6_K_q8_K_generic */
+float orc_vec_dot_q6_K_q8_K(int64_t k, const orc_block_q6_K *w, const orc_block_q8_K *a) {
+    const int64_t nb = k / ORC_QK_K;
+    float lane_sum[8] = {0};
+    for (int64_t i = 0; i < nb; ++i) {
+        int8_t q[ORC_QK_K];
+        const uint8_t *ql = w[i].ql;
+        const uint8_t *qh = w[i].qh;
+        for (int n = 0; n < ORC_QK_K; n += 128) {
+            for (int l = 0; l < 32; ++l) {
+                q[n + l + 0] = (int8_t)((ql[l + 0] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+                q[n + l + 32] = (int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                q[n + l + 64] = (int8_t)((ql[l + 0] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                q[n + l + 96] = (int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+            }
+            ql += 64;
+            qh += 32;
+        }
+        int32_t lane[8] = {0};
+        for (int j = 0; j < 16; ++j) {
+            const int32_t scale = w[i].scales[j];
+            for (int l = 0; l < 16; ++l) {
+                const int16_t p = (int16_t)(a[i].qs[16 * j + l] * q[16 * j + l]);
+                lane[l & 7] += scale * p;
+            }
+        }
+        const float d = orc_fp16_to_fp32(w[i].d) * a[i].d;
+        for (int l = 0; l < 8; ++l) lane_sum[l] += d * lane[l];
+    }
+    float sumf = 0;
+    for (int l = 0; l < 8; ++l) sumf += lane_sum[l];
+    return sumf;
+}
+
+/* Prefill-path dot: activations in per-32 int8 blocks with an fp32 scale.
+ * Integer partial sums per 32 (per 16 for Q6_K) are exact; the fp32 order is
+ * sequential over K.  This format is the benchmark's own prescription (ggml's
+ * GPU backends use the same idea with an fp16 scale), not a ggml CPU routine. */
+float orc_vec_dot_q8x32(int type, int64_t k, const void *wv, const orc_block_q8x32 *a) {
+    float acc = 0;
+    if (type == ORC_TYPE_Q8_0) {
+        const orc_block_q8_0 *w = (const orc_block_q8_0 *)wv;
+        for (int64_t b = 0; b < k / 32; ++b) {
+            int32_t s = 0;
+            for (int l = 0; l < 32; ++l) s += w[b].qs[l] * a[b].qs[l];
+            acc += (orc_fp16_to_fp32(w[b].d) * a[b].d) * (float)s;
+        }
+    } else if (type == ORC_TYPE_Q4_K) {
+        const orc_block_q4_K *w = (const orc_block_q4_K *)wv;
+        for (int64_t i = 0; i < k / ORC_QK_K; ++i) {
+            const float d = orc_fp16_to_fp32(w[i].d);
+            const float dmin = orc_fp16_to_fp32(w[i].dmin);
+            for (int j = 0; j < 8; ++j) {
+                uint8_t sc, m;
+                orc_get_scale_min_k4(j, w[i].scales, &sc, &m);
+                const orc_block_q8x32 *ab = &a[i * 8 + j];
+                const uint8_t *q4 = w[i].qs + 32 * (j / 2);
+                int32_t s = 0;
+                for (int l = 0; l < 32; ++l) {
+                    const int q = (j & 1) ? (q4[l] >> 4) : (q4[l] & 0xF);
+                    s += q * ab->qs[l];
+                }
+                acc += ((d * sc) * ab->d) * (float)s - ((dmin * m) * ab->d) * (float)ab->isum;
+            }
+        }
+    } else if (type == ORC_TYPE_Q6_K) {
+        const orc_block_q6_K *w = (const orc_block_q6_K *)wv;
+        for (int64_t i = 0; i < k / ORC_QK_K; ++i) {
+            int8_t q[ORC_QK_K];
+            const uint8_t *ql = w[i].ql;
+            const uint8_t *qh = w[i].qh;
+            for (int n = 0; n < ORC_QK_K; n += 128) {
+                for (int l = 0; l < 32; ++l) {
+                    q[n + l + 0] = (int8_t)((ql[l + 0] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+                    q[n + l + 32] = (int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                    q[n + l + 64] = (int8_t)((ql[l + 0] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                    q[n + l + 96] = (int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+                }
+                ql += 64;
+                qh += 32;
+            }
+            const float d = orc_fp16_to_fp32(w[i].d);
+            for (int j = 0; j < 16; ++j) {
+                const orc_block_q8x32 *ab = &a[i * 8 + j / 2];
+                int32_t s = 0;
+                for (int l = 0; l < 16; ++l) s += q[16 * j + l] * ab->qs[16 * (j & 1) + l];
+                acc += ((d * w[i].scales[j]) * ab->d) * (float)s;
+            }
+        }
+    }
+    return acc;
+}
+
+/* ---------------------------------------------------------------- mul_mat */
+
+static size_t act_row_bytes(int type, int act, int64_t K) {
+    if (act == ORC_ACT_Q8X32) return (size_t)(K / 32) * sizeof(orc_block_q8x32);
+    if (type == ORC_TYPE_Q8_0) return (size_t)(K / 32) * sizeof(orc_block_q8_0);
+    return (size_t)(K / ORC_QK_K) * sizeof(orc_block_q8_K);
+}
+
+static void quantize_act_row(int type, int act, const float *x, void *out, int64_t K) {
+    if (act == ORC_ACT_Q8X32)
+        orc_quantize_row_q8x32(x, (orc_block_q8x32 *)out, K);
+    else if (type == ORC_TYPE_Q8_0)
+        orc_quantize_row_q8_0(x, (orc_block_q8_0 *)out, K);
+    else
+        orc_quantize_row_q8_K(x, (orc_block_q8_K *)out, K);
+}
+
+static float dot_quantized(int type, int act, int64_t K, const void *wrow, const void *arow) {
+    if (act == ORC_ACT_Q8X32) return orc_vec_dot_q8x32(type, K, wrow, (const orc_block_q8x32 *)arow);
+    switch (type) {
+    case ORC_TYPE_Q8_0:
+        return orc_vec_dot_q8_0_q8_0(K, (const orc_block_q8_0 *)wrow, (const orc_block_q8_0 *)arow);
+    case ORC_TYPE_Q4_K:
+        return orc_vec_dot_q4_K_q8_K(K, (const orc_block_q4_K *)wrow, (const orc_block_q8_K *)arow);
+    default:
+        return orc_vec_dot_q6_K_q8_K(K, (const orc_block_q6_K *)wrow, (const orc_block_q8_K *)arow);
+    }
+}
+
+int orc_mul_mat_f64(int type, const void *w, int64_t K, int64_t N, const float *x, int64_t M,
+                    double *y, int nthreads) {
+    const size_t rb = orc_row_bytes(type, K);
+    if (rb == 0) return -1;
+    if (nthreads < 1) nthreads = 1;
+#pragma omp parallel num_threads(nthreads)
+    {
+        float *row = (float *)malloc((size_t)K * sizeof(float));
+#pragma omp for schedule(static)
+        for (int64_t n = 0; n < N; ++n) {
+            orc_dequantize_row(type, (const char *)w + (size_t)n * rb, row, K);
+            for (int64_t m = 0; m < M; ++m) {
+                const float *xr = x + m * K;
+                double s = 0;
+                for (int64_t kk = 0; kk < K; ++kk) s += (double)row[kk] * (double)xr[kk];
+                y[m * N + n] = s;
+            }
+        }
+        free(row);
+    }
+    return 0;
+}
+
+/* ggml-cpu.c ggml_compute_forward_mul_mat: src1 rows are converted once to the
+ * weight type's vec_dot_type, then every (row of W, row of x) pair is one vec_dot. */
+int orc_mul_mat(int type, const void *w, int64_t K, int64_t N, const float *x, int64_t M, float *y,
+                int act, int nthreads) {
+    const size_t rb = orc_row_bytes(type, K);
+    if (rb == 0) return -1;
+    if (nthreads < 1) nthreads = 1;
+    if (act == ORC_ACT_F64) {
+        double *yd = (double *)malloc((size_t)M * N * sizeof(double));
+        if (!yd) return -2;
+        orc_mul_mat_f64(type, w, K, N, x, M, yd, nthreads);
+        for (int64_t i = 0; i < M * N; ++i) y[i] = (float)yd[i];
+        free(yd);
+        return 0;
+    }
+    const size_t ab = act_row_bytes(type, act, K);
+    char *aq = (char *)malloc(ab * (size_t)M);
+    if (!aq) return -2;
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+    for (int64_t m = 0; m < M; ++m) quantize_act_row(type, act, x + m * K, aq + (size_t)m * ab, K);
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+    for (int64_t n = 0; n < N; ++n) {
+        const void *wrow = (const char *)w + (size_t)n * rb;
+        for (int64_t m = 0; m < M; ++m)
+            y[m * N + n] = dot_quantized(type, act, K, wrow, aq + (size_t)m * ab);
+    }
+    free(aq);
+    return 0;
+}
+
+/* ggml-cpu.c ggml_compute_forward_mul_mat_id: for token b and slot j the row
+ * b[b, j % nb1, :] is multiplied by expert ids[b, j]; dst is [B, n_used, N]. */
+int orc_mul_mat_id(int type, const void *as, int64_t K, int64_t N, int64_t E, const float *b,
+                   int64_t nb1, const int32_t *ids, int64_t n_used, int64_t B, float *y, int act,
+                   int nthreads) {
+    const size_t rb = orc_row_bytes(type, K);
+    if (rb == 0 || (nb1 != 1 && nb1 != n_used)) return -1;
+    for (int64_t i = 0; i < B * n_used; ++i)
+        if (ids[i] < 0 || ids[i] >= E) return -3;
+    const size_t expert_bytes = rb * (size_t)N;
+    for (int64_t t = 0; t < B; ++t) {
+        for (int64_t j = 0; j < n_used; ++j) {
+            const void *we = (const char *)as + (size_t)ids[t * n_used + j] * expert_bytes;
+            const float *xr = b + (t * nb1 + (j % nb1)) * K;
+            int rc = orc_mul_mat(type, we, K, N, xr, 1, y + (t * n_used + j) * N, act, nthreads);
+            if (rc) return rc;
+        }
+    }
+    return 0;
+}
+
+/* llama-graph.cpp build_moe_ffn (SiLU-gated, weights applied after down):
+ *   up = mul_mat_id(up_exps, x); gate = mul_mat_id(gate_exps, x);
+ *   h = silu(gate) * up; e = mul_mat_id(down_exps, h); e *= w; y = e[0] + e[1] + ... */
+int orc_moe_ffn(int type_gate_up, int type_down, const void *gate, const void *up, const void *down,
+                int64_t d_model, int64_t d_ff, int64_t E, const float *x, const int32_t *ids,
+                const float *weights, int64_t n_used, int64_t B, float *y, int act, int nthreads) {
+    const size_t n_slot = (size_t)B * n_used;
+    float *g = (float *)malloc(n_slot * d_ff * sizeof(float));
+    float *u = (float *)malloc(n_slot * d_ff * sizeof(float));
+    float *e = (float *)malloc(n_slot * d_model * sizeof(float));
+    int rc = -2;
+    if (g && u && e) {
+        rc = orc_mul_mat_id(type_gate_up, up, d_model, d_ff, E, x, 1, ids, n_used, B, u, act, nthreads);
+        if (!rc)
+            rc = orc_mul_mat_id(type_gate_up, gate, d_model, d_ff, E, x, 1, ids, n_used, B, g, act,
+                                nthreads);
+        if (!rc) {
+            for (size_t i = 0; i < n_slot * (size_t)d_ff; ++i) {
+                const float gv = g[i];
+                g[i] = (gv / (1.0f + expf(-gv))) * u[i];
+            }
+            rc = orc_mul_mat_id(type_down, down, d_ff, d_model, E, g, n_used, ids, n_used, B, e, act,
+                                nthreads);
+        }
+        if (!rc) {
+            for (int64_t t = 0; t < B; ++t) {
+                for (int64_t c = 0; c < d_model; ++c) {
+                    float s = e[(t * n_used + 0) * d_model + c] * weights[t * n_used + 0];
+                    for (int64_t j = 1; j < n_used; ++j)
+                        s += e[(t * n_used + j) * d_model + c] * weights[t * n_used + j];
+                    y[t * d_model + c] = s;
+                }
+            }
+        }
+    }
+    free(g);
+    free(u);
+    free(e);
+    return rc;
+}
+
+/* ---------------------------------------------------------------- timing */
+
+int orc_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+double orc_time_mul_mat(int type, const void *w, int64_t K, int64_t N, const float *x, int64_t M,
+                        float *y, int act, int nthreads, int reps) {
+    struct timespec t0, t1;
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    for (int r = 0; r < reps; ++r) orc_mul_mat(type, w, K, N, x, M, y, act, nthreads);
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    return (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
+}
