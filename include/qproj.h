@@ -1,0 +1,139 @@
+/*
+ * qproj -- MI355X (gfx950) quantized projection operators behind a plain C ABI.
+ *
+ * The operators keep the semantics of the two ggml graph ops that Magnitude's
+ * engine reaches for every linear layer through its single native call
+ *   context.decode(batch)      /root/reference/inference/crates/icn-engine/src/lib.rs:2264
+ * (-> llama_decode -> ggml backend graph_compute):
+ *   GGML_OP_MUL_MAT    (src0 = W[K,N] quantized, src1 = x[K,M] f32) -> dst[N,M] f32
+ *   GGML_OP_MUL_MAT_ID (as = W[K,N,E], b = x[K,n_used|1,B], ids[n_used,B] i32) -> dst[N,n_used,B]
+ * over GGML_TYPE_Q8_0 / Q4_K / Q6_K weights.  A ggml backend module is what the
+ * reference loads for this work
+ *   load_backends_from_path(<installation>/backends)
+ *                              /root/reference/inference/crates/icn-server/src/main.rs:5290
+ * and each entry point below names the backend-interface member it stands in for.
+ *
+ * Conventions
+ *   - every function returns a qproj_status (0 = ok); nothing aborts or throws across the
+ *     boundary, so a host can run its decode-failure recovery
+ *     (/root/reference/inference/crates/icn-engine/src/lib.rs:1597-1617);
+ *   - weight bytes are handed over on the HOST in GGUF block layout, verbatim, and the
+ *     library owns their device copy (ggml buffer set_tensor);
+ *   - activations, ids and outputs are DEVICE pointers owned by the caller (ggml tensors
+ *     living in backend buffers); all work is enqueued on the context's HIP stream;
+ *   - a context is used by one thread at a time (the reference serialises native calls on one
+ *     executor thread: /root/reference/design/inference/engine.md:49-50).
+ *   - row-major, ggml element order: x is [M][K], y is [M][N], W is N rows of K weights.
+ */
+#ifndef QPROJ_H
+#define QPROJ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct qproj_ctx qproj_ctx;
+typedef struct qproj_weight qproj_weight;
+
+/* values are ggml's enum ggml_type ids, so a GGUF tensor-info type passes through unchanged
+ * (the reference reads them at /root/reference/inference/crates/icn-models/src/gguf.rs:240-279) */
+enum qproj_type { QPROJ_TYPE_Q8_0 = 8, QPROJ_TYPE_Q4_K = 12, QPROJ_TYPE_Q6_K = 14 };
+
+enum qproj_status {
+    QPROJ_OK = 0,
+    QPROJ_ERR_INVALID_ARG = 1, /* null pointer, bad shape, unsupported type                 */
+    QPROJ_ERR_HIP = 2,         /* a HIP runtime call failed; see qproj_last_error           */
+    QPROJ_ERR_OOM = 3,         /* device allocation failed                                   */
+    QPROJ_ERR_UNSUPPORTED = 4, /* valid request this build has no kernel for                */
+    QPROJ_ERR_NO_DEVICE = 5    /* no gfx950 device visible                                   */
+};
+
+/* How a mul_mat treats its f32 activations.
+ *   GGML  : rows are quantized to the weight type's ggml vec_dot_type first (Q8_0 blocks for Q8_0
+ *           weights, Q8_K super-blocks for Q4_K/Q6_K) and the dot products are integer, exactly as
+ *           ggml's CPU backend computes MUL_MAT.  This is the drop-in mode.
+ *   F32   : fp32 activations times dequantized weights, fp32 accumulation (no activation rounding).
+ *   Q8X32 : rows are quantized to per-32 int8 blocks with an fp32 scale; int8 MFMA for large M.
+ */
+enum qproj_act { QPROJ_ACT_GGML = 0, QPROJ_ACT_F32 = 1, QPROJ_ACT_Q8X32 = 2 };
+
+/* ggml_backend_reg / ggml_backend_dev: number of usable gfx950 devices. */
+int qproj_device_count(int *count);
+
+/* ggml_backend_dev_init.  `stream` is a hipStream_t to enqueue on, or NULL for a stream the
+ * context creates (default priority) and owns. */
+int qproj_ctx_create(int device, void *stream, qproj_ctx **out);
+int qproj_ctx_destroy(qproj_ctx *ctx);
+/* ggml_backend_synchronize */
+int qproj_sync(qproj_ctx *ctx);
+/* text of the most recent failure on this context ("" if none); never NULL */
+const char *qproj_last_error(const qproj_ctx *ctx);
+/* the stream work is enqueued on (hipStream_t) */
+void *qproj_stream(const qproj_ctx *ctx);
+
+/* bytes of one row of K weights in GGUF layout; 0 if K is not a multiple of the block */
+size_t qproj_row_bytes(int type, int64_t K);
+
+/* ggml_backend_buffer set_tensor for a quantized weight: copies n_expert * N rows of K weights
+ * (GGUF layout, expert-major) to the device.  Q8_0 and Q6_K blocks are re-laid out into
+ * same-size aligned planes on the way; qproj_download returns the original bytes. */
+int qproj_upload(qproj_ctx *ctx, int type, int64_t K, int64_t N, int64_t n_expert,
+                 const void *gguf_bytes, qproj_weight **out);
+/* same, source already on the device (GGUF layout) */
+int qproj_upload_from_device(qproj_ctx *ctx, int type, int64_t K, int64_t N, int64_t n_expert,
+                             const void *gguf_bytes_dev, qproj_weight **out);
+/* ggml_backend_buffer get_tensor: GGUF-layout bytes back to the host */
+int qproj_download(qproj_ctx *ctx, const qproj_weight *w, void *gguf_bytes_out);
+int qproj_weight_free(qproj_ctx *ctx, qproj_weight *w);
+int qproj_weight_info(const qproj_weight *w, int *type, int64_t *K, int64_t *N, int64_t *n_expert,
+                      size_t *gguf_bytes);
+
+/* ggml to_float (dequantize_row_*): out_dev = f32 [n_expert*N][K], bit-exact with ggml's
+ * dequantize_row_q8_0 / q4_K / q6_K. */
+int qproj_dequantize(qproj_ctx *ctx, const qproj_weight *w, float *out_dev);
+
+/* ggml from_float of the activation side (quantize_row_q8_0 / quantize_row_q8_K) or the per-32
+ * prefill format, for M rows of K floats.  `kind` = QPROJ_ACT_GGML with `wtype` selecting Q8_0 vs
+ * Q8_K, or QPROJ_ACT_Q8X32.  Output planes in `out_dev` (size from qproj_act_bytes):
+ *   Q8_0  : int8 qs[M][K] | f32 d[M][K/32]   (d already rounded through fp16)
+ *   Q8_K  : int8 qs[M][K] | f32 d[M][K/256] | int16 bsums[M][K/16]
+ *   Q8X32 : int8 qs[M][K] | f32 d[M][K/32]  | int32 isum[M][K/32]
+ * each plane starting at a 256-byte aligned offset, in that order. */
+size_t qproj_act_bytes(int kind, int wtype, int64_t M, int64_t K);
+int qproj_quantize_activations(qproj_ctx *ctx, int kind, int wtype, const float *x_dev, int64_t M,
+                               int64_t K, void *out_dev);
+
+/* GGML_OP_MUL_MAT: y_dev[M][N] = x_dev[M][K] . W^T.  Picks the decode (M=1), small-batch
+ * (M<=16) or prefill kernel from M.  W must have n_expert == 1. */
+int qproj_mul_mat(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int64_t M, float *y_dev,
+                  int act);
+
+/* Several MUL_MATs that share one activation (q/k/v, gate/up) in one launch: y_dev[i] is
+ * [M][N_i].  Same results as n separate qproj_mul_mat calls. */
+int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev,
+                        int64_t M, float *const *y_dev, int act);
+
+/* GGML_OP_MUL_MAT_ID: ids_dev = int32 [B][n_used]; x_dev = f32 [B][nb1][K] with nb1 in
+ * {1, n_used}; y_dev = f32 [B][n_used][N].  Expert ids outside [0, n_expert) are an error
+ * reported by the next qproj_sync (the ids live on the device). */
+int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w_exps, const float *x_dev, int64_t nb1,
+                     const int32_t *ids_dev, int64_t n_used, int64_t B, float *y_dev, int act);
+
+/* The MoE feed-forward of llama.cpp's build_moe_ffn, fused:
+ *   y[b] = sum_j weights[b][j] * down_e( silu(gate_e x_b) * (up_e x_b) ),  e = ids[b][j]
+ * x_dev f32 [B][d_model]; ids_dev int32 [B][n_used]; weights_dev f32 [B][n_used];
+ * y_dev f32 [B][d_model].  gate/up are [d_model -> d_ff], down is [d_ff -> d_model]. */
+int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate_exps, const qproj_weight *up_exps,
+                  const qproj_weight *down_exps, const float *x_dev, const int32_t *ids_dev,
+                  const float *weights_dev, int64_t n_used, int64_t B, float *y_dev, int act);
+
+/* library build tag: "qproj-<version>-gfx950" */
+const char *qproj_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

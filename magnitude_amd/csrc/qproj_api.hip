@@ -1,0 +1,583 @@
+// C ABI of the qproj library: contexts, weight upload, operator dispatch.
+#include "../../include/qproj.h"
+
+#include <stdio.h>
+#include <string.h>
+
+#include <algorithm>
+#include <new>
+#include <string>
+
+#include "qproj_internal.h"
+
+using namespace qproj;
+
+struct qproj_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool own_stream = false;
+    std::string err;
+    uint8_t *ws = nullptr;      // scratch: quantized activations, MoE lists and intermediates
+    size_t ws_bytes = 0;
+    int32_t *flag_dev = nullptr;  // raised by kernels that meet bad device-side input
+};
+
+struct qproj_weight {
+    int type = 0;
+    int64_t K = 0, N = 0, E = 0;
+    size_t gguf_bytes = 0;
+    uint8_t *dev = nullptr;
+    size_t dev_bytes = 0;
+    WeightView view{};
+};
+
+namespace {
+
+constexpr size_t kAlign = 256;
+inline size_t align_up(size_t v) { return (v + kAlign - 1) / kAlign * kAlign; }
+
+int fail(qproj_ctx *ctx, int status, const char *what, hipError_t e = hipSuccess) {
+    if (ctx) {
+        char buf[512];
+        if (e != hipSuccess)
+            snprintf(buf, sizeof buf, "%s: %s", what, hipGetErrorString(e));
+        else
+            snprintf(buf, sizeof buf, "%s", what);
+        ctx->err = buf;
+    }
+    return status;
+}
+
+#define QP_HIP(ctx, call)                                                         \
+    do {                                                                          \
+        hipError_t e_ = (call);                                                   \
+        if (e_ != hipSuccess) {                                                   \
+            (void)hipGetLastError();                                              \
+            return fail(ctx, e_ == hipErrorOutOfMemory ? QPROJ_ERR_OOM : QPROJ_ERR_HIP, #call, e_); \
+        }                                                                         \
+    } while (0)
+
+bool type_ok(int t) { return t == kTypeQ8_0 || t == kTypeQ4_K || t == kTypeQ6_K; }
+int block_elems(int t) { return t == kTypeQ8_0 ? 32 : 256; }
+size_t block_bytes(int t) { return t == kTypeQ8_0 ? 34 : (t == kTypeQ4_K ? 144 : 210); }
+
+int ensure_ws(qproj_ctx *ctx, size_t bytes) {
+    if (bytes <= ctx->ws_bytes) return QPROJ_OK;
+    if (ctx->ws) {
+        QP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        QP_HIP(ctx, hipFree(ctx->ws));
+        ctx->ws = nullptr;
+        ctx->ws_bytes = 0;
+    }
+    const size_t want = align_up(bytes + bytes / 4);
+    QP_HIP(ctx, hipMalloc((void **)&ctx->ws, want));
+    ctx->ws_bytes = want;
+    return QPROJ_OK;
+}
+
+// planes of a quantized-activation buffer, in the order the header documents
+struct ActPlanes {
+    size_t off_qs = 0, off_d = 0, off_aux = 0, total = 0;
+    int kind = 0;
+};
+
+int act_kind_for(int act, int wtype) {
+    if (act == kActQ8X32) return kActKindQ8X32;
+    return wtype == kTypeQ8_0 ? kActKindQ8_0 : kActKindQ8_K;
+}
+
+ActPlanes act_planes(int kind, int64_t M, int64_t K) {
+    ActPlanes p;
+    p.kind = kind;
+    p.off_qs = 0;
+    p.off_d = align_up((size_t)(M * K));
+    const int64_t dblk = kind == kActKindQ8_K ? 256 : 32;
+    p.off_aux = p.off_d + align_up((size_t)(M * (K / dblk)) * 4);
+    size_t aux = 0;
+    if (kind == kActKindQ8_K) aux = (size_t)(M * (K / 16)) * 2;
+    if (kind == kActKindQ8X32) aux = (size_t)(M * (K / 32)) * 4;
+    p.total = p.off_aux + align_up(aux);
+    return p;
+}
+
+ActView act_view(const ActPlanes &p, uint8_t *base, int64_t K) {
+    ActView a{};
+    a.kind = p.kind;
+    a.K = K;
+    a.qs = reinterpret_cast<const int8_t *>(base + p.off_qs);
+    a.d = reinterpret_cast<const float *>(base + p.off_d);
+    a.bsums = p.kind == kActKindQ8_K ? reinterpret_cast<const int16_t *>(base + p.off_aux) : nullptr;
+    a.isum = p.kind == kActKindQ8X32 ? reinterpret_cast<const int32_t *>(base + p.off_aux) : nullptr;
+    return a;
+}
+
+hipError_t run_quantize(qproj_ctx *ctx, const ActPlanes &p, uint8_t *base, const float *x, int64_t M, int64_t K) {
+    return launch_quantize_act(p.kind, x, M, K, reinterpret_cast<int8_t *>(base + p.off_qs),
+                               reinterpret_cast<float *>(base + p.off_d),
+                               reinterpret_cast<int16_t *>(base + p.off_aux),
+                               reinterpret_cast<int32_t *>(base + p.off_aux), ctx->stream);
+}
+
+ActView act_rows(const ActView &a, int64_t m0) {
+    ActView r = a;
+    const int64_t dblk = a.kind == kActKindQ8_K ? 256 : 32;
+    r.qs = a.qs + m0 * a.K;
+    r.d = a.d + m0 * (a.K / dblk);
+    if (a.bsums) r.bsums = a.bsums + m0 * (a.K / 16);
+    if (a.isum) r.isum = a.isum + m0 * (a.K / 32);
+    return r;
+}
+
+int pow2_ceil(int64_t m) {
+    int p = 1;
+    while (p < m) p <<= 1;
+    return p;
+}
+
+int make_view(qproj_weight *w) {
+    WeightView &v = w->view;
+    v = WeightView{};
+    v.type = w->type;
+    v.K = w->K;
+    v.N = w->N;
+    v.E = w->E;
+    v.nb = w->K / block_elems(w->type);
+    const int64_t rows = w->N * w->E;
+    const size_t nblk = (size_t)(rows * v.nb);
+    uint8_t *b = w->dev;
+    if (w->type == kTypeQ4_K) {
+        v.q4k = b;
+        w->dev_bytes = nblk * 144;
+    } else if (w->type == kTypeQ8_0) {
+        v.q8_qs = reinterpret_cast<const int8_t *>(b);
+        const size_t o = align_up(nblk * 32);
+        v.q8_d = reinterpret_cast<const uint16_t *>(b + o);
+        w->dev_bytes = o + nblk * 2;
+    } else {
+        v.q6_ql = b;
+        size_t o = align_up(nblk * 128);
+        v.q6_qh = b + o;
+        o += align_up(nblk * 64);
+        v.q6_sc = reinterpret_cast<const int8_t *>(b + o);
+        o += align_up(nblk * 16);
+        v.q6_d = reinterpret_cast<const uint16_t *>(b + o);
+        w->dev_bytes = o + nblk * 2;
+    }
+    return QPROJ_OK;
+}
+
+size_t planes_bytes(int type, size_t nblk) {
+    if (type == kTypeQ4_K) return nblk * 144;
+    if (type == kTypeQ8_0) return align_up(nblk * 32) + nblk * 2;
+    return align_up(nblk * 128) + align_up(nblk * 64) + align_up(nblk * 16) + nblk * 2;
+}
+
+int upload_common(qproj_ctx *ctx, int type, int64_t K, int64_t N, int64_t n_expert, const void *src,
+                  bool src_on_device, qproj_weight **out) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (!out || !src) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_upload: null argument");
+    *out = nullptr;
+    if (!type_ok(type)) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_upload: unsupported weight type");
+    if (K <= 0 || N <= 0 || n_expert <= 0 || K % block_elems(type) != 0)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_upload: K must be a positive multiple of the block size");
+    if (K > (int64_t)1 << 24 || N * n_expert > (int64_t)1 << 31)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_upload: shape too large");
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    qproj_weight *w = new (std::nothrow) qproj_weight();
+    if (!w) return fail(ctx, QPROJ_ERR_OOM, "qproj_upload: host allocation failed");
+    w->type = type;
+    w->K = K;
+    w->N = N;
+    w->E = n_expert;
+    const size_t nblk = (size_t)(N * n_expert) * (size_t)(K / block_elems(type));
+    w->gguf_bytes = nblk * block_bytes(type);
+    const size_t dev_bytes = planes_bytes(type, nblk);
+    hipError_t e = hipMalloc((void **)&w->dev, dev_bytes);
+    if (e != hipSuccess) {
+        delete w;
+        (void)hipGetLastError();
+        return fail(ctx, QPROJ_ERR_OOM, "qproj_upload: hipMalloc", e);
+    }
+    make_view(w);
+    int rc = QPROJ_OK;
+    if (type == kTypeQ4_K) {
+        e = hipMemcpyAsync(w->dev, src, w->gguf_bytes, src_on_device ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice,
+                           ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e != hipSuccess) rc = fail(ctx, QPROJ_ERR_HIP, "qproj_upload: copy", e);
+    } else {
+        uint8_t *staging = nullptr;
+        const uint8_t *gg = static_cast<const uint8_t *>(src);
+        if (!src_on_device) {
+            e = hipMalloc((void **)&staging, w->gguf_bytes);
+            if (e == hipSuccess) e = hipMemcpyAsync(staging, src, w->gguf_bytes, hipMemcpyHostToDevice, ctx->stream);
+            gg = staging;
+        }
+        if (e == hipSuccess) e = launch_repack_to_planes(type, gg, w->dev, w->view, (int64_t)nblk, ctx->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (staging) (void)hipFree(staging);
+        if (e != hipSuccess) rc = fail(ctx, e == hipErrorOutOfMemory ? QPROJ_ERR_OOM : QPROJ_ERR_HIP, "qproj_upload: repack", e);
+    }
+    if (rc != QPROJ_OK) {
+        (void)hipGetLastError();
+        (void)hipFree(w->dev);
+        delete w;
+        return rc;
+    }
+    *out = w;
+    return QPROJ_OK;
+}
+
+// dense mul_mat over quantized activations already sitting in `a` (M rows)
+int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
+                    float *const *y) {
+    for (int64_t m0 = 0; m0 < M; m0 += 16) {
+        const int64_t mc = std::min<int64_t>(16, M - m0);
+        GemvArgs g{};
+        g.n_targets = n;
+        for (int i = 0; i < n; ++i) {
+            g.t[i].w = w[i]->view;
+            g.t[i].y = y[i] + m0 * w[i]->N;
+        }
+        g.a = act_rows(a, m0);
+        g.M = (int)mc;
+        g.x_div = 1;
+        QP_HIP(ctx, launch_gemv_q8act(g, pow2_ceil(mc), 1, ctx->stream));
+    }
+    return QPROJ_OK;
+}
+
+int grouped_mt(int64_t n_pairs, int64_t E) {
+    if (n_pairs * 4 <= E) return 1;
+    if (n_pairs <= E) return 2;
+    if (n_pairs <= 4 * E) return 4;
+    if (n_pairs <= 8 * E) return 8;
+    return 16;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *qproj_version(void) { return "qproj-0.1-gfx950"; }
+
+int qproj_device_count(int *count) {
+    if (!count) return QPROJ_ERR_INVALID_ARG;
+    *count = 0;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) {
+        (void)hipGetLastError();
+        return QPROJ_ERR_NO_DEVICE;
+    }
+    int ok = 0;
+    for (int i = 0; i < n; ++i) {
+        hipDeviceProp_t p;
+        if (hipGetDeviceProperties(&p, i) == hipSuccess && strncmp(p.gcnArchName, "gfx950", 6) == 0) ok++;
+    }
+    *count = ok;
+    return ok > 0 ? QPROJ_OK : QPROJ_ERR_NO_DEVICE;
+}
+
+int qproj_ctx_create(int device, void *stream, qproj_ctx **out) {
+    if (!out) return QPROJ_ERR_INVALID_ARG;
+    *out = nullptr;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n <= 0) {
+        (void)hipGetLastError();
+        return QPROJ_ERR_NO_DEVICE;
+    }
+    if (device < 0 || device >= n) return QPROJ_ERR_INVALID_ARG;
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, device) != hipSuccess) return QPROJ_ERR_HIP;
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0) return QPROJ_ERR_NO_DEVICE;  // kernels exist for gfx950 only
+    qproj_ctx *ctx = new (std::nothrow) qproj_ctx();
+    if (!ctx) return QPROJ_ERR_OOM;
+    ctx->device = device;
+    if (hipSetDevice(device) != hipSuccess) {
+        delete ctx;
+        return QPROJ_ERR_HIP;
+    }
+    if (stream) {
+        ctx->stream = static_cast<hipStream_t>(stream);
+    } else {
+        if (hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking) != hipSuccess) {
+            delete ctx;
+            return QPROJ_ERR_HIP;
+        }
+        ctx->own_stream = true;
+    }
+    if (hipMalloc((void **)&ctx->flag_dev, 256) != hipSuccess ||
+        hipMemsetAsync(ctx->flag_dev, 0, 256, ctx->stream) != hipSuccess ||
+        hipStreamSynchronize(ctx->stream) != hipSuccess) {
+        if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return QPROJ_ERR_HIP;
+    }
+    *out = ctx;
+    return QPROJ_OK;
+}
+
+int qproj_ctx_destroy(qproj_ctx *ctx) {
+    if (!ctx) return QPROJ_OK;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->ws) (void)hipFree(ctx->ws);
+    if (ctx->flag_dev) (void)hipFree(ctx->flag_dev);
+    if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return QPROJ_OK;
+}
+
+int qproj_sync(qproj_ctx *ctx) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    int32_t flag = 0;
+    QP_HIP(ctx, hipMemcpyAsync(&flag, ctx->flag_dev, sizeof flag, hipMemcpyDeviceToHost, ctx->stream));
+    QP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (flag) {
+        QP_HIP(ctx, hipMemsetAsync(ctx->flag_dev, 0, sizeof flag, ctx->stream));
+        QP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "expert id outside [0, n_expert) in a MUL_MAT_ID batch");
+    }
+    return QPROJ_OK;
+}
+
+const char *qproj_last_error(const qproj_ctx *ctx) { return ctx ? ctx->err.c_str() : "null context"; }
+
+void *qproj_stream(const qproj_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+size_t qproj_row_bytes(int type, int64_t K) {
+    if (!type_ok(type) || K <= 0 || K % block_elems(type) != 0) return 0;
+    return (size_t)(K / block_elems(type)) * block_bytes(type);
+}
+
+int qproj_upload(qproj_ctx *ctx, int type, int64_t K, int64_t N, int64_t n_expert, const void *gguf_bytes,
+                 qproj_weight **out) {
+    return upload_common(ctx, type, K, N, n_expert, gguf_bytes, false, out);
+}
+
+int qproj_upload_from_device(qproj_ctx *ctx, int type, int64_t K, int64_t N, int64_t n_expert,
+                             const void *gguf_bytes_dev, qproj_weight **out) {
+    return upload_common(ctx, type, K, N, n_expert, gguf_bytes_dev, true, out);
+}
+
+int qproj_download(qproj_ctx *ctx, const qproj_weight *w, void *out) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (!w || !out) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_download: null argument");
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    if (w->type == kTypeQ4_K) {
+        QP_HIP(ctx, hipMemcpyAsync(out, w->dev, w->gguf_bytes, hipMemcpyDeviceToHost, ctx->stream));
+        QP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        return QPROJ_OK;
+    }
+    uint8_t *staging = nullptr;
+    QP_HIP(ctx, hipMalloc((void **)&staging, w->gguf_bytes));
+    const int64_t nblk = w->N * w->E * w->view.nb;
+    hipError_t e = launch_repack_to_gguf(w->type, w->view, staging, nblk, ctx->stream);
+    if (e == hipSuccess) e = hipMemcpyAsync(out, staging, w->gguf_bytes, hipMemcpyDeviceToHost, ctx->stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    (void)hipFree(staging);
+    if (e != hipSuccess) return fail(ctx, QPROJ_ERR_HIP, "qproj_download", e);
+    return QPROJ_OK;
+}
+
+int qproj_weight_free(qproj_ctx *ctx, qproj_weight *w) {
+    if (!w) return QPROJ_OK;
+    if (ctx) {
+        (void)hipSetDevice(ctx->device);
+        (void)hipStreamSynchronize(ctx->stream);
+    }
+    if (w->dev) (void)hipFree(w->dev);
+    delete w;
+    return QPROJ_OK;
+}
+
+int qproj_weight_info(const qproj_weight *w, int *type, int64_t *K, int64_t *N, int64_t *n_expert,
+                      size_t *gguf_bytes) {
+    if (!w) return QPROJ_ERR_INVALID_ARG;
+    if (type) *type = w->type;
+    if (K) *K = w->K;
+    if (N) *N = w->N;
+    if (n_expert) *n_expert = w->E;
+    if (gguf_bytes) *gguf_bytes = w->gguf_bytes;
+    return QPROJ_OK;
+}
+
+int qproj_dequantize(qproj_ctx *ctx, const qproj_weight *w, float *out_dev) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (!w || !out_dev) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_dequantize: null argument");
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    QP_HIP(ctx, launch_dequantize(w->view, out_dev, ctx->stream));
+    return QPROJ_OK;
+}
+
+size_t qproj_act_bytes(int kind, int wtype, int64_t M, int64_t K) {
+    if (M <= 0 || K <= 0) return 0;
+    if (kind != kActGGML && kind != kActQ8X32) return 0;
+    const int k = act_kind_for(kind, wtype);
+    if (K % (k == kActKindQ8_K ? 256 : 32) != 0) return 0;
+    return act_planes(k, M, K).total;
+}
+
+int qproj_quantize_activations(qproj_ctx *ctx, int kind, int wtype, const float *x_dev, int64_t M, int64_t K,
+                               void *out_dev) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (!x_dev || !out_dev) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_quantize_activations: null argument");
+    if (qproj_act_bytes(kind, wtype, M, K) == 0)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_quantize_activations: bad kind or shape");
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    const ActPlanes p = act_planes(act_kind_for(kind, wtype), M, K);
+    QP_HIP(ctx, run_quantize(ctx, p, static_cast<uint8_t *>(out_dev), x_dev, M, K));
+    return QPROJ_OK;
+}
+
+int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
+                        float *const *y_dev, int act) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (n <= 0 || n > kMaxTargets || !w || !y_dev || !x_dev)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: null argument or more than 4 tensors");
+    if (M < 0) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: negative M");
+    for (int i = 0; i < n; ++i) {
+        if (!w[i] || !y_dev[i]) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: null tensor");
+        if (w[i]->E != 1) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: expert tensors need qproj_mul_mat_id");
+        if (w[i]->K != w[0]->K || w[i]->type != w[0]->type)
+            return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat_multi: tensors must share K and type");
+    }
+    if (M == 0) return QPROJ_OK;
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    const int64_t K = w[0]->K;
+    if (act == kActGGML || act == kActQ8X32) {
+        if (act == kActQ8X32 && w[0]->type != kTypeQ4_K)
+            return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat: the per-32 int8 path is built for Q4_K weights");
+        const ActPlanes p = act_planes(act_kind_for(act, w[0]->type), M, K);
+        int rc = ensure_ws(ctx, p.total);
+        if (rc) return rc;
+        QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, M, K));
+        const ActView a = act_view(p, ctx->ws, K);
+        if (act == kActGGML) return run_dense_q8act(ctx, n, w, a, M, y_dev);
+        for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], ctx->stream));
+        return QPROJ_OK;
+    }
+    if (act == kActF32) {
+        for (int64_t m0 = 0; m0 < M; m0 += 4) {
+            const int64_t mc = std::min<int64_t>(4, M - m0);
+            GemvArgs g{};
+            g.n_targets = n;
+            for (int i = 0; i < n; ++i) {
+                g.t[i].w = w[i]->view;
+                g.t[i].y = y_dev[i] + m0 * w[i]->N;
+            }
+            g.x = x_dev + m0 * K;
+            g.M = (int)mc;
+            g.x_div = 1;
+            QP_HIP(ctx, launch_gemv_f32(g, pow2_ceil(mc), 1, ctx->stream));
+        }
+        return QPROJ_OK;
+    }
+    return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: unknown activation mode");
+}
+
+int qproj_mul_mat(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int64_t M, float *y_dev, int act) {
+    const qproj_weight *ws[1] = {w};
+    float *ys[1] = {y_dev};
+    return qproj_mul_mat_multi(ctx, 1, ws, x_dev, M, ys, act);
+}
+
+int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int64_t nb1,
+                     const int32_t *ids_dev, int64_t n_used, int64_t B, float *y_dev, int act) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (!w || !x_dev || !ids_dev || !y_dev) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat_id: null argument");
+    if (n_used <= 0 || B < 0 || (nb1 != 1 && nb1 != n_used))
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat_id: nb1 must be 1 or n_used");
+    if (act != kActGGML) return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat_id: only the ggml activation mode");
+    if (B == 0) return QPROJ_OK;
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    const int64_t K = w->K, n_pairs = B * n_used, rows = B * nb1;
+    const ActPlanes p = act_planes(act_kind_for(act, w->type), rows, K);
+    const size_t off_order = p.total;
+    const size_t off_offsets = off_order + align_up((size_t)n_pairs * 4);
+    const size_t total = off_offsets + align_up((size_t)(w->E + 1) * 4);
+    int rc = ensure_ws(ctx, total);
+    if (rc) return rc;
+    QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, rows, K));
+    int32_t *order = reinterpret_cast<int32_t *>(ctx->ws + off_order);
+    int32_t *offsets = reinterpret_cast<int32_t *>(ctx->ws + off_offsets);
+    QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, w->E, order, offsets, ctx->flag_dev, ctx->stream));
+    GemvArgs g{};
+    g.n_targets = 1;
+    g.t[0].w = w->view;
+    g.t[0].y = y_dev;
+    g.a = act_view(p, ctx->ws, K);
+    g.order = order;
+    g.offsets = offsets;
+    g.x_div = nb1 == 1 ? (int)n_used : 1;
+    QP_HIP(ctx, launch_gemv_q8act(g, grouped_mt(n_pairs, w->E), (int)w->E, ctx->stream));
+    return QPROJ_OK;
+}
+
+int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, const qproj_weight *down,
+                  const float *x_dev, const int32_t *ids_dev, const float *weights_dev, int64_t n_used, int64_t B,
+                  float *y_dev, int act) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (!gate || !up || !down || !x_dev || !ids_dev || !weights_dev || !y_dev)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_moe_ffn: null argument");
+    if (act != kActGGML) return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_moe_ffn: only the ggml activation mode");
+    const int64_t d_model = gate->K, d_ff = gate->N, E = gate->E;
+    if (up->K != d_model || up->N != d_ff || up->E != E || up->type != gate->type || down->K != d_ff ||
+        down->N != d_model || down->E != E || n_used <= 0 || B < 0)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_moe_ffn: gate/up/down shapes do not agree");
+    if (d_ff % block_elems(down->type) != 0 || (down->type != kTypeQ8_0 && d_ff % 256 != 0))
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_moe_ffn: d_ff must be a multiple of the block size");
+    if (B == 0) return QPROJ_OK;
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    const int64_t n_pairs = B * n_used;
+    const ActPlanes px = act_planes(act_kind_for(act, gate->type), B, d_model);
+    const ActPlanes ph = act_planes(act_kind_for(act, down->type), n_pairs, d_ff);
+    size_t off = px.total;
+    const size_t off_order = off;
+    off += align_up((size_t)n_pairs * 4);
+    const size_t off_offsets = off;
+    off += align_up((size_t)(E + 1) * 4);
+    const size_t off_h = off;
+    off += align_up((size_t)(n_pairs * d_ff) * 4);
+    const size_t off_hq = off;
+    off += ph.total;
+    const size_t off_e = off;
+    off += align_up((size_t)(n_pairs * d_model) * 4);
+    int rc = ensure_ws(ctx, off);
+    if (rc) return rc;
+    uint8_t *ws = ctx->ws;
+    int32_t *order = reinterpret_cast<int32_t *>(ws + off_order);
+    int32_t *offsets = reinterpret_cast<int32_t *>(ws + off_offsets);
+    float *h = reinterpret_cast<float *>(ws + off_h);
+    float *e = reinterpret_cast<float *>(ws + off_e);
+    const int mt = grouped_mt(n_pairs, E);
+
+    QP_HIP(ctx, run_quantize(ctx, px, ws, x_dev, B, d_model));
+    QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, E, order, offsets, ctx->flag_dev, ctx->stream));
+    GemvArgs g{};
+    g.n_targets = 2;
+    g.t[0].w = gate->view;
+    g.t[0].y = h;
+    g.t[1].w = up->view;
+    g.t[1].y = h;
+    g.a = act_view(px, ws, d_model);
+    g.order = order;
+    g.offsets = offsets;
+    g.x_div = (int)n_used;
+    QP_HIP(ctx, launch_moe_swiglu_gemv(g, mt, (int)E, ctx->stream));
+    QP_HIP(ctx, run_quantize(ctx, ph, ws + off_hq, h, n_pairs, d_ff));
+    GemvArgs gd{};
+    gd.n_targets = 1;
+    gd.t[0].w = down->view;
+    gd.t[0].y = e;
+    gd.a = act_view(ph, ws + off_hq, d_ff);
+    gd.order = order;
+    gd.offsets = offsets;
+    gd.x_div = 1;
+    QP_HIP(ctx, launch_gemv_q8act(gd, mt, (int)E, ctx->stream));
+    QP_HIP(ctx, launch_moe_combine(e, weights_dev, B, n_used, d_model, y_dev, ctx->stream));
+    return QPROJ_OK;
+}
+
+}  // extern "C"

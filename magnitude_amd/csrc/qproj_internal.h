@@ -1,0 +1,86 @@
+// Host/device shared declarations of the qproj library (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace qproj {
+
+constexpr int kTypeQ8_0 = 8;
+constexpr int kTypeQ4_K = 12;
+constexpr int kTypeQ6_K = 14;
+
+constexpr int kActGGML = 0;
+constexpr int kActF32 = 1;
+constexpr int kActQ8X32 = 2;
+
+constexpr int kWave = 64;
+
+// Device-side view of an uploaded weight.  Q4_K keeps the GGUF block layout (144-byte
+// blocks are 16-byte aligned as they are).  Q8_0 and Q6_K blocks (34 and 210 bytes) are only
+// 2-byte aligned in GGUF, so upload splits every field into its own contiguous plane, same
+// total bytes, which makes every vector load naturally aligned and coalesced.
+struct WeightView {
+    int type;
+    int64_t K, N, E;       // N rows per expert, E experts; rows are indexed e*N + n
+    int64_t nb;            // blocks per row (K/32 for Q8_0, K/256 otherwise)
+    const uint8_t *q4k;    // Q4_K: [rows][nb][144]
+    const int8_t *q8_qs;   // Q8_0: [rows][K]
+    const uint16_t *q8_d;  // Q8_0: [rows][nb] fp16
+    const uint8_t *q6_ql;  // Q6_K: [rows][nb][128]
+    const uint8_t *q6_qh;  // Q6_K: [rows][nb][64]
+    const int8_t *q6_sc;   // Q6_K: [rows][nb][16]
+    const uint16_t *q6_d;  // Q6_K: [rows][nb] fp16
+};
+
+// Quantized activations, plane per field (row stride in elements is K, K/blk, ...).
+struct ActView {
+    int kind;              // 0: Q8_0 blocks, 1: Q8_K super-blocks, 2: Q8X32
+    int64_t K;
+    const int8_t *qs;      // [rows][K]
+    const float *d;        // [rows][K/32] (Q8_0, Q8X32) or [rows][K/256] (Q8_K)
+    const int16_t *bsums;  // Q8_K: [rows][K/16]
+    const int32_t *isum;   // Q8X32: [rows][K/32]
+};
+constexpr int kActKindQ8_0 = 0;
+constexpr int kActKindQ8_K = 1;
+constexpr int kActKindQ8X32 = 2;
+
+// One (weight, output) pair of a multi-tensor launch.
+struct GemvTarget {
+    WeightView w;
+    float *y;              // [rows][N]
+    int first_block;       // first blockIdx.x that belongs to this target
+};
+constexpr int kMaxTargets = 4;
+
+struct GemvArgs {
+    int n_targets;
+    GemvTarget t[kMaxTargets];
+    ActView a;
+    const float *x;        // f32 activations (F32 mode) [rows][K]
+    int M;                 // activation rows in this launch (dense mode), <= MT
+    // expert-grouped mode (MUL_MAT_ID); null order = dense
+    const int32_t *order;   // pair indices sorted by expert
+    const int32_t *offsets; // [E+1] ranges into order
+    int x_div;              // activation row of pair p is p / x_div
+};
+
+// ---- launchers (each returns the hipError_t of the launch) ----
+hipError_t launch_dequantize(const WeightView &w, float *out, hipStream_t s);
+hipError_t launch_repack_to_planes(int type, const uint8_t *gguf, uint8_t *planes_base, const WeightView &w,
+                                   int64_t n_blocks, hipStream_t s);
+hipError_t launch_repack_to_gguf(int type, const WeightView &w, uint8_t *gguf, int64_t n_blocks, hipStream_t s);
+hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
+                               int16_t *bsums, int32_t *isum, hipStream_t s);
+hipError_t launch_gemv_q8act(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
+hipError_t launch_gemv_f32(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
+hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_expert, int32_t *order,
+                            int32_t *offsets, int32_t *error_flag, hipStream_t s);
+hipError_t launch_moe_swiglu_gemv(const GemvArgs &gate_up, int mt, int n_experts_grid, hipStream_t s);
+hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, int64_t n_used, int64_t N,
+                              float *y, hipStream_t s);
+hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
+
+}  // namespace qproj
