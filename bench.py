@@ -1,0 +1,328 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized projection path on one MI355X.
+
+A "step" is one decoded token's pass over the projections of a 32-layer 8B-class dense model in
+Q4_K_M (config 2 of BASELINE.json, repeated over 32 DISTINCT layers = 4.41 GB of weights so that
+every step streams from HBM, not from the 256 MB Infinity Cache): per layer q/k/v (one launch),
+o, gate/up (one launch) in Q4_K and down in Q6_K, each preceded by the activation quantizer, in
+the ggml activation mode (the reference CPU path's arithmetic).  `value` is algorithmic GGUF bytes
+per step / time.  Extra legs report the dominant kernel against the HBM roofline, the int8-MFMA
+prefill GEMM (config 4), the MoE feed-forward (config 5) and the CPU oracle on the host cores.
+
+    python bench.py --gpus 1 --steps 20 --warmup 3 [--legs step,roofline,prefill,moe,cpu]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+INT8_PEAK_TOPS = 5000.0
+Q4_K, Q6_K, Q8_0 = 12, 14, 8
+D_MODEL, D_KV, D_FF = 4096, 1024, 14336
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def gguf_bytes(qtype, n, k):
+    return n * (k // (32 if qtype == Q8_0 else 256)) * {Q8_0: 34, Q4_K: 144, Q6_K: 210}[qtype]
+
+
+def gemv_bytes(qtype, n, k, m=1):
+    """algorithmic bytes of one projection: GGUF weight bytes + fp32 activations in + fp32 out"""
+    return gguf_bytes(qtype, n, k) + m * k * 4 + m * n * 4
+
+
+LAYER_TENSORS = [("q", Q4_K, D_MODEL, D_MODEL), ("k", Q4_K, D_KV, D_MODEL), ("v", Q4_K, D_KV, D_MODEL),
+                 ("o", Q4_K, D_MODEL, D_MODEL), ("gate", Q4_K, D_FF, D_MODEL), ("up", Q4_K, D_FF, D_MODEL),
+                 ("down", Q6_K, D_MODEL, D_FF)]
+LAYER_BYTES = sum(gemv_bytes(t, n, k) for _, t, n, k in LAYER_TENSORS)
+LAYER_WEIGHT_BYTES = sum(gguf_bytes(t, n, k) for _, t, n, k in LAYER_TENSORS)
+
+
+class Timer:
+    """HIP events on the stream the library launches on."""
+
+    def __init__(self, torch, stream):
+        self.torch, self.stream = torch, stream
+
+    def time_ms(self, fn, iters):
+        t = self.torch
+        with t.cuda.stream(self.stream):
+            a, b = t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True)
+            a.record(self.stream)
+            for _ in range(iters):
+                fn()
+            b.record(self.stream)
+        b.synchronize()
+        return a.elapsed_time(b) / iters
+
+
+def capture(torch, stream, fn):
+    """Captures fn() (launches on `stream` only) into a HIP graph; returns replay() or None."""
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            fn()
+        return g.replay
+    except Exception as e:  # capture is an optimisation of the launch path, not of the kernels
+        log(f"[bench] graph capture unavailable ({type(e).__name__}: {e}); timing eager launches")
+        try:
+            torch.cuda.synchronize()
+        except Exception:
+            pass
+        return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--layers", type=int, default=32)
+    ap.add_argument("--legs", default="step,roofline,prefill,moe,cpu")
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--split-quantize", action="store_true",
+                    help="run the activation quantizer as a separate launch instead of inside the projection kernel")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy (counter calibration for rocprofv3 --pmc)")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (no sharding, no collectives); use --gpus 1", file=sys.stderr)
+        return 2
+    legs = set(args.legs.split(","))
+
+    import torch
+
+    from magnitude_amd import ACT_GGML, ACT_Q8X32, Context, synth
+
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.Stream(device=dev)
+    ctx = Context(0, stream=stream.cuda_stream)
+    timer = Timer(torch, stream)
+    props = torch.cuda.get_device_properties(0)
+    log(f"[bench] device {props.name} ({getattr(props, 'gcnArchName', '?')}), {props.multi_processor_count} CUs")
+
+    out = {
+        "metric": "Q4_K GEMV achieved HBM GB/s (% peak) + prefill GEMM TOPS, 8B shapes",
+        "value": None, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 x int4/int6 weights -> int32 dot, fp32 scale (u8 bytes streamed)",
+        "data": "synthetic: N(0,0.02) weights quantized to GGUF Q4_K/Q6_K on the device, N(0,1) fp32 activations",
+        "config": {"workload": "configs[1]: Q4_K_M decode projections (q,k,v,o,gate,up Q4_K; down Q6_K), batch 1, "
+                               f"d_model 4096, FFN 14336, {args.layers} distinct layers per step",
+                   "layers": args.layers, "act_mode": "ggml (Q8_K activations, integer dots)",
+                   "launches_per_layer": ("4 quantize + 4 projection" if args.split_quantize else
+                                          "4 (q/k/v and gate/up share a launch; activations quantized in the kernel prologue)")},
+    }
+
+    # ------------------------------------------------------------------ weights
+    L = args.layers
+    layers = []
+    need_layers = bool(legs & {"step", "roofline", "cpu"})
+    if need_layers:
+        t0 = time.time()
+        for l in range(L):
+            lw = {}
+            for i, (name, qt, n, k) in enumerate(LAYER_TENSORS):
+                blocks = synth.random_weight(qt, n, k, seed=1000 * l + i, device=dev)
+                lw[name] = ctx.upload_from_device(qt, k, n, blocks)
+                del blocks
+            layers.append(lw)
+        torch.cuda.synchronize()
+        log(f"[bench] {L} layers of weights ({L * LAYER_WEIGHT_BYTES / 1e9:.2f} GB) ready in {time.time() - t0:.1f}s")
+
+    g = torch.Generator(device=dev).manual_seed(7)
+    x_attn = torch.randn((1, D_MODEL), generator=g, device=dev)
+    x_o = torch.randn((1, D_MODEL), generator=g, device=dev)
+    x_ffn = torch.randn((1, D_MODEL), generator=g, device=dev)
+    x_down = torch.randn((1, D_FF), generator=g, device=dev)
+    lib = ctx.lib
+    abuf = [torch.empty(int(lib.qproj_act_bytes(ACT_GGML, qt, 1, k)), dtype=torch.uint8, device=dev)
+            for qt, k in ((Q4_K, D_MODEL), (Q4_K, D_MODEL), (Q4_K, D_MODEL), (Q6_K, D_FF))]
+    y = {name: torch.empty((1, n), device=dev) for name, _, n, _ in LAYER_TENSORS}
+    torch.cuda.synchronize()
+
+    groups = [("qkv", ["q", "k", "v"], x_attn, 0), ("o", ["o"], x_o, 1), ("gate_up", ["gate", "up"], x_ffn, 2),
+              ("down", ["down"], x_down, 3)]
+
+    def launch(lw, grp, fused):
+        _, names, x, ai = grp
+        ws = [lw[n] for n in names]
+        ys = [y[n] for n in names]
+        if fused:      # one launch: the kernel quantizes the activation row in its prologue
+            ctx.mul_mat_multi(ws, x, ACT_GGML, outs=ys, sync=False)
+        else:          # activation quantizer as its own launch, then the projection
+            ctx.quantize_activations_raw(x, ACT_GGML, ws[0].qtype, out=abuf[ai], sync=False)
+            ctx.mul_mat_quantized(ws, abuf[ai], ACT_GGML, 1, ys, sync=False)
+
+    def layer_pass(lw):
+        for grp in groups:
+            launch(lw, grp, not args.split_quantize)
+
+    def step():
+        for lw in layers:
+            layer_pass(lw)
+
+    # ------------------------------------------------------------------ step leg (headline)
+    if "step" in legs:
+        step()
+        ctx.sync()
+        run = None if args.no_graph else capture(torch, stream, step)
+        out["config"]["hip_graph"] = run is not None
+        run = run or step
+        for _ in range(args.warmup):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            run()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+        bytes_step = L * LAYER_BYTES
+        out["ms_per_step"] = dt * 1e3
+        out["value"] = bytes_step / dt / 1e9
+        out["pct_hbm_peak"] = 100.0 * out["value"] / HBM_PEAK_GBS
+        out["tokens_per_s_projection_only"] = 1.0 / dt
+        out["bytes_per_step"] = bytes_step
+        log(f"[bench] step: {dt * 1e3:.3f} ms  {out['value']:.0f} GB/s ({out['pct_hbm_peak']:.1f}% of 8 TB/s)  "
+            f"{1.0 / dt:.0f} tok/s (projections only)")
+
+    # ------------------------------------------------------------------ roofline leg: dominant kernel
+    if "roofline" in legs:
+        reps = max(5, args.steps)
+        per = {}
+        for grp in groups:
+            def all_layers(grp=grp):
+                for lw in layers:
+                    launch(lw, grp, not args.split_quantize)
+            all_layers()
+            ctx.sync()
+            run = None if args.no_graph else capture(torch, stream, all_layers)
+            run = run or all_layers
+            for _ in range(3):
+                run()
+            torch.cuda.synchronize()
+            ms = timer.time_ms(run, reps) / L
+            nbytes = sum(gemv_bytes(lw_t, n, k) for nm, lw_t, n, k in LAYER_TENSORS if nm in grp[1]) \
+                - (len(grp[1]) - 1) * grp[2].numel() * 4      # the shared activation row is read once
+            per[grp[0]] = {"us_per_launch": ms * 1e3, "bytes_per_launch": nbytes,
+                           "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+            log(f"[bench] kernel {grp[0]:8s}: {ms * 1e3:7.2f} us  {per[grp[0]]['GBps']:6.0f} GB/s "
+                f"({100 * per[grp[0]]['frac_hbm_peak']:.1f}% of peak)")
+        dom = per["gate_up"]
+        out["roofline"] = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": dom["frac_hbm_peak"], "traffic": None,
+                           "kernel": "gemv_decode_kernel<Q4_K, M=1>: gate+up (2 x 4096->14336) in one launch, "
+                                     "activation quantized in the prologue",
+                           "bytes_per_launch": dom["bytes_per_launch"], "us_per_launch": dom["us_per_launch"],
+                           "launches_timed": reps * L, "other_kernels": {k: v for k, v in per.items() if k != "gate_up"}}
+        if args.calib_copy:
+            a = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+            b = torch.empty_like(a)
+            with torch.cuda.stream(stream):
+                for _ in range(5):
+                    b.copy_(a)
+            torch.cuda.synchronize()
+
+    # ------------------------------------------------------------------ prefill leg (config 4)
+    if "prefill" in legs:
+        res = []
+        for (k, n) in ((4096, 14336), (14336, 4096), (4096, 4096)):
+            blocks = synth.random_weight(Q4_K, n, k, seed=77 + n, device=dev)
+            w = ctx.upload_from_device(Q4_K, k, n, blocks)
+            del blocks
+            for m in (512, 2048, 4096):
+                x = torch.randn((m, k), generator=g, device=dev)
+                cols = torch.randperm(k, generator=g, device=dev)[: k // 100]
+                x[:, cols] *= 20.0
+                yb = torch.empty((m, n), device=dev)
+                qb = torch.empty(int(lib.qproj_act_bytes(ACT_Q8X32, Q4_K, m, k)), dtype=torch.uint8, device=dev)
+                torch.cuda.synchronize()
+                fq = lambda: ctx.quantize_activations_raw(x, ACT_Q8X32, Q4_K, out=qb, sync=False)
+                fg = lambda: ctx.mul_mat_quantized([w], qb, ACT_Q8X32, m, [yb], sync=False)
+                fq(); fg(); ctx.sync()
+                it = 5 if m * n * k > 1e11 else 10
+                tq = timer.time_ms(fq, it)
+                tg = timer.time_ms(fg, it)
+                ops = 2.0 * m * n * k
+                res.append({"M": m, "K": k, "N": n, "gemm_ms": tg, "quantize_ms": tq,
+                            "gemm_tops": ops / (tg * 1e-3) / 1e12,
+                            "end_to_end_tops": ops / ((tg + tq) * 1e-3) / 1e12,
+                            "frac_int8_peak": ops / (tg * 1e-3) / 1e12 / INT8_PEAK_TOPS})
+                log(f"[bench] prefill M={m} K={k} N={n}: gemm {tg:.3f} ms = {res[-1]['gemm_tops']:.1f} TOPS "
+                    f"({100 * res[-1]['frac_int8_peak']:.1f}% of int8 peak), quantize {tq:.3f} ms")
+                del x, yb, qb
+            w.free()
+        head = [r for r in res if (r["M"], r["K"], r["N"]) == (4096, 4096, 14336)][0]
+        out["prefill"] = {"act_format": "per-32 int8 + fp32 scale", "mfma": "v_mfma_i32_32x32x32_i8",
+                          "headline_tops": head["gemm_tops"], "headline_frac_int8_peak": head["frac_int8_peak"],
+                          "peak_tops": INT8_PEAK_TOPS, "shapes": res}
+
+    # ------------------------------------------------------------------ MoE leg (config 5)
+    if "moe" in legs:
+        E, top, dm, dff = 128, 8, 2048, 768
+        exps = {}
+        for i, (name, n, k) in enumerate((("gate", dff, dm), ("up", dff, dm), ("down", dm, dff))):
+            blocks = synth.random_weight(Q4_K, E * n, k, seed=500 + i, device=dev)
+            exps[name] = ctx.upload_from_device(Q4_K, k, n, blocks, n_expert=E)
+            del blocks
+        per_expert = 2 * gguf_bytes(Q4_K, dff, dm) + gguf_bytes(Q4_K, dm, dff)
+        res = []
+        for B in (1, 8, 64):
+            ids = torch.stack([torch.randperm(E, generator=g, device=dev)[:top] for _ in range(B)]).to(torch.int32)
+            wts = torch.softmax(torch.randn((B, top), generator=g, device=dev), dim=1)
+            x = torch.randn((B, dm), generator=g, device=dev)
+            distinct = int(torch.unique(ids).numel())
+            torch.cuda.synchronize()
+            f = lambda: ctx.moe_ffn(exps["gate"], exps["up"], exps["down"], x, ids, wts, ACT_GGML, sync=False)
+            f(); ctx.sync()
+            ms = timer.time_ms(f, 20)
+            byts = distinct * per_expert + B * dm * 4 * 2
+            res.append({"B": B, "distinct_experts": distinct, "ms": ms, "GBps": byts / (ms * 1e-3) / 1e9,
+                        "frac_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
+            log(f"[bench] moe B={B}: {ms * 1e3:.1f} us, {distinct} experts, {res[-1]['GBps']:.0f} GB/s")
+        out["moe"] = {"experts": E, "top": top, "d_model": dm, "d_ff": dff, "batches": res,
+                      "note": "5 launches per call, eager; not rotated out of the Infinity Cache"}
+        for w in exps.values():
+            w.free()
+
+    # ------------------------------------------------------------------ CPU baseline (oracle, host cores)
+    if "cpu" in legs:
+        from oracle import oracle as orc
+        import numpy as np
+        orc.build()
+        nl = min(4, L)
+        host = [[(qt, n, k, ctx.download(layers[l][name])) for name, qt, n, k in LAYER_TENSORS] for l in range(nl)]
+        xs = {D_MODEL: x_attn.cpu().numpy(), D_FF: x_down.cpu().numpy()}
+        threads = min(orc.max_threads(), 16)
+        t_end = time.time() + args.cpu_seconds
+        passes, spent = 0, 0.0
+        while passes < 2 or time.time() < t_end:
+            for lw in host:
+                for qt, n, k, blocks in lw:
+                    spent += orc.time_mul_mat(qt, blocks, k, xs[k], orc.ACT_GGML, threads, 1)
+            passes += 1
+        cpu_gbs = passes * nl * LAYER_BYTES / spent / 1e9
+        out["cpu_baseline"] = {"value": cpu_gbs, "unit": "GB/s", "cores": threads, "kind": "port",
+                               "sample": f"{passes} passes over {nl} of the same layers (7 projections each, M=1, "
+                                         f"ggml activation mode), {spent:.1f} s of OpenMP C on the host",
+                               "host_cpus": os.cpu_count()}
+        log(f"[bench] cpu baseline: {cpu_gbs:.2f} GB/s on {threads} threads")
+
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -116,6 +116,12 @@ int qproj_mul_mat(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int
 int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev,
                         int64_t M, float *const *y_dev, int act);
 
+/* The second half of a MUL_MAT on its own: `act_dev` holds M rows already quantized by
+ * qproj_quantize_activations(kind, type of w[0], ...).  ggml converts src1 once per MUL_MAT; a
+ * caller that feeds one activation to several weights (q/k/v) converts once and calls this. */
+int qproj_mul_mat_quantized(qproj_ctx *ctx, int n, const qproj_weight *const *w, const void *act_dev,
+                            int kind, int64_t M, float *const *y_dev);
+
 /* GGML_OP_MUL_MAT_ID: ids_dev = int32 [B][n_used]; x_dev = f32 [B][nb1][K] with nb1 in
  * {1, n_used}; y_dev = f32 [B][n_used][N].  Expert ids outside [0, n_expert) are an error
  * reported by the next qproj_sync (the ids live on the device). */

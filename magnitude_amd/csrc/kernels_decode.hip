@@ -1,0 +1,338 @@
+// Decode-regime projection (1..4 activation rows): a persistent, software-pipelined GEMV.
+//
+// One 1024-thread workgroup per CU.  The workgroup quantizes the activation rows (or copies
+// rows quantized earlier) into LDS once; when a single K-chunk covers the whole row every lane
+// then keeps its slice of the activations in registers for the rest of the kernel.  Each of
+// the 16 waves walks its own run of consecutive weight rows, R at a time, with two register
+// buffers filled and drained alternately, so the loads of step i+1 are outstanding while step i
+// is computed.  Row addresses are a wave-uniform base plus 32-bit offsets, so the scalar unit
+// does a handful of operations per step and the vector unit only the dot products.
+#include "actquant_device.h"
+#include "gemv_frags.h"
+
+namespace qproj {
+
+namespace {
+
+constexpr int kDecodeThreads = 1024;
+constexpr int kDecodeWaves = kDecodeThreads / 64;
+
+// activations into LDS: FUSE quantizes fp32 rows here; otherwise planes quantized earlier are copied
+template <int QT, int MT, bool FUSE>
+__device__ __forceinline__ void stage_activations(uint8_t *smem, const GemvArgs &args, int64_t K, int kpad) {
+    constexpr int BLK = Geo<QT>::kBlk;
+    int8_t *sq = reinterpret_cast<int8_t *>(smem);
+    float *sd = reinterpret_cast<float *>(smem + MT * kpad);
+    int16_t *sb = reinterpret_cast<int16_t *>(smem + MT * kpad + MT * (kpad / BLK) * 4);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int m = 0; m < MT; ++m) {
+        const bool have = m < args.M;
+        if (FUSE) {
+            const float *x = args.x + (int64_t)m * K;
+            const int n_chunks = (int)((K + 255) / 256);
+            for (int ch = wave; ch < n_chunks; ch += kDecodeWaves) {
+                const int e0 = ch * 256 + 4 * lane;
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (have && e0 < K) v = *reinterpret_cast<const float4 *>(x + e0);
+                if (QT == kTypeQ8_0) {
+                    int s;
+                    float dd;
+                    const uint32_t packed = wave_quantize_q8_32(v, s, dd);
+                    if (e0 < K) {
+                        *reinterpret_cast<uint32_t *>(sq + m * kpad + e0) = packed;
+                        if ((lane & 7) == 0) sd[m * (kpad / 32) + (e0 >> 5)] = h2f(f2h(dd));
+                    }
+                } else {
+                    int bsum;
+                    float dd;
+                    const uint32_t packed = wave_quantize_q8k(v, lane, bsum, dd);
+                    *reinterpret_cast<uint32_t *>(sq + m * kpad + e0) = packed;
+                    if ((lane & 3) == 0) sb[m * (kpad / 16) + ch * 16 + (lane >> 2)] = (int16_t)bsum;
+                    if (lane == 0) sd[m * (kpad / 256) + ch] = dd;
+                }
+            }
+        } else {
+            const ActView &a = args.a;
+            for (int i = tid; i < K / 16; i += kDecodeThreads) {
+                uint4 v = make_uint4(0, 0, 0, 0);
+                if (have) v = *reinterpret_cast<const uint4 *>(a.qs + (int64_t)m * K + i * 16);
+                *reinterpret_cast<uint4 *>(sq + m * kpad + i * 16) = v;
+            }
+            for (int i = tid; i < K / BLK; i += kDecodeThreads)
+                sd[m * (kpad / BLK) + i] = have ? a.d[(int64_t)m * (K / BLK) + i] : 0.f;
+            if (QT != kTypeQ8_0)
+                for (int i = tid; i < K / 16; i += kDecodeThreads)
+                    sb[m * (kpad / 16) + i] = have ? a.bsums[(int64_t)m * (K / 16) + i] : (int16_t)0;
+        }
+    }
+}
+
+template <int QT, int R>
+__device__ __forceinline__ void issue(Raw<QT> (&raw)[R], const RowPtr<QT> &rp, int g, int c, int last_row, int nb, int lane) {
+    constexpr int BPC = Geo<QT>::kChunk / Geo<QT>::kBlk;
+    // Lanes past the end of a row (last, partial chunk) and rows past the end of the run load the
+    // last valid block / row instead: always in bounds, never used.
+    int blk = c * BPC + lane / Geo<QT>::kLanesPerBlk;
+    if (blk >= nb) blk = nb - 1;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int rel = g * R + r;
+        if (rel > last_row) rel = last_row;
+        raw[r].load(rp, (uint32_t)blk, lane, (uint32_t)rel);
+    }
+}
+
+// XREG: the lane's activation slices live in `xr` (one chunk covers K); otherwise they are read
+// from the LDS image for chunk c.
+template <int QT, int MT, int R, bool XREG>
+__device__ __forceinline__ void consume(const Raw<QT> (&raw)[R], float (&acc)[MT][R], const Dot<QT> (&xr)[MT], const XTile &xt,
+                                        int g, int c, int nch, int nb, int n_rows, int64_t row_begin, int64_t N,
+                                        float *y, int M, int lane) {
+    constexpr int CH = Geo<QT>::kChunk;
+#ifdef QPROJ_PROBE_NOCOMPUTE
+    if (true) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const uint32_t *w = reinterpret_cast<const uint32_t *>(&raw[r]);
+            uint32_t x = 0;
+#pragma unroll
+            for (int i = 0; i < (int)(sizeof(Raw<QT>) / 4); ++i) x ^= w[i];
+            acc[0][r] += __int_as_float(x & 0x3fffff);
+        }
+    } else
+#endif
+    if (lane_block<QT>((int64_t)c * CH, lane) < nb) {
+        Frag<QT> f[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) f[r].unpack(raw[r], lane);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            if (XREG) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[m][r] += xr[m].dot(f[r]);
+            } else {
+                Dot<QT> dx;
+                dx.load_x(xt, m, c * CH, lane);
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[m][r] += dx.dot(f[r]);
+            }
+        }
+    }
+    if (c + 1 == nch) {  // row group finished: reduce over the wave, store, start over
+        constexpr int V = MT * R;
+#pragma unroll
+        for (int v0 = 0; v0 < V; v0 += 4) {
+            float q[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) q[i] = (v0 + i < V) ? acc[(v0 + i) / R][(v0 + i) % R] : 0.f;
+            const float t = wave_sum4(q, lane);
+            const int i = lane - 12;  // lanes 12..15 hold the four sums
+            if (i >= 0 && i < 4 && v0 + i < V) {
+                const int m = (v0 + i) / R, r = (v0 + i) % R;
+                if (m < M && g * R + r < n_rows) y[(int64_t)m * N + row_begin + g * R + r] = t;
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[m][r] = 0.f;
+    }
+}
+
+template <int QT, int MT, int R, bool XREG, bool FUSE>
+__global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvArgs args, int kpad) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int CH = Geo<QT>::kChunk;
+    constexpr int BLK = Geo<QT>::kBlk;
+    const int lane = threadIdx.x & 63;
+    const int wave = uniform(threadIdx.x >> 6);
+    const int gw = blockIdx.x * kDecodeWaves + wave;  // global wave index
+    const int64_t K = args.t[0].w.K;
+    const int nb = (int)args.t[0].w.nb;
+    const int nch = XREG ? 1 : kpad / CH;
+
+    // this wave's target and run of rows (selected once; everything below is wave-uniform)
+    WeightView w = args.t[0].w;
+    float *y = args.t[0].y;
+    int wave_first = 0, rpw = args.t[0].rows_per_wave;
+#pragma unroll
+    for (int i = 1; i < kMaxTargets; ++i) {
+        if (i < args.n_targets && gw >= args.t[i].first_block) {
+            w = args.t[i].w;
+            y = args.t[i].y;
+            wave_first = args.t[i].first_block;
+            rpw = args.t[i].rows_per_wave;
+        }
+    }
+    const int64_t N = w.N;
+    const int64_t row_begin = (int64_t)(gw - wave_first) * rpw;
+    int n_rows = 0;  // rows this wave owns
+    if (row_begin < N) n_rows = (int)((N - row_begin) < rpw ? (N - row_begin) : rpw);
+    n_rows = uniform(n_rows);
+    const int n_groups = (n_rows + R - 1) / R;
+    const int n_iter = n_groups * nch;
+    const int last_row = n_rows > 0 ? n_rows - 1 : 0;
+    RowPtr<QT> rp;
+    rp.set(w, row_begin < N ? row_begin : 0);
+
+    Raw<QT> buf_a[R], buf_b[R];
+    issue<QT, R>(buf_a, rp, 0, 0, last_row, nb, lane);  // in flight while the activations are staged
+
+#ifndef QPROJ_PROBE_NOSTAGE
+    stage_activations<QT, MT, FUSE>(smem, args, K, kpad);
+    __syncthreads();
+#endif
+
+    XTile xt;
+    xt.qs = reinterpret_cast<const int8_t *>(smem);
+    xt.d = reinterpret_cast<const float *>(smem + MT * kpad);
+    xt.bs = reinterpret_cast<const int16_t *>(smem + MT * kpad + MT * (kpad / BLK) * 4);
+    xt.kt = kpad;
+    Dot<QT> xr[MT];
+    if (XREG) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) xr[m].load_x(xt, m, 0, lane);
+    }
+
+    float acc[MT][R];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[m][r] = 0.f;
+
+    // (g, c) = (row group, chunk) cursors; the issue cursor runs one step ahead of the consume
+    // cursor and stops on the last step, whose cache lines were just fetched, so every issue is
+    // unconditional and no wait ever has to cover a maybe-issued load.
+    if (XREG) {  // one chunk per row: the step index is the row group
+        for (int g = 0; g < n_groups; g += 2) {
+            issue<QT, R>(buf_b, rp, g + 1 < n_groups ? g + 1 : n_groups - 1, 0, last_row, nb, lane);
+            __builtin_amdgcn_sched_barrier(0);
+            consume<QT, MT, R, XREG>(buf_a, acc, xr, xt, g, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
+            issue<QT, R>(buf_a, rp, g + 2 < n_groups ? g + 2 : n_groups - 1, 0, last_row, nb, lane);
+            __builtin_amdgcn_sched_barrier(0);
+            if (g + 1 < n_groups) consume<QT, MT, R, XREG>(buf_b, acc, xr, xt, g + 1, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
+        }
+        return;
+    }
+    int ig = 0, ic = 0, cg = 0, cc = 0, issued = 0;
+    auto advance = [&](int &g, int &c) {
+        c += 1;
+        if (c == nch) {
+            c = 0;
+            g += 1;
+        }
+    };
+    for (int it = 0; it < n_iter; it += 2) {
+        if (issued + 1 < n_iter) { advance(ig, ic); ++issued; }
+        issue<QT, R>(buf_b, rp, uniform(ig), uniform(ic), last_row, nb, lane);
+        __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the arithmetic that follows
+        consume<QT, MT, R, XREG>(buf_a, acc, xr, xt, uniform(cg), uniform(cc), nch, nb, n_rows, row_begin, N, y, args.M, lane);
+        advance(cg, cc);
+        if (issued + 1 < n_iter) { advance(ig, ic); ++issued; }
+        issue<QT, R>(buf_a, rp, uniform(ig), uniform(ic), last_row, nb, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        if (it + 1 < n_iter) {
+            consume<QT, MT, R, XREG>(buf_b, acc, xr, xt, uniform(cg), uniform(cc), nch, nb, n_rows, row_begin, N, y, args.M, lane);
+            advance(cg, cc);
+        }
+    }
+}
+
+int cu_count() {
+    static int n = [] {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+        return v;
+    }();
+    return n;
+}
+
+int env_int(const char *name, int dflt) {
+    const char *e = getenv(name);
+    return e && *e ? atoi(e) : dflt;
+}
+
+template <int QT, int MT, int R, bool XREG, bool FUSE>
+hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
+    constexpr int CH = Geo<QT>::kChunk;
+    constexpr int BLK = Geo<QT>::kBlk;
+    GemvArgs a = args;
+    int64_t rows_total = 0;
+    for (int i = 0; i < a.n_targets; ++i) rows_total += a.t[i].w.N;
+    if (rows_total == 0) return hipSuccess;
+    // one workgroup per CU, fewer when there are not enough rows to give every wave one
+    static const int wgs_per_cu = env_int("QPROJ_DECODE_WGS_PER_CU", 1);
+    int64_t grid = (int64_t)cu_count() * wgs_per_cu;
+    const int64_t need = (rows_total + kDecodeWaves - 1) / kDecodeWaves;  // at least one row per wave
+    if (grid > need) grid = need;
+    const int n_waves = (int)grid * kDecodeWaves;
+    // waves are dealt to the targets in proportion to their rows; a wave never straddles targets
+    int given = 0;
+    for (int i = 0; i < a.n_targets; ++i) {
+        const int left_after = a.n_targets - 1 - i;  // every later target gets at least one wave
+        int share = (int)((a.t[i].w.N * n_waves + rows_total - 1) / rows_total);
+        if (share < 1) share = 1;
+        if (i == a.n_targets - 1 || given + share > n_waves - left_after) share = n_waves - left_after - given;
+        if (share < 1) return hipErrorInvalidValue;
+        a.t[i].first_block = given;
+        int rpw = (int)((a.t[i].w.N + share - 1) / share);
+        a.t[i].rows_per_wave = rpw;
+        if ((int64_t)rpw * (int64_t)a.t[i].w.nb * 256 >= ((int64_t)1 << 31)) return hipErrorInvalidValue;  // 32-bit row offsets
+        given += share;
+    }
+    const int64_t K = a.t[0].w.K;
+    const int kpad = (int)((K + CH - 1) / CH * CH);
+    const size_t smem = (size_t)MT * kpad + (size_t)MT * (kpad / BLK) * 4 + (QT != kTypeQ8_0 ? (size_t)MT * (kpad / 16) * 2 : 0);
+    auto kern = &gemv_decode_kernel<QT, MT, R, XREG, FUSE>;
+    if (smem > 48 * 1024) {
+        static size_t allowed = 0;
+        if (smem > allowed) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) return e;
+            allowed = smem;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kDecodeThreads), smem, s, a, kpad);
+    return hipGetLastError();
+}
+
+template <int QT, bool FUSE>
+hipError_t launch_decode_mt(const GemvArgs &args, int mt, hipStream_t s) {
+    const bool one_chunk = QT != kTypeQ8_0 && args.t[0].w.K <= Geo<QT>::kChunk;
+    switch (mt) {
+    case 1: {
+        // two rows per step only when every wave has at least two rows to walk
+        int64_t rows_total = 0;
+        for (int i = 0; i < args.n_targets; ++i) rows_total += args.t[i].w.N;
+        const bool pairs = rows_total >= (int64_t)2 * cu_count() * kDecodeWaves;
+        if (one_chunk) return pairs ? launch_decode<QT, 1, 2, true, FUSE>(args, s) : launch_decode<QT, 1, 1, true, FUSE>(args, s);
+        return pairs ? launch_decode<QT, 1, 2, false, FUSE>(args, s) : launch_decode<QT, 1, 1, false, FUSE>(args, s);
+    }
+    case 2: return one_chunk ? launch_decode<QT, 2, 2, true, FUSE>(args, s) : launch_decode<QT, 2, 2, false, FUSE>(args, s);
+    case 4: return launch_decode<QT, 4, 1, false, FUSE>(args, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+// the largest K whose activation rows fit the LDS image (mt rows)
+bool decode_kernel_fits(int type, int mt, int64_t K) {
+    const int ch = type == kTypeQ8_0 ? 1024 : 4096;
+    const int blk = type == kTypeQ8_0 ? 32 : 256;
+    const int64_t kpad = (K + ch - 1) / ch * ch;
+    const int64_t smem = mt * kpad + mt * (kpad / blk) * 4 + (type != kTypeQ8_0 ? mt * (kpad / 16) * 2 : 0);
+    return mt <= 4 && smem <= 96 * 1024;
+}
+
+hipError_t launch_gemv_decode(const GemvArgs &args, int mt, bool fuse_quantize, hipStream_t s) {
+    switch (args.t[0].w.type) {
+    case kTypeQ4_K: return fuse_quantize ? launch_decode_mt<kTypeQ4_K, true>(args, mt, s) : launch_decode_mt<kTypeQ4_K, false>(args, mt, s);
+    case kTypeQ6_K: return fuse_quantize ? launch_decode_mt<kTypeQ6_K, true>(args, mt, s) : launch_decode_mt<kTypeQ6_K, false>(args, mt, s);
+    case kTypeQ8_0: return fuse_quantize ? launch_decode_mt<kTypeQ8_0, true>(args, mt, s) : launch_decode_mt<kTypeQ8_0, false>(args, mt, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace qproj

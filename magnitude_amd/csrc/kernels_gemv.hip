@@ -8,20 +8,19 @@
 // staged once per workgroup in LDS and shared by the R rows; all multiplies are v_dot4_i32_i8.
 // Integer partial sums are exact; each lane keeps an fp32 partial per (activation row, weight
 // row) and one DPP wave reduction per output finishes the dot product.
-#include "qproj_device.h"
-#include "qproj_internal.h"
+#include "gemv_frags.h"
 
 namespace qproj {
 
 namespace {
 
-template <int QT> struct Geo;
-template <> struct Geo<kTypeQ4_K> { static constexpr int kChunk = 2048; static constexpr int kBlk = 256; };
-template <> struct Geo<kTypeQ6_K> { static constexpr int kChunk = 2048; static constexpr int kBlk = 256; };
-template <> struct Geo<kTypeQ8_0> { static constexpr int kChunk = 1024; static constexpr int kBlk = 32; };
-
 // K-tile staged in LDS per activation row count: MT * kTile bytes of int8 (<= 32 KiB).
-__host__ __device__ constexpr int tile_k(int mt) { return mt <= 1 ? 16384 : (mt == 2 ? 8192 : (mt == 4 ? 4096 : 2048)); }
+// Never smaller than one chunk of the weight type (4096 for the K-quants).
+__host__ __device__ constexpr int tile_k(int qt, int mt) {
+    const int base = mt <= 1 ? 16384 : (mt == 2 ? 8192 : (mt == 4 ? 4096 : 2048));
+    const int chunk = qt == kTypeQ8_0 ? 1024 : 4096;
+    return base > chunk ? base : chunk;
+}
 
 struct TargetSel {
     WeightView w;
@@ -46,163 +45,10 @@ __device__ __forceinline__ TargetSel select_target(const GemvArgs &a) {
     return s;
 }
 
-// ------------------------------------------------------------------------------------------
-// per-type weight fragments: what one lane holds of one weight row for one chunk
-
-template <int QT> struct Frag;
-
-template <> struct Frag<kTypeQ4_K> {
-    uint32_t lo[4], hi[4];  // 16 low-nibble weights (sub-block 2c) and 16 high-nibble (2c+1)
-    int sc0, sc1, m0, m1;
-    float d, dmin;
-    __device__ __forceinline__ void load(const WeightView &w, int64_t row, int64_t sb, int lane) {
-        const int sub = lane & 7, c = sub >> 1, h = sub & 1;
-        const uint8_t *blk = w.q4k + (row * w.nb + sb) * 144;
-        const uint4 hd = *reinterpret_cast<const uint4 *>(blk);
-        const uint4 q = *reinterpret_cast<const uint4 *>(blk + 16 + 32 * c + 16 * h);
-        const uint32_t qq[4] = {q.x, q.y, q.z, q.w};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            lo[i] = qq[i] & 0x0f0f0f0fu;
-            hi[i] = (qq[i] >> 4) & 0x0f0f0f0fu;
-        }
-        const ScalesK4 s = unpack_scales_k4(hd.y, hd.z, hd.w);
-        sc0 = (int)scale_k4(s, 2 * c);
-        sc1 = (int)scale_k4(s, 2 * c + 1);
-        m0 = (int)min_k4(s, 2 * c);
-        m1 = (int)min_k4(s, 2 * c + 1);
-        d = h2f(hd.x);
-        dmin = h2f(hd.x >> 16);
-    }
-};
-
-template <> struct Frag<kTypeQ6_K> {
-    uint32_t q[4][2];  // group g (32g + l0 .. +8 of the lane's 128-half), values 0..63
-    int sc[4];
-    float d;
-    __device__ __forceinline__ void load(const WeightView &w, int64_t row, int64_t sb, int lane) {
-        const int i = lane & 7, h = i >> 2, l0 = 8 * (i & 3);
-        const int64_t b = row * w.nb + sb;
-        const uint2 A = *reinterpret_cast<const uint2 *>(w.q6_ql + b * 128 + 64 * h + l0);
-        const uint2 B = *reinterpret_cast<const uint2 *>(w.q6_ql + b * 128 + 64 * h + 32 + l0);
-        const uint2 H = *reinterpret_cast<const uint2 *>(w.q6_qh + b * 64 + 32 * h + l0);
-        const uint2 S = *reinterpret_cast<const uint2 *>(w.q6_sc + b * 16 + 8 * h);
-        const uint32_t a[2] = {A.x, A.y}, bb[2] = {B.x, B.y}, hh[2] = {H.x, H.y};
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            q[0][t] = (a[t] & 0x0f0f0f0fu) | ((hh[t] << 4) & 0x30303030u);
-            q[1][t] = (bb[t] & 0x0f0f0f0fu) | ((hh[t] << 2) & 0x30303030u);
-            q[2][t] = ((a[t] >> 4) & 0x0f0f0f0fu) | (hh[t] & 0x30303030u);
-            q[3][t] = ((bb[t] >> 4) & 0x0f0f0f0fu) | ((hh[t] >> 2) & 0x30303030u);
-        }
-        const int e = l0 >> 4;  // which 16-weight scale group of the 32-group
-        const uint64_t s64 = (uint64_t)S.x | ((uint64_t)S.y << 32);
-#pragma unroll
-        for (int g = 0; g < 4; ++g) sc[g] = (int)(int8_t)(s64 >> (8 * (2 * g + e)));
-        d = h2f(w.q6_d[b]);
-    }
-};
-
-template <> struct Frag<kTypeQ8_0> {
-    uint32_t q[4];  // 16 int8 weights: half of a 32-block
-    float d;
-    __device__ __forceinline__ void load(const WeightView &w, int64_t row, int64_t blk, int lane) {
-        const uint4 v = *reinterpret_cast<const uint4 *>(w.q8_qs + row * w.K + blk * 32 + 16 * (lane & 1));
-        q[0] = v.x; q[1] = v.y; q[2] = v.z; q[3] = v.w;
-        d = h2f(w.q8_d[row * w.nb + blk]);
-    }
-};
-
-// LDS image of the staged activations of one K-tile
-struct XTile {
-    const int8_t *qs;     // [MT][KT]
-    const float *d;       // [MT][KT / blk]
-    const int16_t *bs;    // [MT][KT / 16]  (Q8_K only)
-    int kt;               // KT
-};
-
-// fp32 partial of (weight fragment) . (activation row m, chunk at c0) for each type
-template <int QT> struct Dot;
-
-template <> struct Dot<kTypeQ4_K> {
-    uint32_t xl[4], xh[4];
-    int bl, bh;
-    float xd;
-    __device__ __forceinline__ void load_x(const XTile &x, int m, int c0, int lane) {
-        const int sbl = lane >> 3, sub = lane & 7, c = sub >> 1, h = sub & 1;
-        const int xo = c0 + sbl * 256 + 64 * c + 16 * h;
-        const uint4 a = *reinterpret_cast<const uint4 *>(x.qs + m * x.kt + xo);
-        const uint4 b = *reinterpret_cast<const uint4 *>(x.qs + m * x.kt + xo + 32);
-        xl[0] = a.x; xl[1] = a.y; xl[2] = a.z; xl[3] = a.w;
-        xh[0] = b.x; xh[1] = b.y; xh[2] = b.z; xh[3] = b.w;
-        const int bi = m * (x.kt / 16) + (c0 + sbl * 256) / 16 + 4 * c + h;
-        bl = x.bs[bi];
-        bh = x.bs[bi + 2];
-        xd = x.d[m * (x.kt / 256) + c0 / 256 + sbl];
-    }
-    __device__ __forceinline__ float dot(const Frag<kTypeQ4_K> &f) const {
-        int sl = 0, sh = 0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            sl = dot4(f.lo[i], xl[i], sl);
-            sh = dot4(f.hi[i], xh[i], sh);
-        }
-        const int isum = f.sc0 * sl + f.sc1 * sh;
-        const int msum = f.m0 * bl + f.m1 * bh;
-        return fmaf(f.d * xd, (float)isum, -((f.dmin * xd) * (float)msum));
-    }
-};
-
-template <> struct Dot<kTypeQ6_K> {
-    uint32_t xg[4][2];
-    int asum[4];
-    float xd;
-    __device__ __forceinline__ void load_x(const XTile &x, int m, int c0, int lane) {
-        const int sbl = lane >> 3, i = lane & 7, h = i >> 2, l0 = 8 * (i & 3);
-        const int xo = c0 + sbl * 256 + 128 * h + l0;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const uint2 v = *reinterpret_cast<const uint2 *>(x.qs + m * x.kt + xo + 32 * g);
-            xg[g][0] = v.x;
-            xg[g][1] = v.y;
-            asum[g] = dot4(0x01010101u, v.x, dot4(0x01010101u, v.y, 0));
-        }
-        xd = x.d[m * (x.kt / 256) + c0 / 256 + sbl];
-    }
-    __device__ __forceinline__ float dot(const Frag<kTypeQ6_K> &f) const {
-        int isum = 0;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int s = dot4(f.q[g][0], xg[g][0], dot4(f.q[g][1], xg[g][1], 0));
-            isum += f.sc[g] * (s - 32 * asum[g]);
-        }
-        return (f.d * xd) * (float)isum;
-    }
-};
-
-template <> struct Dot<kTypeQ8_0> {
-    uint32_t xq[4];
-    float xd;
-    __device__ __forceinline__ void load_x(const XTile &x, int m, int c0, int lane) {
-        const int xo = c0 + 16 * lane;
-        const uint4 a = *reinterpret_cast<const uint4 *>(x.qs + m * x.kt + xo);
-        xq[0] = a.x; xq[1] = a.y; xq[2] = a.z; xq[3] = a.w;
-        xd = x.d[m * (x.kt / 32) + (c0 >> 5) + (lane >> 1)];
-    }
-    __device__ __forceinline__ float dot(const Frag<kTypeQ8_0> &f) const {
-        int s = 0;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) s = dot4(f.q[i], xq[i], s);
-        return (float)s * (f.d * xd);
-    }
-};
-
-// ------------------------------------------------------------------------------------------
-
 template <int QT, int MT>
 __device__ __forceinline__ void stage_tile(uint8_t *smem, const ActView &a, const int64_t *arow, int kt0,
                                            int kt_len, int kt_pad) {
-    constexpr int KT = tile_k(MT);
+    constexpr int KT = tile_k(QT, MT);
     constexpr int BLK = Geo<QT>::kBlk;
     int8_t *sq = reinterpret_cast<int8_t *>(smem);
     float *sd = reinterpret_cast<float *>(smem + MT * KT);
@@ -220,7 +66,7 @@ __device__ __forceinline__ void stage_tile(uint8_t *smem, const ActView &a, cons
             if (r >= 0 && i * BLK < kt_len) v = a.d[r * (a.K / BLK) + kt0 / BLK + i];
             sd[m * (KT / BLK) + i] = v;
         }
-        if (QT == kTypeQ4_K) {
+        if (QT != kTypeQ8_0) {
             for (int i = tid; i < kt_pad / 16; i += 256) {
                 int16_t v = 0;
                 if (r >= 0 && i * 16 < kt_len) v = a.bsums[r * (a.K / 16) + kt0 / 16 + i];
@@ -231,9 +77,9 @@ __device__ __forceinline__ void stage_tile(uint8_t *smem, const ActView &a, cons
 }
 
 constexpr size_t gemv_smem_bytes(int qt, int mt) {
-    const int kt = tile_k(mt);
+    const int kt = tile_k(qt, mt);
     const int blk = qt == kTypeQ8_0 ? 32 : 256;
-    return (size_t)mt * kt + (size_t)mt * (kt / blk) * 4 + (qt == kTypeQ4_K ? (size_t)mt * (kt / 16) * 2 : 0);
+    return (size_t)mt * kt + (size_t)mt * (kt / blk) * 4 + (qt != kTypeQ8_0 ? (size_t)mt * (kt / 16) * 2 : 0);
 }
 
 // QT weight type; MT activation rows per pass; R weight rows per wave; GROUPED: blockIdx.y is an
@@ -242,12 +88,13 @@ constexpr size_t gemv_smem_bytes(int qt, int mt) {
 template <int QT, int MT, int R, bool GROUPED, bool SWIGLU>
 __global__ __launch_bounds__(256) void gemv_q8act_kernel(const GemvArgs args) {
     extern __shared__ __align__(16) uint8_t smem[];
-    constexpr int KT = tile_k(MT);
+    constexpr int KT = tile_k(QT, MT);
     constexpr int CH = Geo<QT>::kChunk;
     constexpr int BLK = Geo<QT>::kBlk;
     constexpr int NT = SWIGLU ? 2 : 1;
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = uniform(threadIdx.x >> 6);
     TargetSel T;
     if (SWIGLU) {
         T.w = args.t[0].w;
@@ -301,7 +148,7 @@ __global__ __launch_bounds__(256) void gemv_q8act_kernel(const GemvArgs args) {
             __syncthreads();
             for (int c0 = 0; c0 < kt_len; c0 += CH) {
                 // block index of this lane inside the row
-                const int64_t blk = (QT == kTypeQ8_0) ? (kt0 + c0) / 32 + (lane >> 1) : (kt0 + c0) / 256 + (lane >> 3);
+                const int64_t blk = lane_block<QT>(kt0 + c0, lane);
                 if (blk < nb) {
                     Frag<QT> f[NT][R];
 #pragma unroll
@@ -310,7 +157,11 @@ __global__ __launch_bounds__(256) void gemv_q8act_kernel(const GemvArgs args) {
                         for (int r = 0; r < R; ++r) {
                             int64_t row = row0 + r;
                             if (row >= N) row = N - 1;
-                            f[t][r].load(t == 0 ? T.w : args.t[1].w, e_base + row, blk, lane);
+                            RowPtr<QT> rp;
+                            rp.set(t == 0 ? T.w : args.t[1].w, e_base + row);
+                            Raw<QT> raw;
+                            raw.load(rp, (uint32_t)blk, lane);
+                            f[t][r].unpack(raw, lane);
                         }
                     }
 #pragma unroll
@@ -351,7 +202,14 @@ hipError_t launch_one(const GemvArgs &args, int n_experts_grid, hipStream_t s) {
     }
     if (total_blocks == 0) return hipSuccess;
     const dim3 grid((unsigned)total_blocks, (unsigned)(GROUPED ? n_experts_grid : 1));
-    hipLaunchKernelGGL((gemv_q8act_kernel<QT, MT, R, GROUPED, SWIGLU>), grid, dim3(256), gemv_smem_bytes(QT, MT), s, a);
+    constexpr size_t smem = gemv_smem_bytes(QT, MT);
+    if (smem > 48 * 1024) {  // above the default dynamic-LDS allowance: opt in once per kernel
+        static hipError_t attr = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(&gemv_q8act_kernel<QT, MT, R, GROUPED, SWIGLU>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (attr != hipSuccess) return attr;
+    }
+    hipLaunchKernelGGL((gemv_q8act_kernel<QT, MT, R, GROUPED, SWIGLU>), grid, dim3(256), smem, s, a);
     return hipGetLastError();
 }
 

@@ -2,6 +2,7 @@
 #include "../../include/qproj.h"
 
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -229,8 +230,26 @@ int upload_common(qproj_ctx *ctx, int type, int64_t K, int64_t N, int64_t n_expe
 }
 
 // dense mul_mat over quantized activations already sitting in `a` (M rows)
+bool use_decode_kernel(int type, int64_t M, int64_t K) {
+    static const bool off = getenv("QPROJ_NO_DECODE_KERNEL") != nullptr;
+    return !off && M <= 4 && decode_kernel_fits(type, pow2_ceil(M), K);
+}
+
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
                     float *const *y) {
+    if (use_decode_kernel(w[0]->type, M, w[0]->K)) {
+        GemvArgs g{};
+        g.n_targets = n;
+        for (int i = 0; i < n; ++i) {
+            g.t[i].w = w[i]->view;
+            g.t[i].y = y[i];
+        }
+        g.a = a;
+        g.M = (int)M;
+        g.x_div = 1;
+        QP_HIP(ctx, launch_gemv_decode(g, pow2_ceil(M), false, ctx->stream));
+        return QPROJ_OK;
+    }
     for (int64_t m0 = 0; m0 < M; m0 += 16) {
         const int64_t mc = std::min<int64_t>(16, M - m0);
         GemvArgs g{};
@@ -446,6 +465,20 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
     if (M == 0) return QPROJ_OK;
     QP_HIP(ctx, hipSetDevice(ctx->device));
     const int64_t K = w[0]->K;
+    if (act == kActGGML && use_decode_kernel(w[0]->type, M, K)) {
+        // decode regime: the kernel quantizes the activation rows itself, no scratch needed
+        GemvArgs g{};
+        g.n_targets = n;
+        for (int i = 0; i < n; ++i) {
+            g.t[i].w = w[i]->view;
+            g.t[i].y = y_dev[i];
+        }
+        g.x = x_dev;
+        g.M = (int)M;
+        g.x_div = 1;
+        QP_HIP(ctx, launch_gemv_decode(g, pow2_ceil(M), true, ctx->stream));
+        return QPROJ_OK;
+    }
     if (act == kActGGML || act == kActQ8X32) {
         if (act == kActQ8X32 && w[0]->type != kTypeQ4_K)
             return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat: the per-32 int8 path is built for Q4_K weights");
@@ -475,6 +508,29 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
         return QPROJ_OK;
     }
     return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: unknown activation mode");
+}
+
+int qproj_mul_mat_quantized(qproj_ctx *ctx, int n, const qproj_weight *const *w, const void *act_dev, int kind,
+                            int64_t M, float *const *y_dev) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (n <= 0 || n > kMaxTargets || !w || !y_dev || !act_dev)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat_quantized: null argument or more than 4 tensors");
+    if (kind != kActGGML && kind != kActQ8X32)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat_quantized: kind must name a quantized format");
+    for (int i = 0; i < n; ++i) {
+        if (!w[i] || !y_dev[i] || w[i]->E != 1 || w[i]->K != w[0]->K || w[i]->type != w[0]->type)
+            return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat_quantized: tensors must be dense and share K and type");
+    }
+    if (M <= 0) return M == 0 ? QPROJ_OK : fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat_quantized: negative M");
+    if (kind == kActQ8X32 && w[0]->type != kTypeQ4_K)
+        return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat_quantized: the per-32 int8 path is built for Q4_K weights");
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    const int64_t K = w[0]->K;
+    const ActPlanes p = act_planes(act_kind_for(kind, w[0]->type), M, K);
+    const ActView a = act_view(p, static_cast<uint8_t *>(const_cast<void *>(act_dev)), K);
+    if (kind == kActGGML) return run_dense_q8act(ctx, n, w, a, M, y_dev);
+    for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], ctx->stream));
+    return QPROJ_OK;
 }
 
 int qproj_mul_mat(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int64_t M, float *y_dev, int act) {

@@ -40,6 +40,23 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// Sums of FOUR per-lane values at once, "transposed": after the call, lane 12 + i of every row of
+// 16 lanes holds the 64-lane sum of v[i].  The first two steps fold pairs of values into
+// alternating lanes, so the whole thing costs about as much as one and a half plain reductions.
+__device__ __forceinline__ float wave_sum4(const float (&v)[4], int lane) {
+    const bool odd = lane & 1, hi2 = lane & 2;
+    // lanes xor 1: even lanes collect v0 / v2, odd lanes collect v1 / v3
+    const float s01 = (odd ? v[1] : v[0]) + dpp_move<0xB1>(odd ? v[0] : v[1]);
+    const float s23 = (odd ? v[3] : v[2]) + dpp_move<0xB1>(odd ? v[2] : v[3]);
+    // lanes xor 2: lane & 3 == i now collects v[i] over its quad
+    float t = (hi2 ? s23 : s01) + dpp_move<0x4E>(hi2 ? s01 : s23);
+    t += dpp_move<0x114>(t);  // row_shr:4
+    t += dpp_move<0x118>(t);  // row_shr:8  -> lanes 12..15 of each row hold the row's sums
+    t += __shfl_xor(t, 16);
+    t += __shfl_xor(t, 32);
+    return t;
+}
+
 // The 6-bit (scale, min) pairs of a Q4_K super-block, unpacked four at a time from the 12-byte
 // field (three dwords s0, s1, s2).  Byte j of `sc_lo`/`mn_lo` is sub-block j (0..3); byte j of
 // `sc_hi`/`mn_hi` is sub-block 4+j.

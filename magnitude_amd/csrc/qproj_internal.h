@@ -51,7 +51,8 @@ constexpr int kActKindQ8X32 = 2;
 struct GemvTarget {
     WeightView w;
     float *y;              // [rows][N]
-    int first_block;       // first blockIdx.x that belongs to this target
+    int first_block;       // first blockIdx.x (tiled kernels) or first wave (decode kernel) of the target
+    int rows_per_wave;     // decode kernel: consecutive rows each wave of the target walks
 };
 constexpr int kMaxTargets = 4;
 
@@ -75,6 +76,9 @@ hipError_t launch_repack_to_gguf(int type, const WeightView &w, uint8_t *gguf, i
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
                                int16_t *bsums, int32_t *isum, hipStream_t s);
 hipError_t launch_gemv_q8act(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
+// persistent decode kernel (mt <= 4 rows); fuse_quantize: args.x holds fp32 rows, else args.a
+bool decode_kernel_fits(int type, int mt, int64_t K);
+hipError_t launch_gemv_decode(const GemvArgs &args, int mt, bool fuse_quantize, hipStream_t s);
 hipError_t launch_gemv_f32(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
 hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_expert, int32_t *order,
                             int32_t *offsets, int32_t *error_flag, hipStream_t s);

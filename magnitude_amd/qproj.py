@@ -24,7 +24,9 @@ BLOCK_ELEMS = {TYPE_Q8_0: 32, TYPE_Q4_K: 256, TYPE_Q6_K: 256}
 
 STATUS_NAMES = {0: "OK", 1: "INVALID_ARG", 2: "HIP", 3: "OOM", 4: "UNSUPPORTED", 5: "NO_DEVICE"}
 
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libqproj.so")
+# QPROJ_LIBRARY points at another build of the same library (e.g. an instrumented one)
+LIB_PATH = os.environ.get("QPROJ_LIBRARY") or os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib",
+                                                           "libqproj.so")
 
 # every symbol include/qproj.h declares: (restype, argtypes)
 _vp, _i64, _i32, _sz = C.c_void_p, C.c_int64, C.c_int, C.c_size_t
@@ -47,6 +49,7 @@ SYMBOLS = {
     "qproj_quantize_activations": (_i32, [_vp, _i32, _i32, _vp, _i64, _i64, _vp]),
     "qproj_mul_mat": (_i32, [_vp, _vp, _vp, _i64, _vp, _i32]),
     "qproj_mul_mat_multi": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i64, C.POINTER(_vp), _i32]),
+    "qproj_mul_mat_quantized": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i32, _i64, C.POINTER(_vp)]),
     "qproj_mul_mat_id": (_i32, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _i32]),
     "qproj_moe_ffn": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i32]),
     "qproj_version": (C.c_char_p, []),
@@ -241,6 +244,35 @@ class Context:
         if sync:
             self.sync()
         return ys
+
+    def quantize_activations_raw(self, x: torch.Tensor, kind: int, wtype: int,
+                                 out: Optional[torch.Tensor] = None, sync: bool = True) -> torch.Tensor:
+        """Activation quantizer into one opaque device buffer, for mul_mat_quantized."""
+        x = x.contiguous()
+        m, k = x.shape
+        nbytes = int(self.lib.qproj_act_bytes(kind, wtype, m, k))
+        if nbytes == 0:
+            raise ValueError("bad activation shape or kind")
+        buf = out if out is not None else torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        if sync:
+            torch.cuda.current_stream().synchronize()
+        self._check(self.lib.qproj_quantize_activations(self.handle, kind, wtype, _ptr(x), m, k, _ptr(buf)))
+        if sync:
+            self.sync()
+        return buf
+
+    def mul_mat_quantized(self, ws: Sequence[Weight], act: torch.Tensor, kind: int, m: int,
+                          outs: Sequence[torch.Tensor], sync: bool = True):
+        """MUL_MAT over activations quantized beforehand (shared by all of `ws`)."""
+        n = len(ws)
+        wa = (_vp * n)(*[w.handle for w in ws])
+        ya = (_vp * n)(*[_ptr(y) for y in outs])
+        if sync:
+            torch.cuda.current_stream().synchronize()
+        self._check(self.lib.qproj_mul_mat_quantized(self.handle, n, wa, _ptr(act), kind, m, ya))
+        if sync:
+            self.sync()
+        return outs
 
     def mul_mat_id(self, w: Weight, x: torch.Tensor, ids: torch.Tensor, act: int = ACT_GGML,
                    sync: bool = True) -> torch.Tensor:
