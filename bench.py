@@ -228,11 +228,13 @@ def main():
                            "bytes_per_launch": dom["bytes_per_launch"], "us_per_launch": dom["us_per_launch"],
                            "launches_timed": reps * L, "other_kernels": {k: v for k, v in per.items() if k != "gate_up"}}
         if args.calib_copy:
-            a = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+            # a plain elementwise kernel of known traffic (reads 256 MiB, writes 256 MiB) to scale the
+            # FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this same command
+            a = torch.zeros(64 << 20, dtype=torch.int32, device=dev)
             b = torch.empty_like(a)
             with torch.cuda.stream(stream):
                 for _ in range(5):
-                    b.copy_(a)
+                    torch.add(a, 1, out=b)
             torch.cuda.synchronize()
 
     # ------------------------------------------------------------------ prefill leg (config 4)
