@@ -82,6 +82,18 @@ def capture(torch, stream, fn):
         return None
 
 
+def measured_traffic(summary="decode_gate_up_q4k.txt"):
+    """HBM bytes per launch of the dominant kernel, from the committed rocprofv3 counter summary
+    (FETCH_SIZE + WRITE_SIZE, each scaled by a copy kernel of known size); None if not recorded."""
+    try:
+        for line in open(os.path.join(ROOT, "profiles", summary)):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1])
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -222,7 +234,7 @@ def main():
                 f"({100 * per[grp[0]]['frac_hbm_peak']:.1f}% of peak)")
         dom = per["gate_up"]
         out["roofline"] = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": dom["frac_hbm_peak"], "traffic": None,
+                           "frac": dom["frac_hbm_peak"], "traffic": measured_traffic(),
                            "kernel": "gemv_decode_kernel<Q4_K, M=1>: gate+up (2 x 4096->14336) in one launch, "
                                      "activation quantized in the prologue",
                            "bytes_per_launch": dom["bytes_per_launch"], "us_per_launch": dom["us_per_launch"],
