@@ -1,14 +1,21 @@
 // Prefill projection: Q4_K weights x per-32 int8 activations on the int8 matrix cores.
 //
-//   y[m][n] = sum_blk (d_n*sc_{n,blk}) * da_{m,blk} * I_{m,n,blk} - (dmin_n*mn_{n,blk}) * (da_{m,blk}*isum_{m,blk})
+//   y[m][n] = sum_blk (d_n*sc_{n,blk}) * da_{m,blk} * I_{m,n,blk}  -  sum_blk (dmin_n*mn_{n,blk}) * (da_{m,blk}*isum_{m,blk})
 //   I_{m,n,blk} = sum over the 32 weights of the sub-block of q * a      (exact, int32)
 //
-// A workgroup owns a 128 (tokens) x 128 (weight rows) tile and walks K in steps of 128 (four
-// sub-blocks).  Per step the 4-bit weights are expanded to int8 into LDS together with the
-// activation tile; each of the 4 waves owns a 64x64 sub-tile = 2x2 v_mfma_i32_32x32x32_i8
-// products per sub-block.  An int32 accumulator is only meaningful inside one sub-block
-// (both operands change scale every 32), so every product is folded into the fp32 accumulators
-// right away: acc += float(I) * (da * ws) - asum * wm.
+// A workgroup owns a 128 (tokens) x 128 (weight rows) tile; each of its 8 waves a 32x64
+// sub-tile = two v_mfma_i32_32x32x32_i8 products per 32-wide sub-block.  Both operands change
+// scale every 32 K-elements, so an int32 accumulator is meaningful for ONE product only: each
+// product is folded into the fp32 accumulators right away (cvt, scale product, fma per output).
+// That fp32 work, not the matrix cores, bounds this kernel, so everything else is kept off the
+// vector ALU:
+//   - the min term is a separate small GEMM over K/32 (activation block sums x mins) done on the
+//     fp16 matrix cores before the main loop, with both operands split into fp16 high and low
+//     parts (the mins are 17-bit products, split exactly; the sums keep 22 bits);
+//   - the weight-side scales d*sc of a lane's own output column are unpacked from the block
+//     header by that lane and held in registers for the 8 sub-blocks of a super-block;
+//   - LDS holds only the two int8 operand tiles and the transposed activation scales, double
+//     buffered over K-steps of 128 so that the global loads of step s+1 overlap step s.
 #include "qproj_device.h"
 #include "qproj_internal.h"
 
@@ -18,140 +25,224 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr int BM = 128, BN = 128, BK = 128;
 constexpr int LDT = BK + 16;  // LDS row stride in bytes, padded against bank conflicts
+constexpr float kMinPrescale = 0.0625f;  // keeps da*isum inside fp16 range for |x| up to ~1e5
 
-struct GemmSmem {
-    int8_t a[BM * LDT];      // activations  [m][k]
-    int8_t b[BN * LDT];      // weights      [n][k], nibbles expanded
-    float a_d[4][BM];        // da           [sub-block][m]
-    float a_s[4][BM];        // da * isum
-    float w_s[4][BN];        // d * sc       [sub-block][n]
-    float w_m[4][BN];        // dmin * mn
+struct GemmStage {
+    int8_t a[BM * LDT];  // activations  [m][k]
+    int8_t b[BN * LDT];  // weights      [n][k], nibbles expanded
+    float a_d[4][BM];    // da           [sub-block][m]
 };
 
-__global__ __launch_bounds__(256) void gemm_q4k_q8x32_kernel(const WeightView w, const ActView a, int64_t M,
-                                                             float *__restrict__ y) {
-    __shared__ GemmSmem sm;
+struct GemmSmem {
+    GemmStage st[2];
+    float w_s[8][BN];  // d*sc of the 8 sub-blocks of the current super-block [n]
+};
+
+// registers one thread carries from global memory to LDS for one K-step
+struct StageRegs {
+    uint4 act[2];
+    uint4 wq;
+    float4 ad;  // threads 0..127: activation scales; threads 128..255: block header of a weight row
+};
+
+__device__ __forceinline__ void split_h(float v, _Float16 &hi, _Float16 &lo) {
+    hi = (_Float16)v;
+    lo = (_Float16)(v - (float)hi);
+}
+
+constexpr int kGemmThreads = 512;
+
+__global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const WeightView w, const ActView a, int64_t M,
+                                                               float *__restrict__ y) {
+    extern __shared__ __align__(16) uint8_t smem_raw[];
+    GemmSmem &sm = *reinterpret_cast<GemmSmem *>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave >> 1, wn = wave & 1;  // 4 x 2 waves
     const int64_t n0 = (int64_t)blockIdx.x * BN, m0 = (int64_t)blockIdx.y * BM;
     const int64_t N = w.N, K = w.K;
     const int64_t kb32 = K / 32;
+    const int l32 = lane & 31, lh = lane >> 5;
 
-    float acc[2][2][16];
+    // the lane's two output columns (clamped for loads; stores are guarded)
+    int64_t ncol[2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int j = 0; j < 2; ++j) {
+        int64_t n = n0 + wn * 64 + j * 32 + l32;
+        ncol[j] = n < N ? n : N - 1;
+    }
+
+    v16f acc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+    // ---------------------------------------------------------------- min term on the fp16 cores
+    // acc = -(1/prescale) * sum_kb A[m][kb] * B[n][kb] is built as +sum with negated B and scaled later
+    {
+        const int64_t n_steps = (kb32 + 15) / 16;  // 16 sub-blocks = two super-blocks per product
+        for (int64_t s = 0; s < n_steps; ++s) {
+            v8h ah, al, bh[2], bl[2];
+            {
+                int64_t m = m0 + wm * 32 + l32;
+                int64_t kb = s * 16 + 8 * lh;  // this half-wave's super-block; past the end of K: zeros
+                const bool live = m < M && kb < kb32;
+                if (m >= M) m = M - 1;
+                if (kb >= kb32) kb = kb32 - 8;
+                const int64_t o = m * kb32 + kb;
+                const float4 d0 = *reinterpret_cast<const float4 *>(a.d + o);
+                const float4 d1 = *reinterpret_cast<const float4 *>(a.d + o + 4);
+                const int4 s0 = *reinterpret_cast<const int4 *>(a.isum + o);
+                const int4 s1 = *reinterpret_cast<const int4 *>(a.isum + o + 4);
+                const float av[8] = {d0.x * (float)s0.x, d0.y * (float)s0.y, d0.z * (float)s0.z, d0.w * (float)s0.w,
+                                     d1.x * (float)s1.x, d1.y * (float)s1.y, d1.z * (float)s1.z, d1.w * (float)s1.w};
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    _Float16 h, l;
+                    split_h(live ? av[t] * kMinPrescale : 0.f, h, l);
+                    ah[t] = h;
+                    al[t] = l;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                int64_t sb = s * 2 + lh;
+                const bool live = sb < w.nb;
+                if (!live) sb = w.nb - 1;
+                const uint4 hd = *reinterpret_cast<const uint4 *>(w.q4k + (ncol[j] * w.nb + sb) * 144);
+                const ScalesK4 sc = unpack_scales_k4(hd.y, hd.z, hd.w);
+                const float dmin = live ? h2f(hd.x >> 16) : 0.f;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    _Float16 h, l;
+                    split_h(-(dmin * (float)min_k4(sc, t)), h, l);
+                    bh[j][t] = h;
+                    bl[j][t] = l;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j], acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[j], acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[j], acc[j], 0, 0, 0);
+            }
+        }
+        const float inv = 1.0f / kMinPrescale;
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+            for (int v = 0; v < 16; ++v) acc[j][v] *= inv;
+    }
 
-    for (int64_t k0 = 0; k0 < K; k0 += BK) {
-        __syncthreads();
-        // ---- activations: 128 rows x 128 B
+    // ---------------------------------------------------------------- main loop, int8 cores
+    auto load_stage = [&](StageRegs &r, int64_t k0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int idx = tid + 256 * i;
+        for (int i = 0; i < 2; ++i) {  // activations: 128 rows x 128 B
+            const int idx = tid + kGemmThreads * i;
             const int row = idx >> 3, seg = idx & 7;
-            uint4 v = make_uint4(0, 0, 0, 0);
-            if (m0 + row < M) v = *reinterpret_cast<const uint4 *>(a.qs + (m0 + row) * K + k0 + 16 * seg);
-            *reinterpret_cast<uint4 *>(sm.a + row * LDT + 16 * seg) = v;
+            int64_t m = m0 + row;
+            r.act[i] = make_uint4(0, 0, 0, 0);
+            if (m < M) r.act[i] = *reinterpret_cast<const uint4 *>(a.qs + m * K + k0 + 16 * seg);
         }
-        // ---- weights: 128 rows x half a super-block (two 64-weight chunks = 64 packed bytes)
-        {
-            const int row = tid >> 1, ch = tid & 1;
+        {  // weights: 128 rows x 64 packed bytes (two 64-weight chunks of the super-block)
+            const int row = tid >> 2, part = tid & 3;
             int64_t n = n0 + row;
             if (n >= N) n = N - 1;
-            const int64_t sb = k0 >> 8;
-            const int c = (int)((k0 & 255) >> 6) + ch;  // chunk inside the super-block
-            const uint8_t *blk = w.q4k + (n * w.nb + sb) * 144;
-            const uint4 p0 = *reinterpret_cast<const uint4 *>(blk + 16 + 32 * c);
-            const uint4 p1 = *reinterpret_cast<const uint4 *>(blk + 16 + 32 * c + 16);
-            const uint32_t pk[8] = {p0.x, p0.y, p0.z, p0.w, p1.x, p1.y, p1.z, p1.w};
-            uint32_t *dst = reinterpret_cast<uint32_t *>(sm.b + row * LDT + 64 * ch);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                dst[i] = pk[i] & 0x0f0f0f0fu;             // sub-block 2c
-                dst[8 + i] = (pk[i] >> 4) & 0x0f0f0f0fu;  // sub-block 2c+1
-            }
+            const int c2 = (int)((k0 & 255) >> 5);  // 32-byte chunk pair index * 2
+            const uint8_t *blk = w.q4k + (n * w.nb + (k0 >> 8)) * 144 + 16 + 16 * c2 + 16 * part;
+            r.wq = *reinterpret_cast<const uint4 *>(blk);
         }
-        // ---- scales
-        if (tid < 128) {
-            int64_t n = n0 + tid;
+        r.ad = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (tid < BM) {
+            if (m0 + tid < M) r.ad = *reinterpret_cast<const float4 *>(a.d + (m0 + tid) * kb32 + (k0 >> 5));
+        } else if (tid < BM + BN && (k0 & 255) == 0) {  // a new super-block starts: its header
+            int64_t n = n0 + (tid - BM);
             if (n >= N) n = N - 1;
-            const uint4 hd = *reinterpret_cast<const uint4 *>(w.q4k + (n * w.nb + (k0 >> 8)) * 144);
-            const ScalesK4 s = unpack_scales_k4(hd.y, hd.z, hd.w);
-            const float d = h2f(hd.x), dmin = h2f(hd.x >> 16);
-            const int j0 = (int)((k0 & 255) >> 5);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                sm.w_s[j][tid] = d * (float)scale_k4(s, j0 + j);
-                sm.w_m[j][tid] = dmin * (float)min_k4(s, j0 + j);
-            }
-        } else {
-            const int row = tid - 128;
-            float4 dv = make_float4(0.f, 0.f, 0.f, 0.f);
-            int4 sv = make_int4(0, 0, 0, 0);
-            if (m0 + row < M) {
-                dv = *reinterpret_cast<const float4 *>(a.d + (m0 + row) * kb32 + (k0 >> 5));
-                sv = *reinterpret_cast<const int4 *>(a.isum + (m0 + row) * kb32 + (k0 >> 5));
-            }
-            sm.a_d[0][row] = dv.x; sm.a_d[1][row] = dv.y; sm.a_d[2][row] = dv.z; sm.a_d[3][row] = dv.w;
-            sm.a_s[0][row] = dv.x * (float)sv.x; sm.a_s[1][row] = dv.y * (float)sv.y;
-            sm.a_s[2][row] = dv.z * (float)sv.z; sm.a_s[3][row] = dv.w * (float)sv.w;
+            r.ad = *reinterpret_cast<const float4 *>(w.q4k + (n * w.nb + (k0 >> 8)) * 144);
         }
-        __syncthreads();
+    };
+    auto store_stage = [&](const StageRegs &r, GemmStage &st, int64_t k0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int idx = tid + kGemmThreads * i;
+            const int row = idx >> 3, seg = idx & 7;
+            *reinterpret_cast<uint4 *>(st.a + row * LDT + 16 * seg) = r.act[i];
+        }
+        {
+            // 16 packed bytes = bytes 16*(part&1).. of chunk (part>>1): low nibbles -> sub-block 2c, high -> 2c+1
+            const int row = tid >> 2, part = tid & 3, ch = part >> 1, half = part & 1;
+            int8_t *base = st.b + row * LDT + 64 * ch + 16 * half;
+            *reinterpret_cast<uint4 *>(base) = make_uint4(r.wq.x & 0x0f0f0f0fu, r.wq.y & 0x0f0f0f0fu, r.wq.z & 0x0f0f0f0fu, r.wq.w & 0x0f0f0f0fu);
+            *reinterpret_cast<uint4 *>(base + 32) = make_uint4((r.wq.x >> 4) & 0x0f0f0f0fu, (r.wq.y >> 4) & 0x0f0f0f0fu,
+                                                               (r.wq.z >> 4) & 0x0f0f0f0fu, (r.wq.w >> 4) & 0x0f0f0f0fu);
+        }
+        if (tid < BM) {
+            st.a_d[0][tid] = r.ad.x;
+            st.a_d[1][tid] = r.ad.y;
+            st.a_d[2][tid] = r.ad.z;
+            st.a_d[3][tid] = r.ad.w;
+        } else if (tid < BM + BN && (k0 & 255) == 0) {
+            const uint32_t h0 = __float_as_uint(r.ad.x);
+            const ScalesK4 sc = unpack_scales_k4(__float_as_uint(r.ad.y), __float_as_uint(r.ad.z), __float_as_uint(r.ad.w));
+            const float d = h2f(h0);
+            float *dst = &sm.w_s[0][tid - BM];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) dst[t * BN] = d * (float)scale_k4(sc, t);
+        }
+    };
 
-        // ---- four sub-blocks
-#pragma unroll
+    StageRegs regs;
+    load_stage(regs, 0);
+    store_stage(regs, sm.st[0], 0);
+    __syncthreads();
+
+    const int64_t n_ksteps = K / BK;
+    for (int64_t ks = 0; ks < n_ksteps; ++ks) {
+        const int64_t k0 = ks * BK;
+        const GemmStage &st = sm.st[ks & 1];
+        if (ks + 1 < n_ksteps) load_stage(regs, k0 + BK);  // in flight during the arithmetic below
+        const float *wsp = &sm.w_s[(k0 & 255) >> 5][wn * 64 + l32];
+#pragma unroll 1
         for (int kb = 0; kb < 4; ++kb) {
-            v4i af[2], bf[2];
-            float ws[2], wmn[2];
+            const v4i af = *reinterpret_cast<const v4i *>(st.a + (wm * 32 + l32) * LDT + kb * 32 + 16 * lh);
+            v4i bf[2];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                af[i] = *reinterpret_cast<const v4i *>(sm.a + (wm * 64 + i * 32 + (lane & 31)) * LDT + kb * 32 + 16 * (lane >> 5));
-                bf[i] = *reinterpret_cast<const v4i *>(sm.b + (wn * 64 + i * 32 + (lane & 31)) * LDT + kb * 32 + 16 * (lane >> 5));
-                ws[i] = sm.w_s[kb][wn * 64 + i * 32 + (lane & 31)];
-                wmn[i] = sm.w_m[kb][wn * 64 + i * 32 + (lane & 31)];
+            for (int j = 0; j < 2; ++j)
+                bf[j] = *reinterpret_cast<const v4i *>(st.b + (wn * 64 + j * 32 + l32) * LDT + kb * 32 + 16 * lh);
+            const float w0 = wsp[kb * BN], w1 = wsp[kb * BN + 32];
+            float ad[16];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float4 d4 = *reinterpret_cast<const float4 *>(&st.a_d[kb][wm * 32 + 8 * g + 4 * lh]);
+                ad[4 * g + 0] = d4.x; ad[4 * g + 1] = d4.y; ad[4 * g + 2] = d4.z; ad[4 * g + 3] = d4.w;
             }
+            const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            const v16i I0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf[0], z, 0, 0, 0);
+            const v16i I1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf[1], z, 0, 0, 0);
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                float ad[16], as[16];
+            for (int v = 0; v < 16; ++v) acc[0][v] = fmaf((float)I0[v], ad[v] * w0, acc[0][v]);
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const int r = wm * 64 + i * 32 + 8 * g + 4 * (lane >> 5);
-                    const float4 d4 = *reinterpret_cast<const float4 *>(&sm.a_d[kb][r]);
-                    const float4 s4 = *reinterpret_cast<const float4 *>(&sm.a_s[kb][r]);
-                    ad[4 * g + 0] = d4.x; ad[4 * g + 1] = d4.y; ad[4 * g + 2] = d4.z; ad[4 * g + 3] = d4.w;
-                    as[4 * g + 0] = s4.x; as[4 * g + 1] = s4.y; as[4 * g + 2] = s4.z; as[4 * g + 3] = s4.w;
-                }
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-                    const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], z, 0, 0, 0);
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        acc[i][j][v] = fmaf((float)I[v], ad[v] * ws[j], acc[i][j][v]);
-                        acc[i][j][v] = fmaf(-as[v], wmn[j], acc[i][j][v]);
-                    }
-                }
-            }
+            for (int v = 0; v < 16; ++v) acc[1][v] = fmaf((float)I1[v], ad[v] * w1, acc[1][v]);
         }
+        // the next step starts a new super-block: its scales replace the ones other waves may still read
+        if (((k0 + BK) & 255) == 0) __syncthreads();
+        if (ks + 1 < n_ksteps) store_stage(regs, sm.st[(ks + 1) & 1], k0 + BK);
+        __syncthreads();
     }
 
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int j = 0; j < 2; ++j) {
+        const int64_t n = n0 + wn * 64 + j * 32 + l32;
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int64_t n = n0 + wn * 64 + j * 32 + (lane & 31);
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int64_t m = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (m < M && n < N) y[m * N + n] = acc[i][j][v];
-            }
+        for (int v = 0; v < 16; ++v) {
+            const int64_t m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (m < M && n < N) y[m * N + n] = acc[j][v];
         }
     }
 }
@@ -159,9 +250,12 @@ __global__ __launch_bounds__(256) void gemm_q4k_q8x32_kernel(const WeightView w,
 }  // namespace
 
 hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
-    if (w.type != kTypeQ4_K || w.K % BK != 0) return hipErrorInvalidValue;
+    if (w.type != kTypeQ4_K || w.K % 256 != 0 || M <= 0) return hipErrorInvalidValue;
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8x32_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem));
+    if (attr != hipSuccess) return attr;
     const dim3 grid((unsigned)((w.N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
-    hipLaunchKernelGGL(gemm_q4k_q8x32_kernel, grid, dim3(256), 0, s, w, a, M, y);
+    hipLaunchKernelGGL(gemm_q4k_q8x32_kernel, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y);
     return hipGetLastError();
 }
 
