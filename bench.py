@@ -9,7 +9,7 @@ the ggml activation mode (the reference CPU path's arithmetic).  `value` is algo
 per step / time.  Extra legs report the dominant kernel against the HBM roofline, the int8-MFMA
 prefill GEMM (config 4), the MoE feed-forward (config 5) and the CPU oracle on the host cores.
 
-    python bench.py --gpus 1 --steps 20 --warmup 3 [--legs step,roofline,prefill,moe,cpu]
+    python bench.py --gpus 1 --steps 20 --warmup 3 [--legs step,roofline,verify,q8_0,prefill,moe,cpu]
 """
 from __future__ import annotations
 
@@ -100,7 +100,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=32)
-    ap.add_argument("--legs", default="step,roofline,prefill,moe,cpu")
+    ap.add_argument("--legs", default="step,roofline,verify,q8_0,prefill,moe,cpu")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--split-quantize", action="store_true",
                     help="run the activation quantizer as a separate launch instead of inside the projection kernel")
@@ -141,7 +141,7 @@ def main():
     # ------------------------------------------------------------------ weights
     L = args.layers
     layers = []
-    need_layers = bool(legs & {"step", "roofline", "cpu"})
+    need_layers = bool(legs & {"step", "roofline", "verify", "cpu"})
     if need_layers:
         t0 = time.time()
         for l in range(L):
@@ -248,6 +248,59 @@ def main():
                 for _ in range(5):
                     torch.add(a, 1, out=b)
             torch.cuda.synchronize()
+
+    # ------------------------------------------------------------------ speculative-verify leg (config 3)
+    if "verify" in legs:
+        res = []
+        for m in (2, 4, 8, 16):
+            xs = {D_MODEL: torch.randn((m, D_MODEL), generator=g, device=dev),
+                  D_FF: torch.randn((m, D_FF), generator=g, device=dev)}
+            ys = {name: torch.empty((m, n), device=dev) for name, _, n, _ in LAYER_TENSORS}
+            for gname, names in (("gate_up", ["gate", "up"]), ("down", ["down"])):
+                k = {nm: kk for nm, _, _, kk in LAYER_TENSORS}[names[0]]
+
+                def all_layers(names=names, k=k):
+                    for lw in layers:
+                        ctx.mul_mat_multi([lw[n] for n in names], xs[k], ACT_GGML, outs=[ys[n] for n in names], sync=False)
+                all_layers()
+                ctx.sync()
+                run = (None if args.no_graph else capture(torch, stream, all_layers)) or all_layers
+                run()
+                torch.cuda.synchronize()
+                ms = timer.time_ms(run, max(5, args.steps)) / L
+                nbytes = sum(gemv_bytes(t, n, kk, m) for nm, t, n, kk in LAYER_TENSORS if nm in names) \
+                    - (len(names) - 1) * m * k * 4
+                res.append({"M": m, "group": gname, "us_per_launch": ms * 1e3, "GBps": nbytes / (ms * 1e-3) / 1e9,
+                            "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
+                log(f"[bench] verify M={m:2d} {gname:8s}: {ms * 1e3:7.2f} us  {res[-1]['GBps']:6.0f} GB/s "
+                    f"({100 * res[-1]['frac_hbm_peak']:.1f}% of peak)")
+        out["verify"] = {"note": "weights read once for all M rows; ggml activation mode", "shapes": res}
+
+    # ------------------------------------------------------------------ Q8_0 leg (config 1)
+    if "q8_0" in legs:
+        nrot = 24            # distinct 4096x4096 Q8_0 matrices (17.8 MB each) rotated through, > Infinity Cache
+        ws = []
+        for i in range(nrot):
+            blocks = synth.random_weight(Q8_0, D_MODEL, D_MODEL, seed=9000 + i, device=dev)
+            ws.append(ctx.upload_from_device(Q8_0, D_MODEL, D_MODEL, blocks))
+            del blocks
+        yq = torch.empty((1, D_MODEL), device=dev)
+
+        def rot():
+            for w in ws:
+                ctx.mul_mat_multi([w], x_attn, ACT_GGML, outs=[yq], sync=False)
+        rot()
+        ctx.sync()
+        run = (None if args.no_graph else capture(torch, stream, rot)) or rot
+        run()
+        torch.cuda.synchronize()
+        ms = timer.time_ms(run, max(5, args.steps)) / nrot
+        nbytes = gemv_bytes(Q8_0, D_MODEL, D_MODEL)
+        out["q8_0"] = {"shape": "4096x4096, M=1", "us_per_launch": ms * 1e3, "GBps": nbytes / (ms * 1e-3) / 1e9,
+                       "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        log(f"[bench] q8_0 4096x4096 M=1: {ms * 1e3:.2f} us  {out['q8_0']['GBps']:.0f} GB/s")
+        for w in ws:
+            w.free()
 
     # ------------------------------------------------------------------ prefill leg (config 4)
     if "prefill" in legs:

@@ -1,0 +1,625 @@
+// Small-batch projection (2..16 activation rows, the speculative-verify regime) on the int8 matrix
+// cores: the weights are streamed from HBM once and every row of activations is applied to them.
+//
+// One v_mfma_i32_32x32x32_i8 (Q4_K, Q8_0) or v_mfma_i32_32x32x16_i8 (Q6_K) multiplies the int8
+// activations of up to 32 tokens (A operand) with one sub-block of 32 weight rows (B operand), so
+// that lane l ends up with the integer dots of weight row l%32 against 8 (or 16) tokens.  A
+// sub-block's integer scale is applied with one v_mad_i32_i24 per output, the super-block's fp32
+// scales once per 256 weights.  The terms that ggml takes from the activation block sums (the
+// Q4_K mins, the -32 offset of Q6_K) are two more products each: block sums split into a signed
+// high and a 6-bit low byte against the 6-bit mins / 8-bit scales.
+//
+// Data movement.  The B operand wants lane l to hold bytes of weight row l%32, i.e. 32 rows that
+// lie K/256 blocks apart in memory; loading it that way touches every cache line from five
+// instructions and thrashes the vector L1.  Instead a wave copies the 32 rows' current
+// super-block with fully coalesced 16-byte loads (consecutive lanes = consecutive 16-byte pieces
+// of a row's block), two super-blocks ahead of the arithmetic, parks the registers in a
+// wave-private LDS region and reads the region back in operand order.  The quantized
+// activations of the workgroup's K range are staged in LDS once.
+//
+// Work split.  A workgroup is 4 waves = rw row groups (32 rows each) x kw K-parts; the K-parts
+// of a row group are summed through LDS in a fixed order.  When one workgroup cannot hold the
+// whole K range (LDS) or there would be too few workgroups, K is also cut into chunks whose
+// results go to a scratch buffer that a second small kernel sums in chunk order, so results do
+// not depend on scheduling.
+#include <stdlib.h>
+
+#include <algorithm>
+
+#include "qproj_device.h"
+#include "qproj_internal.h"
+
+namespace qproj {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+
+struct MfmaTarget {
+    WeightView w;
+    float *y;
+    float *part;       // [n_chunks][M][N] when n_chunks > 1
+    int first_wg;
+    int n_rowsets;
+};
+
+struct MfmaArgs {
+    int n_targets;
+    MfmaTarget t[kMaxTargets];
+    ActView a;
+    int M, n_chunks, chunk_sb, kw, rw, n_wgs;
+};
+
+template <int QT>
+struct Cfg;
+template <>
+struct Cfg<kTypeQ4_K> {
+    static constexpr int kAux = 16;      // per (token, super-block): 8 high + 8 low bytes of the 32-wide block sums
+    static constexpr int kDx = 1;        // activation scales per super-block
+    static constexpr int kRegion = 32 * 144;
+};
+template <>
+struct Cfg<kTypeQ6_K> {
+    static constexpr int kAux = 32;      // 16 high + 16 low bytes of the 16-wide block sums
+    static constexpr int kDx = 1;
+    static constexpr int kQl = 0, kQh = 32 * 144, kSc = kQh + 32 * 80, kD = kSc + 32 * 16;
+    static constexpr int kRegion = kD + 32 * 4;
+};
+template <>
+struct Cfg<kTypeQ8_0> {
+    static constexpr int kAux = 0;
+    static constexpr int kDx = 8;        // Q8_0 activations carry a scale per 32
+    static constexpr int kD = 32 * 272;
+    static constexpr int kRegion = kD + 32 * 16;
+};
+
+struct Layout {
+    int lda, off_dx, off_aux, off_w, total;
+};
+template <int QT, int MT, int W>
+__host__ __device__ inline Layout layout(int chunk_sb) {
+    Layout l;
+    l.lda = chunk_sb * 256 + 16;
+    l.off_dx = MT * l.lda;
+    l.off_aux = l.off_dx + chunk_sb * Cfg<QT>::kDx * MT * 4;
+    l.off_w = l.off_aux + chunk_sb * MT * Cfg<QT>::kAux;
+    l.total = l.off_w + W * Cfg<QT>::kRegion;   // a region doubles as the wave's partial tile at the end
+    return l;
+}
+
+__device__ __forceinline__ int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ v4i as_v4i(const uint4 &u) { return v4i{(int)u.x, (int)u.y, (int)u.z, (int)u.w}; }
+__device__ __forceinline__ long as_i64(uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); }
+__device__ __forceinline__ int sbyte(uint32_t w, int i) { return (int)(int8_t)(w >> (8 * i)); }
+
+// ------------------------------------------------------------------------------------------------
+// Coalesced copy of one super-block of 32 consecutive rows: global -> registers -> wave's LDS region.
+// `row0 + r` is clamped to N - 1 so that a ragged last row group reads valid memory.
+template <int QT>
+struct Stager;
+
+template <>
+struct Stager<kTypeQ4_K> {
+    const uint8_t *base;   // wave-uniform: block 0 of row0
+    uint32_t off[5], lds[5];
+    uint4 r[5];
+    // 288 pieces of 16 bytes: piece p = lane + 64k is bytes 16j.. of row p / 9, j = p % 9
+    // (lanes 32..63 repeat piece 287 in their fifth slot, so every load and store is unpredicated)
+    __device__ __forceinline__ void init(const WeightView &w, int row0, int lane) {
+        const uint32_t row_bytes = (uint32_t)w.nb * 144u;
+        base = w.q4k + (size_t)row0 * row_bytes;
+        const int last = (int)min((int64_t)31, w.N - 1 - row0);
+#pragma unroll
+        for (int k = 0; k < 5; ++k) {
+            int p = lane + 64 * k;
+            if (p > 287) p = 287;
+            const int r = p / 9, j = p - 9 * r;
+            off[k] = (uint32_t)min(r, last) * row_bytes + 16u * j;
+            lds[k] = (uint32_t)p * 16u;
+        }
+    }
+    __device__ __forceinline__ void issue(int sb) {
+        const uint8_t *b = base + (size_t)sb * 144;
+#pragma unroll
+        for (int k = 0; k < 5; ++k) r[k] = *reinterpret_cast<const uint4 *>(b + off[k]);
+    }
+    __device__ __forceinline__ void park(uint8_t *region, int) const {
+#pragma unroll
+        for (int k = 0; k < 5; ++k) *reinterpret_cast<uint4 *>(region + lds[k]) = r[k];
+    }
+};
+
+template <>
+struct Stager<kTypeQ6_K> {
+    // ql: 8 pieces a row (4 per lane), qh: 4 pieces a row (2 per lane), scales: 1 piece a row, d: 2 bytes a row
+    const uint8_t *bl, *bh, *bs, *bd;
+    uint32_t off_l[4], off_h[2], off_s, off_d, lds_l[4], lds_h[2];
+    uint4 l[4], h[2], s;
+    uint32_t d;
+    __device__ __forceinline__ void init(const WeightView &w, int row0, int lane) {
+        const uint32_t nb = (uint32_t)w.nb;
+        bl = w.q6_ql + (size_t)row0 * nb * 128;
+        bh = w.q6_qh + (size_t)row0 * nb * 64;
+        bs = reinterpret_cast<const uint8_t *>(w.q6_sc) + (size_t)row0 * nb * 16;
+        bd = reinterpret_cast<const uint8_t *>(w.q6_d) + (size_t)row0 * nb * 2;
+        const int last = (int)min((int64_t)31, w.N - 1 - row0);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int p = lane + 64 * k, r = p >> 3, j = p & 7;
+            off_l[k] = (uint32_t)min(r, last) * nb * 128u + 16u * j;
+            lds_l[k] = Cfg<kTypeQ6_K>::kQl + r * 144 + 16 * j;
+        }
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            const int p = lane + 64 * k, r = p >> 2, j = p & 3;
+            off_h[k] = (uint32_t)min(r, last) * nb * 64u + 16u * j;
+            lds_h[k] = Cfg<kTypeQ6_K>::kQh + r * 80 + 16 * j;
+        }
+        const uint32_t r = (uint32_t)min(lane & 31, last);
+        off_s = r * nb * 16u;
+        off_d = r * nb * 2u;
+    }
+    __device__ __forceinline__ void issue(int sb) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) l[k] = *reinterpret_cast<const uint4 *>(bl + (size_t)sb * 128 + off_l[k]);
+#pragma unroll
+        for (int k = 0; k < 2; ++k) h[k] = *reinterpret_cast<const uint4 *>(bh + (size_t)sb * 64 + off_h[k]);
+        s = *reinterpret_cast<const uint4 *>(bs + (size_t)sb * 16 + off_s);
+        d = *reinterpret_cast<const uint16_t *>(bd + (size_t)sb * 2 + off_d);
+    }
+    __device__ __forceinline__ void park(uint8_t *region, int lane) const {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) *reinterpret_cast<uint4 *>(region + lds_l[k]) = l[k];
+#pragma unroll
+        for (int k = 0; k < 2; ++k) *reinterpret_cast<uint4 *>(region + lds_h[k]) = h[k];
+        // both lane halves hold the same row's scales and d: identical stores
+        *reinterpret_cast<uint4 *>(region + Cfg<kTypeQ6_K>::kSc + (lane & 31) * 16) = s;
+        *reinterpret_cast<uint32_t *>(region + Cfg<kTypeQ6_K>::kD + (lane & 31) * 4) = d;
+    }
+};
+
+template <>
+struct Stager<kTypeQ8_0> {
+    // one "super-block" = 256 weights = 8 blocks: 16 pieces of quants and one piece of 8 fp16 scales a row
+    const uint8_t *bq, *bd;
+    uint32_t off_q[8], off_d, lds_q[8];
+    uint4 q[8], d;
+    __device__ __forceinline__ void init(const WeightView &w, int row0, int lane) {
+        const uint32_t K = (uint32_t)w.K;
+        bq = reinterpret_cast<const uint8_t *>(w.q8_qs) + (size_t)row0 * K;
+        bd = reinterpret_cast<const uint8_t *>(w.q8_d) + (size_t)row0 * (K / 32) * 2;
+        const int last = (int)min((int64_t)31, w.N - 1 - row0);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int p = lane + 64 * k, r = p >> 4, j = p & 15;
+            off_q[k] = (uint32_t)min(r, last) * K + 16u * j;
+            lds_q[k] = r * 272 + 16 * j;
+        }
+        off_d = (uint32_t)min(lane & 31, last) * (K / 32) * 2u;
+    }
+    __device__ __forceinline__ void issue(int sb) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) q[k] = *reinterpret_cast<const uint4 *>(bq + (size_t)sb * 256 + off_q[k]);
+        d = *reinterpret_cast<const uint4 *>(bd + (size_t)sb * 16 + off_d);
+    }
+    __device__ __forceinline__ void park(uint8_t *region, int lane) const {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) *reinterpret_cast<uint4 *>(region + lds_q[k]) = q[k];
+        *reinterpret_cast<uint4 *>(region + Cfg<kTypeQ8_0>::kD + (lane & 31) * 16) = d;
+    }
+};
+
+// ------------------------------------------------------------------------------------------------
+// One super-block of 32 rows against the staged activations: out[4*i + j] += contribution to token
+// 8*i + 4*h + j of weight row lane % 32.  `region` is the wave's parked copy, `ks` the super-block's
+// index inside the staged K range.
+template <int QT, int NI>
+__device__ __forceinline__ void compute(const uint8_t *region, const uint8_t *smem, const Layout &L, int ks, int lane,
+                                        float (&out)[4 * NI]) {
+    constexpr int MT = 8 * NI, NV = 4 * NI;
+    const int h = lane >> 5, n = lane & 31, mrow = lane & (MT - 1);
+    const v16i z = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    const uint8_t *arow = smem + mrow * L.lda + ks * 256;
+    const float *dxs = reinterpret_cast<const float *>(smem + L.off_dx);
+
+    if constexpr (QT == kTypeQ4_K) {
+        const uint8_t *wrow = region + n * 144;
+        const uint4 hdr = *reinterpret_cast<const uint4 *>(wrow);
+        uint4 qv[4];
+        v4i av[8];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) qv[g] = *reinterpret_cast<const uint4 *>(wrow + 16 + g * 32 + h * 16);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) av[j] = *reinterpret_cast<const v4i *>(arow + j * 32 + h * 16);
+        const uint4 bs = *reinterpret_cast<const uint4 *>(smem + L.off_aux + (ks * MT + mrow) * 16);
+        float4 dxq[NI];
+#pragma unroll
+        for (int i = 0; i < NI; ++i) dxq[i] = *reinterpret_cast<const float4 *>(dxs + ks * MT + 8 * i + 4 * h);
+        __builtin_amdgcn_sched_barrier(0);
+        const ScalesK4 sk = unpack_scales_k4(hdr.y, hdr.z, hdr.w);
+        const float d = h2f(hdr.x), dmin = h2f(hdr.x >> 16);
+        int isum[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) isum[v] = 0;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const uint4 q = qv[g];
+            const v4i lo = {(int)(q.x & 0x0f0f0f0fu), (int)(q.y & 0x0f0f0f0fu), (int)(q.z & 0x0f0f0f0fu),
+                            (int)(q.w & 0x0f0f0f0fu)};
+            const v4i hi = {(int)((q.x >> 4) & 0x0f0f0f0fu), (int)((q.y >> 4) & 0x0f0f0f0fu),
+                            (int)((q.z >> 4) & 0x0f0f0f0fu), (int)((q.w >> 4) & 0x0f0f0f0fu)};
+            const v16i I0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[2 * g], lo, z, 0, 0, 0);
+            const v16i I1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[2 * g + 1], hi, z, 0, 0, 0);
+            const int s0 = (int)scale_k4(sk, 2 * g), s1 = (int)scale_k4(sk, 2 * g + 1);
+#pragma unroll
+            for (int v = 0; v < NV; ++v) isum[v] = __mul24(I1[v], s1) + (__mul24(I0[v], s0) + isum[v]);
+        }
+        const v4i ahi = h ? v4i{0, 0, 0, 0} : v4i{(int)bs.x, (int)bs.y, 0, 0};
+        const v4i alo = h ? v4i{0, 0, 0, 0} : v4i{(int)bs.z, (int)bs.w, 0, 0};
+        const v4i bmn = h ? v4i{0, 0, 0, 0} : v4i{(int)sk.mn_lo, (int)sk.mn_hi, 0, 0};
+        const v16i Mh = __builtin_amdgcn_mfma_i32_32x32x32_i8(ahi, bmn, z, 0, 0, 0);
+        const v16i Ml = __builtin_amdgcn_mfma_i32_32x32x32_i8(alo, bmn, z, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const float dxv[4] = {dxq[i].x, dxq[i].y, dxq[i].z, dxq[i].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int v = 4 * i + j;
+                const int msum = (Mh[v] << 6) + Ml[v];
+                out[v] = fmaf(dxv[j], d * (float)isum[v] - dmin * (float)msum, out[v]);
+            }
+        }
+    } else if constexpr (QT == kTypeQ6_K) {
+        using C = Cfg<kTypeQ6_K>;
+        int isum[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) isum[v] = 0;
+        const uint4 sc = *reinterpret_cast<const uint4 *>(region + C::kSc + n * 16);
+        const uint32_t scw[4] = {sc.x, sc.y, sc.z, sc.w};
+#pragma unroll
+        for (int f = 0; f < 2; ++f)
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                // bytes shared by the four sub-blocks k = 0..3: weights 128f + 32k + 16p + 8h + e
+                const uint2 qa = *reinterpret_cast<const uint2 *>(region + C::kQl + n * 144 + 64 * f + 16 * p + 8 * h);
+                const uint2 qb = *reinterpret_cast<const uint2 *>(region + C::kQl + n * 144 + 64 * f + 32 + 16 * p + 8 * h);
+                const uint2 qh = *reinterpret_cast<const uint2 *>(region + C::kQh + n * 80 + 32 * f + 16 * p + 8 * h);
+                uint32_t wl[4], wh[4];
+                wl[0] = (qa.x & 0x0f0f0f0fu) | ((qh.x << 4) & 0x30303030u);
+                wh[0] = (qa.y & 0x0f0f0f0fu) | ((qh.y << 4) & 0x30303030u);
+                wl[1] = (qb.x & 0x0f0f0f0fu) | ((qh.x << 2) & 0x30303030u);
+                wh[1] = (qb.y & 0x0f0f0f0fu) | ((qh.y << 2) & 0x30303030u);
+                wl[2] = ((qa.x >> 4) & 0x0f0f0f0fu) | (qh.x & 0x30303030u);
+                wh[2] = ((qa.y >> 4) & 0x0f0f0f0fu) | (qh.y & 0x30303030u);
+                wl[3] = ((qb.x >> 4) & 0x0f0f0f0fu) | ((qh.x >> 2) & 0x30303030u);
+                wh[3] = ((qb.y >> 4) & 0x0f0f0f0fu) | ((qh.y >> 2) & 0x30303030u);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const uint2 av = *reinterpret_cast<const uint2 *>(arow + 128 * f + 32 * k + 16 * p + 8 * h);
+                    const v16i I = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64(av.x, av.y), as_i64(wl[k], wh[k]), z, 0, 0, 0);
+                    const int j = 8 * f + 2 * k + p;  // sub-block index
+                    const int s = sbyte(scw[j >> 2], j & 3);
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) isum[v] = __mul24(I[v], s) + isum[v];
+                }
+            }
+        // -32 * sum_j sc_j * bsum_j: block sums split as 64*hi + lo against the 16 scales
+        const uint8_t *aux = smem + L.off_aux + (ks * MT + mrow) * 32;
+        const uint2 bhi = *reinterpret_cast<const uint2 *>(aux + 8 * h);
+        const uint2 blo = *reinterpret_cast<const uint2 *>(aux + 16 + 8 * h);
+        const long bsc = h ? as_i64(sc.z, sc.w) : as_i64(sc.x, sc.y);
+        const v16i Ch = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64(bhi.x, bhi.y), bsc, z, 0, 0, 0);
+        const v16i Cl = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64(blo.x, blo.y), bsc, z, 0, 0, 0);
+        const float d = h2f(*reinterpret_cast<const uint32_t *>(region + C::kD + n * 4));
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const float4 dx = *reinterpret_cast<const float4 *>(dxs + ks * MT + 8 * i + 4 * h);
+            const float dxv[4] = {dx.x, dx.y, dx.z, dx.w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int v = 4 * i + j;
+                const int corr = (Ch[v] << 6) + Cl[v];
+                out[v] = fmaf(dxv[j] * d, (float)(isum[v] - 32 * corr), out[v]);
+            }
+        }
+    } else {
+        using C = Cfg<kTypeQ8_0>;
+        const uint4 dq = *reinterpret_cast<const uint4 *>(region + C::kD + n * 16);
+        const uint32_t dw[4] = {dq.x, dq.y, dq.z, dq.w};
+#pragma unroll
+        for (int blk = 0; blk < 8; ++blk) {
+            const v4i av = *reinterpret_cast<const v4i *>(arow + blk * 32 + h * 16);
+            const uint4 q = *reinterpret_cast<const uint4 *>(region + n * 272 + blk * 32 + h * 16);
+            const v16i I = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, as_v4i(q), z, 0, 0, 0);
+            const float wd = h2f(dw[blk >> 1] >> (16 * (blk & 1)));
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const float4 dx = *reinterpret_cast<const float4 *>(dxs + (ks * 8 + blk) * MT + 8 * i + 4 * h);
+                const float dxv[4] = {dx.x, dx.y, dx.z, dx.w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) out[4 * i + j] = fmaf((float)I[4 * i + j], wd * dxv[j], out[4 * i + j]);
+            }
+        }
+    }
+}
+
+// splits a block sum into a signed high byte and a 6-bit low byte: s = 64*hi + lo
+__device__ __forceinline__ void split_sum(int s, uint32_t &hi, uint32_t &lo, int pos) {
+    hi |= (uint32_t)((s >> 6) & 0xff) << (8 * pos);
+    lo |= (uint32_t)(s & 63) << (8 * pos);
+}
+
+// Copies the quantized activations of super-blocks [c0, c0 + nsb) (all M rows) into LDS.
+template <int QT, int MT, int kThreads>
+__device__ __forceinline__ void stage_activations(const MfmaArgs &g, uint8_t *smem, const Layout &L, int c0, int nsb) {
+    const int tid = threadIdx.x;
+    const int nb = (int)(g.a.K >> 8);
+    const int row16 = nsb * 16;
+    const int total = g.M * row16;
+    for (int base = 0; base < total; base += 4 * kThreads) {
+        uint4 v[4];
+        int dst[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {   // four independent loads in flight per thread
+            const int idx = min(base + u * kThreads + tid, total - 1);
+            const int m = idx / row16, j = idx - m * row16;
+            v[u] = *reinterpret_cast<const uint4 *>(g.a.qs + (size_t)m * g.a.K + (size_t)c0 * 256 + j * 16);
+            dst[u] = m * L.lda + j * 16;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) *reinterpret_cast<uint4 *>(smem + dst[u]) = v[u];
+    }
+    float *dxs = reinterpret_cast<float *>(smem + L.off_dx);
+    constexpr int ND = Cfg<QT>::kDx;
+    const int nd = nsb * ND;  // scales per row in this range
+    for (int idx = tid; idx < g.M * nd; idx += kThreads) {
+        const int m = idx / nd, j = idx - m * nd;
+        dxs[j * MT + m] = g.a.d[(size_t)m * (nb * ND) + c0 * ND + j];
+    }
+    if constexpr (QT != kTypeQ8_0) {
+        for (int idx = tid; idx < g.M * nsb; idx += kThreads) {
+            const int m = idx / nsb, sb = idx - m * nsb;
+            const uint4 *src = reinterpret_cast<const uint4 *>(g.a.bsums + ((size_t)m * nb + c0 + sb) * 16);
+            const uint4 b0 = src[0], b1 = src[1];
+            const uint32_t w[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+            uint8_t *dst = smem + L.off_aux + (sb * MT + m) * Cfg<QT>::kAux;
+            if constexpr (QT == kTypeQ4_K) {
+                uint32_t hi[2] = {0, 0}, lo[2] = {0, 0};
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int s = (int)(int16_t)(w[j] & 0xffff) + (int)(int16_t)(w[j] >> 16);
+                    split_sum(s, hi[j >> 2], lo[j >> 2], j & 3);
+                }
+                *reinterpret_cast<uint4 *>(dst) = make_uint4(hi[0], hi[1], lo[0], lo[1]);
+            } else {
+                uint32_t hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const int s = (int)(int16_t)((w[j >> 1] >> (16 * (j & 1))) & 0xffff);
+                    split_sum(s, hi[j >> 2], lo[j >> 2], j & 3);
+                }
+                *reinterpret_cast<uint4 *>(dst) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+                *reinterpret_cast<uint4 *>(dst + 16) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+            }
+        }
+    }
+}
+
+template <int QT, int NI, int W>
+__global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int MT = 8 * NI, NV = 4 * NI;
+    const Layout L = layout<QT, MT, W>(g.chunk_sb);
+    const int lane = threadIdx.x & 63, wave = uniform(threadIdx.x >> 6);
+    const int h = lane >> 5, nl = lane & 31;
+
+    // workgroup -> (tensor, K chunk, set of rw row groups)
+    int ti = 0;
+#pragma unroll
+    for (int i = 1; i < kMaxTargets; ++i)
+        if (i < g.n_targets && (int)blockIdx.x >= g.t[i].first_wg) ti = i;
+    WeightView w = g.t[0].w;
+    float *y = g.t[0].y, *part = g.t[0].part;
+    int first = g.t[0].first_wg, nrs = g.t[0].n_rowsets;
+#pragma unroll
+    for (int i = 1; i < kMaxTargets; ++i)
+        if (ti == i) {
+            w = g.t[i].w;
+            y = g.t[i].y;
+            part = g.t[i].part;
+            first = g.t[i].first_wg;
+            nrs = g.t[i].n_rowsets;
+        }
+    const int local = (int)blockIdx.x - first;
+    const int c = local / nrs, rs = local - c * nrs;
+    const int nb = (int)(g.a.K >> 8);
+    const int c0 = c * g.chunk_sb, nsb = min(g.chunk_sb, nb - c0);
+
+    // wave -> (row group, K part)
+    const int rgl = wave / g.kw, kp = wave - rgl * g.kw;
+    const int row0 = (rs * g.rw + rgl) * 32;
+    const int part_sb = (nsb + g.kw - 1) / g.kw;
+    const int s0 = min(kp * part_sb, nsb), s1 = min(s0 + part_sb, nsb);  // range inside the staged chunk
+    const bool rows_ok = row0 < (int)w.N;
+    const int steps = rows_ok ? s1 - s0 : 0;
+    const int last = c0 + (steps > 0 ? s1 - 1 : 0);   // loads past the range repeat its last super-block
+
+    Stager<QT> sa, sb_;
+    sa.init(w, rows_ok ? row0 : 0, lane);
+    sb_ = sa;
+    sa.issue(min(c0 + s0, last));
+    sb_.issue(min(c0 + s0 + 1, last));
+
+    stage_activations<QT, MT, W * 64>(g, smem, L, c0, nsb);
+    __syncthreads();
+
+    uint8_t *region = smem + L.off_w + wave * Cfg<QT>::kRegion;
+    float out[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) out[v] = 0.f;
+    int s = 0;
+    for (; s + 1 < steps; s += 2) {
+        sa.park(region, lane);
+        sa.issue(min(c0 + s0 + s + 2, last));
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        compute<QT, NI>(region, smem, L, s0 + s, lane, out);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        sb_.park(region, lane);
+        sb_.issue(min(c0 + s0 + s + 3, last));
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        compute<QT, NI>(region, smem, L, s0 + s + 1, lane, out);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    }
+    if (s < steps) {
+        sa.park(region, lane);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        compute<QT, NI>(region, smem, L, s0 + s, lane, out);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    }
+
+    // sum the K parts of a row group in a fixed order (through the waves' regions), then store
+    if (g.kw > 1) {
+        float *mine = reinterpret_cast<float *>(region);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) mine[(8 * (v >> 2) + 4 * h + (v & 3)) * 32 + nl] = out[v];
+        __syncthreads();
+        if (kp == 0) {
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                const uint8_t *src = region + ((8 * (v >> 2) + 4 * h + (v & 3)) * 32 + nl) * 4;
+                float t = *reinterpret_cast<const float *>(src);
+                for (int q = 1; q < g.kw; ++q) t += *reinterpret_cast<const float *>(src + q * Cfg<QT>::kRegion);
+                out[v] = t;
+            }
+        }
+    }
+    if (kp == 0 && rows_ok) {
+        const int N = (int)w.N;
+        float *dst = g.n_chunks == 1 ? y : part + (size_t)c * g.M * N;
+        const int n = row0 + nl;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int m = 8 * (v >> 2) + 4 * h + (v & 3);
+            if (m < g.M && n < N) dst[(size_t)m * N + n] = out[v];
+        }
+    }
+}
+
+// y[i] = sum over chunks of part[c][i], chunk order fixed
+__global__ __launch_bounds__(256) void sum_chunks_kernel(const MfmaArgs g) {
+    for (int ti = 0; ti < g.n_targets; ++ti) {
+        const size_t n = (size_t)g.M * g.t[ti].w.N;
+        for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+            float s = g.t[ti].part[i];
+            for (int c = 1; c < g.n_chunks; ++c) s += g.t[ti].part[(size_t)c * n + i];
+            g.t[ti].y[i] = s;
+        }
+    }
+}
+
+template <int QT, int NI, int W>
+hipError_t launch_one(const MfmaArgs &g, hipStream_t s) {
+    const Layout L = layout<QT, 8 * NI, W>(g.chunk_sb);
+    auto kern = gemv_mfma_kernel<QT, NI, W>;
+    static int allowed = 0;
+    if (L.total > allowed) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, L.total);
+        if (e != hipSuccess) return e;
+        allowed = L.total;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)g.n_wgs), dim3(W * 64), (size_t)L.total, s, g);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || g.n_chunks == 1) return e;
+    size_t n_out = 0;
+    for (int i = 0; i < g.n_targets; ++i) n_out = std::max(n_out, (size_t)g.M * (size_t)g.t[i].w.N);
+    const unsigned blocks = (unsigned)std::min<size_t>(256, (n_out + 255) / 256);
+    hipLaunchKernelGGL(sum_chunks_kernel, dim3(blocks), dim3(256), 0, s, g);
+    return hipGetLastError();
+}
+
+int waves_per_wg(int type) {
+    static const int w = [] {
+        const char *e = getenv("QPROJ_MFMA_WAVES");
+        const int v = e ? atoi(e) : 8;
+        return v == 4 || v == 16 ? v : 8;
+    }();
+    return w == 16 && type != kTypeQ4_K ? 8 : w;   // 16 regions of the larger formats do not fit LDS
+}
+
+// The split of K: how many chunks (workgroups along K) and K parts (waves along K inside a workgroup).
+struct Split {
+    int n_chunks, chunk_sb, kw;
+};
+Split plan(int64_t K, int64_t M, int64_t total_rg, int W) {
+    const int nb = (int)(K / 256);
+    const int max_sb = M <= 8 ? 32 : 16;  // staged activations stay under ~66 KB of LDS
+    Split p;
+    p.kw = 1;
+    while (p.kw < W && p.kw * 2 <= nb && total_rg * p.kw / W < 200) p.kw *= 2;
+    const int rw = W / p.kw;
+    const int64_t wgs1 = (total_rg + rw - 1) / rw;
+    int nc = (nb + max_sb - 1) / max_sb;
+    if (wgs1 * nc < 128) nc = std::max(nc, (int)std::min<int64_t>(std::max(1, nb / p.kw), (255 + wgs1) / wgs1));
+    p.chunk_sb = (nb + nc - 1) / nc;
+    p.n_chunks = (nb + p.chunk_sb - 1) / p.chunk_sb;
+    return p;
+}
+
+template <int QT, int NI>
+hipError_t launch_w(const MfmaArgs &g, int W, hipStream_t s) {
+    if (W == 4) return launch_one<QT, NI, 4>(g, s);
+    if constexpr (QT == kTypeQ4_K)
+        if (W == 16) return launch_one<QT, NI, 16>(g, s);
+    return launch_one<QT, NI, 8>(g, s);
+}
+
+}  // namespace
+
+bool mfma_gemv_fits(int type, int64_t M, int64_t K) {
+    (void)type;
+    return M >= 1 && M <= 16 && K % 256 == 0;
+}
+
+size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, int64_t total_rg) {
+    const Split p = plan(K, M, total_rg, waves_per_wg(type));
+    return p.n_chunks > 1 ? (size_t)p.n_chunks * (size_t)M * (size_t)sum_n * 4 : 0;
+}
+
+hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s) {
+    MfmaArgs g{};
+    g.n_targets = args.n_targets;
+    g.a = args.a;
+    g.M = args.M;
+    int64_t total_rg = 0;
+    for (int i = 0; i < args.n_targets; ++i) total_rg += (args.t[i].w.N + 31) / 32;
+    const int W = waves_per_wg(args.t[0].w.type);
+    const Split p = plan(args.a.K, args.M, total_rg, W);
+    g.n_chunks = p.n_chunks;
+    g.chunk_sb = p.chunk_sb;
+    g.kw = p.kw;
+    g.rw = W / p.kw;
+    int wg = 0;
+    size_t part_off = 0;
+    for (int i = 0; i < args.n_targets; ++i) {
+        g.t[i].w = args.t[i].w;
+        g.t[i].y = args.t[i].y;
+        g.t[i].part = scratch ? scratch + part_off : nullptr;
+        part_off += (size_t)g.n_chunks * args.M * args.t[i].w.N;
+        const int n_rg = (int)((args.t[i].w.N + 31) / 32);
+        g.t[i].n_rowsets = (n_rg + g.rw - 1) / g.rw;
+        g.t[i].first_wg = wg;
+        wg += g.t[i].n_rowsets * g.n_chunks;
+    }
+    g.n_wgs = wg;
+    if (g.n_chunks > 1 && !scratch) return hipErrorInvalidValue;
+    const int type = args.t[0].w.type;
+    const bool small = args.M <= 8;
+    if (type == kTypeQ4_K) return small ? launch_w<kTypeQ4_K, 1>(g, W, s) : launch_w<kTypeQ4_K, 2>(g, W, s);
+    if (type == kTypeQ6_K) return small ? launch_w<kTypeQ6_K, 1>(g, W, s) : launch_w<kTypeQ6_K, 2>(g, W, s);
+    return small ? launch_w<kTypeQ8_0, 1>(g, W, s) : launch_w<kTypeQ8_0, 2>(g, W, s);
+}
+
+}  // namespace qproj

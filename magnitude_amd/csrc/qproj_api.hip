@@ -235,8 +235,43 @@ bool use_decode_kernel(int type, int64_t M, int64_t K) {
     return !off && M <= 4 && decode_kernel_fits(type, pow2_ceil(M), K);
 }
 
+bool use_mfma_kernel(int type, int64_t M, int64_t K) {
+    static const bool off = getenv("QPROJ_NO_MFMA_GEMV") != nullptr;
+    static const int min_m = getenv("QPROJ_MFMA_MIN_M") ? atoi(getenv("QPROJ_MFMA_MIN_M")) : 3;
+    return !off && M >= min_m && mfma_gemv_fits(type, std::min<int64_t>(M, 16), K);
+}
+
+// scratch bytes run_dense_q8act needs for M rows against these tensors
+size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
+    if (!use_mfma_kernel(w[0]->type, M, w[0]->K)) return 0;
+    int64_t sum_n = 0, rgs = 0;
+    for (int i = 0; i < n; ++i) {
+        sum_n += w[i]->N;
+        rgs += (w[i]->N + 31) / 32;
+    }
+    size_t need = mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, std::min<int64_t>(M, 16), sum_n, rgs);
+    if (M > 16 && M % 16) need = std::max(need, mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, M % 16, sum_n, rgs));
+    return need;
+}
+
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
-                    float *const *y) {
+                    float *const *y, float *scratch) {
+    if (use_mfma_kernel(w[0]->type, M, w[0]->K)) {
+        for (int64_t m0 = 0; m0 < M; m0 += 16) {
+            const int64_t mc = std::min<int64_t>(16, M - m0);
+            GemvArgs g{};
+            g.n_targets = n;
+            for (int i = 0; i < n; ++i) {
+                g.t[i].w = w[i]->view;
+                g.t[i].y = y[i] + m0 * w[i]->N;
+            }
+            g.a = act_rows(a, m0);
+            g.M = (int)mc;
+            g.x_div = 1;
+            QP_HIP(ctx, launch_gemv_mfma(g, scratch, ctx->stream));
+        }
+        return QPROJ_OK;
+    }
     if (use_decode_kernel(w[0]->type, M, w[0]->K)) {
         GemvArgs g{};
         g.n_targets = n;
@@ -465,7 +500,7 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
     if (M == 0) return QPROJ_OK;
     QP_HIP(ctx, hipSetDevice(ctx->device));
     const int64_t K = w[0]->K;
-    if (act == kActGGML && use_decode_kernel(w[0]->type, M, K)) {
+    if (act == kActGGML && !use_mfma_kernel(w[0]->type, M, K) && use_decode_kernel(w[0]->type, M, K)) {
         // decode regime: the kernel quantizes the activation rows itself, no scratch needed
         GemvArgs g{};
         g.n_targets = n;
@@ -483,11 +518,13 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
         if (act == kActQ8X32 && w[0]->type != kTypeQ4_K)
             return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat: the per-32 int8 path is built for Q4_K weights");
         const ActPlanes p = act_planes(act_kind_for(act, w[0]->type), M, K);
-        int rc = ensure_ws(ctx, p.total);
+        const size_t extra = act == kActGGML ? dense_scratch_bytes(n, w, M) : 0;
+        int rc = ensure_ws(ctx, p.total + extra);
         if (rc) return rc;
         QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, M, K));
         const ActView a = act_view(p, ctx->ws, K);
-        if (act == kActGGML) return run_dense_q8act(ctx, n, w, a, M, y_dev);
+        if (act == kActGGML)
+            return run_dense_q8act(ctx, n, w, a, M, y_dev, reinterpret_cast<float *>(ctx->ws + p.total));
         for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], ctx->stream));
         return QPROJ_OK;
     }
@@ -528,7 +565,11 @@ int qproj_mul_mat_quantized(qproj_ctx *ctx, int n, const qproj_weight *const *w,
     const int64_t K = w[0]->K;
     const ActPlanes p = act_planes(act_kind_for(kind, w[0]->type), M, K);
     const ActView a = act_view(p, static_cast<uint8_t *>(const_cast<void *>(act_dev)), K);
-    if (kind == kActGGML) return run_dense_q8act(ctx, n, w, a, M, y_dev);
+    if (kind == kActGGML) {
+        int rc = ensure_ws(ctx, dense_scratch_bytes(n, w, M));
+        if (rc) return rc;
+        return run_dense_q8act(ctx, n, w, a, M, y_dev, reinterpret_cast<float *>(ctx->ws));
+    }
     for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], ctx->stream));
     return QPROJ_OK;
 }

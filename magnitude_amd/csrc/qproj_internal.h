@@ -79,6 +79,11 @@ hipError_t launch_gemv_q8act(const GemvArgs &args, int mt, int n_experts_grid, h
 // persistent decode kernel (mt <= 4 rows); fuse_quantize: args.x holds fp32 rows, else args.a
 bool decode_kernel_fits(int type, int mt, int64_t K);
 hipError_t launch_gemv_decode(const GemvArgs &args, int mt, bool fuse_quantize, hipStream_t s);
+// int8 matrix-core kernel for 1..16 activation rows (K % 256 == 0); `scratch` holds the per-K-chunk
+// results when K > 4096 (mfma_gemv_scratch_bytes, 0 if none is needed)
+bool mfma_gemv_fits(int type, int64_t M, int64_t K);
+size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, int64_t total_row_groups);
+hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s);
 hipError_t launch_gemv_f32(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
 hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_expert, int32_t *order,
                             int32_t *offsets, int32_t *error_flag, hipStream_t s);
