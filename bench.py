@@ -352,15 +352,19 @@ def main():
             x = torch.randn((B, dm), generator=g, device=dev)
             distinct = int(torch.unique(ids).numel())
             torch.cuda.synchronize()
-            f = lambda: ctx.moe_ffn(exps["gate"], exps["up"], exps["down"], x, ids, wts, ACT_GGML, sync=False)
+            yb = torch.empty((B, dm), device=dev)
+            f = lambda: ctx.moe_ffn(exps["gate"], exps["up"], exps["down"], x, ids, wts, ACT_GGML, out=yb, sync=False)
             f(); ctx.sync()
-            ms = timer.time_ms(f, 20)
+            run = (None if args.no_graph else capture(torch, stream, f)) or f
+            run(); torch.cuda.synchronize()
+            ms = timer.time_ms(run, 20)
             byts = distinct * per_expert + B * dm * 4 * 2
             res.append({"B": B, "distinct_experts": distinct, "ms": ms, "GBps": byts / (ms * 1e-3) / 1e9,
                         "frac_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
             log(f"[bench] moe B={B}: {ms * 1e3:.1f} us, {distinct} experts, {res[-1]['GBps']:.0f} GB/s")
         out["moe"] = {"experts": E, "top": top, "d_model": dm, "d_ff": dff, "batches": res,
-                      "note": "5 launches per call, eager; not rotated out of the Infinity Cache"}
+                      "note": "6 launches per call (quantize, group, gate/up+SwiGLU, quantize, down, combine), replayed as a HIP graph; "
+                              "the same experts every replay, so weights may sit in the Infinity Cache"}
         for w in exps.values():
             w.free()
 

@@ -50,6 +50,13 @@ struct MfmaArgs {
     MfmaTarget t[kMaxTargets];
     ActView a;
     int M, n_chunks, chunk_sb, kw, rw, n_wgs;
+    // expert-grouped mode (MUL_MAT_ID): activation rows of expert e are the pairs order[offsets[e]..offsets[e+1])
+    const int32_t *order;
+    const int32_t *offsets;
+    const int32_t *active;  // experts that have pairs; active[n_expert] = how many
+    int n_expert;
+    int x_div;             // activation row of pair p is p / x_div
+    int wgs_per_expert;
 };
 
 template <int QT>
@@ -76,7 +83,7 @@ struct Cfg<kTypeQ8_0> {
 };
 
 struct Layout {
-    int lda, off_dx, off_aux, off_w, total;
+    int lda, off_dx, off_aux, off_map, off_w, total;
 };
 template <int QT, int MT, int W>
 __host__ __device__ inline Layout layout(int chunk_sb) {
@@ -84,7 +91,8 @@ __host__ __device__ inline Layout layout(int chunk_sb) {
     l.lda = chunk_sb * 256 + 16;
     l.off_dx = MT * l.lda;
     l.off_aux = l.off_dx + chunk_sb * Cfg<QT>::kDx * MT * 4;
-    l.off_w = l.off_aux + chunk_sb * MT * Cfg<QT>::kAux;
+    l.off_map = l.off_aux + chunk_sb * MT * Cfg<QT>::kAux;   // MT ints: which pair each staged row is
+    l.off_w = l.off_map + MT * 4;
     l.total = l.off_w + W * Cfg<QT>::kRegion;   // a region doubles as the wave's partial tile at the end
     return l;
 }
@@ -102,15 +110,16 @@ struct Stager;
 
 template <>
 struct Stager<kTypeQ4_K> {
-    const uint8_t *base;   // wave-uniform: block 0 of row0
+    v4i r[5];                 // first member: no padding in front of the 16-byte registers
+    const uint8_t *base[2];   // wave-uniform: block 0 of the first row, per tensor (gate / up)
     uint32_t off[5], lds[5];
-    uint4 r[5];
     // 288 pieces of 16 bytes: piece p = lane + 64k is bytes 16j.. of row p / 9, j = p % 9
     // (lanes 32..63 repeat piece 287 in their fifth slot, so every load and store is unpredicated)
-    __device__ __forceinline__ void init(const WeightView &w, int row0, int lane) {
+    __device__ __forceinline__ void rebase(int t, const WeightView &w, int64_t row) {
+        base[t] = w.q4k + (size_t)row * (size_t)w.nb * 144;
+    }
+    __device__ __forceinline__ void init(const WeightView &w, int last, int lane) {
         const uint32_t row_bytes = (uint32_t)w.nb * 144u;
-        base = w.q4k + (size_t)row0 * row_bytes;
-        const int last = (int)min((int64_t)31, w.N - 1 - row0);
 #pragma unroll
         for (int k = 0; k < 5; ++k) {
             int p = lane + 64 * k;
@@ -120,31 +129,33 @@ struct Stager<kTypeQ4_K> {
             lds[k] = (uint32_t)p * 16u;
         }
     }
-    __device__ __forceinline__ void issue(int sb) {
-        const uint8_t *b = base + (size_t)sb * 144;
+    __device__ __forceinline__ void issue(int t, int sb) {
+        const uint8_t *b = (t ? base[1] : base[0]) + (size_t)sb * 144;
 #pragma unroll
-        for (int k = 0; k < 5; ++k) r[k] = *reinterpret_cast<const uint4 *>(b + off[k]);
+        for (int k = 0; k < 5; ++k) r[k] = *reinterpret_cast<const v4i *>(b + off[k]);
     }
     __device__ __forceinline__ void park(uint8_t *region, int) const {
 #pragma unroll
-        for (int k = 0; k < 5; ++k) *reinterpret_cast<uint4 *>(region + lds[k]) = r[k];
+        for (int k = 0; k < 5; ++k) *reinterpret_cast<v4i *>(region + lds[k]) = r[k];
     }
 };
 
 template <>
 struct Stager<kTypeQ6_K> {
     // ql: 8 pieces a row (4 per lane), qh: 4 pieces a row (2 per lane), scales: 1 piece a row, d: 2 bytes a row
-    const uint8_t *bl, *bh, *bs, *bd;
+    v4i l[4], h[2], s;        // first members: no padding in front of the 16-byte registers
+    const uint8_t *bl[2], *bh[2], *bs[2], *bd[2];
     uint32_t off_l[4], off_h[2], off_s, off_d, lds_l[4], lds_h[2];
-    uint4 l[4], h[2], s;
     uint32_t d;
-    __device__ __forceinline__ void init(const WeightView &w, int row0, int lane) {
+    __device__ __forceinline__ void rebase(int t, const WeightView &w, int64_t row) {
+        const size_t rb = (size_t)row * (size_t)w.nb;
+        bl[t] = w.q6_ql + rb * 128;
+        bh[t] = w.q6_qh + rb * 64;
+        bs[t] = reinterpret_cast<const uint8_t *>(w.q6_sc) + rb * 16;
+        bd[t] = reinterpret_cast<const uint8_t *>(w.q6_d) + rb * 2;
+    }
+    __device__ __forceinline__ void init(const WeightView &w, int last, int lane) {
         const uint32_t nb = (uint32_t)w.nb;
-        bl = w.q6_ql + (size_t)row0 * nb * 128;
-        bh = w.q6_qh + (size_t)row0 * nb * 64;
-        bs = reinterpret_cast<const uint8_t *>(w.q6_sc) + (size_t)row0 * nb * 16;
-        bd = reinterpret_cast<const uint8_t *>(w.q6_d) + (size_t)row0 * nb * 2;
-        const int last = (int)min((int64_t)31, w.N - 1 - row0);
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             const int p = lane + 64 * k, r = p >> 3, j = p & 7;
@@ -161,21 +172,23 @@ struct Stager<kTypeQ6_K> {
         off_s = r * nb * 16u;
         off_d = r * nb * 2u;
     }
-    __device__ __forceinline__ void issue(int sb) {
+    __device__ __forceinline__ void issue(int t, int sb) {
+        const uint8_t *pl = (t ? bl[1] : bl[0]) + (size_t)sb * 128, *ph = (t ? bh[1] : bh[0]) + (size_t)sb * 64;
+        const uint8_t *ps = (t ? bs[1] : bs[0]) + (size_t)sb * 16, *pd = (t ? bd[1] : bd[0]) + (size_t)sb * 2;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) l[k] = *reinterpret_cast<const uint4 *>(bl + (size_t)sb * 128 + off_l[k]);
+        for (int k = 0; k < 4; ++k) l[k] = *reinterpret_cast<const v4i *>(pl + off_l[k]);
 #pragma unroll
-        for (int k = 0; k < 2; ++k) h[k] = *reinterpret_cast<const uint4 *>(bh + (size_t)sb * 64 + off_h[k]);
-        s = *reinterpret_cast<const uint4 *>(bs + (size_t)sb * 16 + off_s);
-        d = *reinterpret_cast<const uint16_t *>(bd + (size_t)sb * 2 + off_d);
+        for (int k = 0; k < 2; ++k) h[k] = *reinterpret_cast<const v4i *>(ph + off_h[k]);
+        s = *reinterpret_cast<const v4i *>(ps + off_s);
+        d = *reinterpret_cast<const uint16_t *>(pd + off_d);
     }
     __device__ __forceinline__ void park(uint8_t *region, int lane) const {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) *reinterpret_cast<uint4 *>(region + lds_l[k]) = l[k];
+        for (int k = 0; k < 4; ++k) *reinterpret_cast<v4i *>(region + lds_l[k]) = l[k];
 #pragma unroll
-        for (int k = 0; k < 2; ++k) *reinterpret_cast<uint4 *>(region + lds_h[k]) = h[k];
+        for (int k = 0; k < 2; ++k) *reinterpret_cast<v4i *>(region + lds_h[k]) = h[k];
         // both lane halves hold the same row's scales and d: identical stores
-        *reinterpret_cast<uint4 *>(region + Cfg<kTypeQ6_K>::kSc + (lane & 31) * 16) = s;
+        *reinterpret_cast<v4i *>(region + Cfg<kTypeQ6_K>::kSc + (lane & 31) * 16) = s;
         *reinterpret_cast<uint32_t *>(region + Cfg<kTypeQ6_K>::kD + (lane & 31) * 4) = d;
     }
 };
@@ -183,14 +196,15 @@ struct Stager<kTypeQ6_K> {
 template <>
 struct Stager<kTypeQ8_0> {
     // one "super-block" = 256 weights = 8 blocks: 16 pieces of quants and one piece of 8 fp16 scales a row
-    const uint8_t *bq, *bd;
+    v4i q[8], d;              // first members: no padding in front of the 16-byte registers
+    const uint8_t *bq[2], *bd[2];
     uint32_t off_q[8], off_d, lds_q[8];
-    uint4 q[8], d;
-    __device__ __forceinline__ void init(const WeightView &w, int row0, int lane) {
+    __device__ __forceinline__ void rebase(int t, const WeightView &w, int64_t row) {
+        bq[t] = reinterpret_cast<const uint8_t *>(w.q8_qs) + (size_t)row * (size_t)w.K;
+        bd[t] = reinterpret_cast<const uint8_t *>(w.q8_d) + (size_t)row * (size_t)(w.K / 32) * 2;
+    }
+    __device__ __forceinline__ void init(const WeightView &w, int last, int lane) {
         const uint32_t K = (uint32_t)w.K;
-        bq = reinterpret_cast<const uint8_t *>(w.q8_qs) + (size_t)row0 * K;
-        bd = reinterpret_cast<const uint8_t *>(w.q8_d) + (size_t)row0 * (K / 32) * 2;
-        const int last = (int)min((int64_t)31, w.N - 1 - row0);
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             const int p = lane + 64 * k, r = p >> 4, j = p & 15;
@@ -199,15 +213,16 @@ struct Stager<kTypeQ8_0> {
         }
         off_d = (uint32_t)min(lane & 31, last) * (K / 32) * 2u;
     }
-    __device__ __forceinline__ void issue(int sb) {
+    __device__ __forceinline__ void issue(int t, int sb) {
+        const uint8_t *pq = (t ? bq[1] : bq[0]) + (size_t)sb * 256, *pd = (t ? bd[1] : bd[0]) + (size_t)sb * 16;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) q[k] = *reinterpret_cast<const uint4 *>(bq + (size_t)sb * 256 + off_q[k]);
-        d = *reinterpret_cast<const uint4 *>(bd + (size_t)sb * 16 + off_d);
+        for (int k = 0; k < 8; ++k) q[k] = *reinterpret_cast<const v4i *>(pq + off_q[k]);
+        d = *reinterpret_cast<const v4i *>(pd + off_d);
     }
     __device__ __forceinline__ void park(uint8_t *region, int lane) const {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) *reinterpret_cast<uint4 *>(region + lds_q[k]) = q[k];
-        *reinterpret_cast<uint4 *>(region + Cfg<kTypeQ8_0>::kD + (lane & 31) * 16) = d;
+        for (int k = 0; k < 8; ++k) *reinterpret_cast<v4i *>(region + lds_q[k]) = q[k];
+        *reinterpret_cast<v4i *>(region + Cfg<kTypeQ8_0>::kD + (lane & 31) * 16) = d;
     }
 };
 
@@ -351,13 +366,17 @@ __device__ __forceinline__ void split_sum(int s, uint32_t &hi, uint32_t &lo, int
     lo |= (uint32_t)(s & 63) << (8 * pos);
 }
 
-// Copies the quantized activations of super-blocks [c0, c0 + nsb) (all M rows) into LDS.
-template <int QT, int MT, int kThreads>
-__device__ __forceinline__ void stage_activations(const MfmaArgs &g, uint8_t *smem, const Layout &L, int c0, int nsb) {
+// Copies the quantized activations of super-blocks [c0, c0 + nsb) into LDS: staged row m (< n_rows) comes from
+// activation row src_row(m).
+template <int QT, int MT, int kThreads, bool MAPPED>
+__device__ __forceinline__ void stage_activations(const MfmaArgs &g, uint8_t *smem, const Layout &L, int c0, int nsb,
+                                                  int n_rows, int m0) {
     const int tid = threadIdx.x;
     const int nb = (int)(g.a.K >> 8);
     const int row16 = nsb * 16;
-    const int total = g.M * row16;
+    const int *map = reinterpret_cast<const int *>(smem + L.off_map);
+    auto src_row = [&](int m) -> size_t { return MAPPED ? (size_t)(map[m] / g.x_div) : (size_t)(m0 + m); };
+    const int total = n_rows * row16;
     for (int base = 0; base < total; base += 4 * kThreads) {
         uint4 v[4];
         int dst[4];
@@ -365,7 +384,7 @@ __device__ __forceinline__ void stage_activations(const MfmaArgs &g, uint8_t *sm
         for (int u = 0; u < 4; ++u) {   // four independent loads in flight per thread
             const int idx = min(base + u * kThreads + tid, total - 1);
             const int m = idx / row16, j = idx - m * row16;
-            v[u] = *reinterpret_cast<const uint4 *>(g.a.qs + (size_t)m * g.a.K + (size_t)c0 * 256 + j * 16);
+            v[u] = *reinterpret_cast<const uint4 *>(g.a.qs + src_row(m) * g.a.K + (size_t)c0 * 256 + j * 16);
             dst[u] = m * L.lda + j * 16;
         }
 #pragma unroll
@@ -374,14 +393,14 @@ __device__ __forceinline__ void stage_activations(const MfmaArgs &g, uint8_t *sm
     float *dxs = reinterpret_cast<float *>(smem + L.off_dx);
     constexpr int ND = Cfg<QT>::kDx;
     const int nd = nsb * ND;  // scales per row in this range
-    for (int idx = tid; idx < g.M * nd; idx += kThreads) {
+    for (int idx = tid; idx < n_rows * nd; idx += kThreads) {
         const int m = idx / nd, j = idx - m * nd;
-        dxs[j * MT + m] = g.a.d[(size_t)m * (nb * ND) + c0 * ND + j];
+        dxs[j * MT + m] = g.a.d[src_row(m) * (nb * ND) + c0 * ND + j];
     }
     if constexpr (QT != kTypeQ8_0) {
-        for (int idx = tid; idx < g.M * nsb; idx += kThreads) {
+        for (int idx = tid; idx < n_rows * nsb; idx += kThreads) {
             const int m = idx / nsb, sb = idx - m * nsb;
-            const uint4 *src = reinterpret_cast<const uint4 *>(g.a.bsums + ((size_t)m * nb + c0 + sb) * 16);
+            const uint4 *src = reinterpret_cast<const uint4 *>(g.a.bsums + (src_row(m) * nb + c0 + sb) * 16);
             const uint4 b0 = src[0], b1 = src[1];
             const uint32_t w[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
             uint8_t *dst = smem + L.off_aux + (sb * MT + m) * Cfg<QT>::kAux;
@@ -407,33 +426,53 @@ __device__ __forceinline__ void stage_activations(const MfmaArgs &g, uint8_t *sm
     }
 }
 
-template <int QT, int NI, int W>
+constexpr int kDense = 0, kGrouped = 1, kGroupedSwiglu = 2;
+
+// MODE kDense: y[m][n] for the M rows of `a`.  kGrouped: the workgroup's expert e multiplies its
+// own pairs, y[pair][n].  kGroupedSwiglu: tensors 0 and 1 are gate and up of the same expert and
+// y[pair][n] = silu(gate . x) * (up . x).
+template <int QT, int NI, int W, int MODE>
 __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int MT = 8 * NI, NV = 4 * NI;
+    constexpr bool GROUPED = MODE != kDense, SWIGLU = MODE == kGroupedSwiglu;
+    constexpr int NT = SWIGLU ? 2 : 1;   // tensors streamed by one wave
     const Layout L = layout<QT, MT, W>(g.chunk_sb);
     const int lane = threadIdx.x & 63, wave = uniform(threadIdx.x >> 6);
     const int h = lane >> 5, nl = lane & 31;
 
-    // workgroup -> (tensor, K chunk, set of rw row groups)
-    int ti = 0;
-#pragma unroll
-    for (int i = 1; i < kMaxTargets; ++i)
-        if (i < g.n_targets && (int)blockIdx.x >= g.t[i].first_wg) ti = i;
+    // workgroup -> (tensor or expert, K chunk, set of rw row groups)
     WeightView w = g.t[0].w;
     float *y = g.t[0].y, *part = g.t[0].part;
-    int first = g.t[0].first_wg, nrs = g.t[0].n_rowsets;
+    int c = 0, rs, expert = 0, pair0 = 0, n_rows = g.M;
+    if constexpr (GROUPED) {
+        const int slot = (int)blockIdx.x / g.wgs_per_expert;   // the grid covers min(E, pairs) experts
+        rs = (int)blockIdx.x - slot * g.wgs_per_expert;
+        if (slot >= g.active[g.n_expert]) return;
+        expert = g.active[slot];
+        pair0 = g.offsets[expert];
+        n_rows = g.offsets[expert + 1] - pair0;
+        if (n_rows <= 0) return;
+    } else {
+        int ti = 0;
 #pragma unroll
-    for (int i = 1; i < kMaxTargets; ++i)
-        if (ti == i) {
-            w = g.t[i].w;
-            y = g.t[i].y;
-            part = g.t[i].part;
-            first = g.t[i].first_wg;
-            nrs = g.t[i].n_rowsets;
-        }
-    const int local = (int)blockIdx.x - first;
-    const int c = local / nrs, rs = local - c * nrs;
+        for (int i = 1; i < kMaxTargets; ++i)
+            if (i < g.n_targets && (int)blockIdx.x >= g.t[i].first_wg) ti = i;
+        int first = g.t[0].first_wg, nrs = g.t[0].n_rowsets;
+#pragma unroll
+        for (int i = 1; i < kMaxTargets; ++i)
+            if (ti == i) {
+                w = g.t[i].w;
+                y = g.t[i].y;
+                part = g.t[i].part;
+                first = g.t[i].first_wg;
+                nrs = g.t[i].n_rowsets;
+            }
+        const int local = (int)blockIdx.x - first;
+        c = local / nrs;
+        rs = local - c * nrs;
+    }
+    const int N = (int)w.N;
     const int nb = (int)(g.a.K >> 8);
     const int c0 = c * g.chunk_sb, nsb = min(g.chunk_sb, nb - c0);
 
@@ -442,67 +481,101 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
     const int row0 = (rs * g.rw + rgl) * 32;
     const int part_sb = (nsb + g.kw - 1) / g.kw;
     const int s0 = min(kp * part_sb, nsb), s1 = min(s0 + part_sb, nsb);  // range inside the staged chunk
-    const bool rows_ok = row0 < (int)w.N;
+    const bool rows_ok = row0 < N;
     const int steps = rows_ok ? s1 - s0 : 0;
-    const int last = c0 + (steps > 0 ? s1 - 1 : 0);   // loads past the range repeat its last super-block
+    const int items = NT * steps;                       // (tensor, super-block) pairs this wave streams
+    const int last_sb = c0 + (steps > 0 ? s1 - 1 : 0);  // loads past the range repeat its last super-block
 
     Stager<QT> sa, sb_;
-    sa.init(w, rows_ok ? row0 : 0, lane);
-    sb_ = sa;
-    sa.issue(min(c0 + s0, last));
-    sb_.issue(min(c0 + s0 + 1, last));
-
-    stage_activations<QT, MT, W * 64>(g, smem, L, c0, nsb);
-    __syncthreads();
-
+    {
+        const int64_t row = (int64_t)expert * N + (rows_ok ? row0 : 0);
+        sa.rebase(0, w, row);
+        sa.rebase(1, SWIGLU ? g.t[1].w : w, row);
+        sa.init(w, rows_ok ? min(31, N - 1 - row0) : 0, lane);
+        sb_.rebase(0, w, row);
+        sb_.rebase(1, SWIGLU ? g.t[1].w : w, row);
+        sb_.init(w, rows_ok ? min(31, N - 1 - row0) : 0, lane);
+    }
+    // item i -> tensor i / steps, super-block c0 + s0 + i % steps (clamped: harmless repeats past the end)
+    auto issue = [&](Stager<QT> &st, int i) {
+        const int t = SWIGLU && steps > 0 && i >= steps ? 1 : 0;
+        st.issue(t, min(c0 + s0 + i - t * steps, last_sb));
+    };
     uint8_t *region = smem + L.off_w + wave * Cfg<QT>::kRegion;
-    float out[NV];
-#pragma unroll
-    for (int v = 0; v < NV; ++v) out[v] = 0.f;
-    int s = 0;
-    for (; s + 1 < steps; s += 2) {
-        sa.park(region, lane);
-        sa.issue(min(c0 + s0 + s + 2, last));
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        compute<QT, NI>(region, smem, L, s0 + s, lane, out);
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        sb_.park(region, lane);
-        sb_.issue(min(c0 + s0 + s + 3, last));
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        compute<QT, NI>(region, smem, L, s0 + s + 1, lane, out);
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    }
-    if (s < steps) {
-        sa.park(region, lane);
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        compute<QT, NI>(region, smem, L, s0 + s, lane, out);
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    }
+    int *map = reinterpret_cast<int *>(smem + L.off_map);
 
-    // sum the K parts of a row group in a fixed order (through the waves' regions), then store
-    if (g.kw > 1) {
-        float *mine = reinterpret_cast<float *>(region);
-#pragma unroll
-        for (int v = 0; v < NV; ++v) mine[(8 * (v >> 2) + 4 * h + (v & 3)) * 32 + nl] = out[v];
+    // dense launches stage all (<= MT) rows at once; an expert with more than MT pairs takes several passes
+    for (int m0 = 0; m0 < (GROUPED ? n_rows : 1); m0 += MT) {
+        const int m_cnt = min(MT, n_rows - m0);
+        issue(sa, 0);
+        issue(sb_, 1);
+        if constexpr (GROUPED) {
+            if (m0 > 0) __syncthreads();   // the previous pass is done with the staged rows and the regions
+            if ((int)threadIdx.x < MT)
+                map[threadIdx.x] = (int)threadIdx.x < m_cnt ? g.order[pair0 + m0 + (int)threadIdx.x] : 0;
+            __syncthreads();
+        }
+        stage_activations<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
         __syncthreads();
-        if (kp == 0) {
+
+        float out[NT][NV];
 #pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                const uint8_t *src = region + ((8 * (v >> 2) + 4 * h + (v & 3)) * 32 + nl) * 4;
-                float t = *reinterpret_cast<const float *>(src);
-                for (int q = 1; q < g.kw; ++q) t += *reinterpret_cast<const float *>(src + q * Cfg<QT>::kRegion);
-                out[v] = t;
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int v = 0; v < NV; ++v) out[t][v] = 0.f;
+        auto consume = [&](int i) {
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            if (SWIGLU && i >= steps)
+                compute<QT, NI>(region, smem, L, s0 + i - steps, lane, out[NT - 1]);
+            else
+                compute<QT, NI>(region, smem, L, s0 + i, lane, out[0]);
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        };
+        int i = 0;
+        for (; i + 1 < items; i += 2) {
+            sa.park(region, lane);
+            issue(sa, i + 2);
+            consume(i);
+            sb_.park(region, lane);
+            issue(sb_, i + 3);
+            consume(i + 1);
+        }
+        if (i < items) {
+            sa.park(region, lane);
+            consume(i);
+        }
+
+        // sum the K parts of a row group in a fixed order (through the waves' regions), then store
+        if (g.kw > 1) {
+            float *mine = reinterpret_cast<float *>(region);
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int v = 0; v < NV; ++v)
+                    mine[t * (MT * 32) + (8 * (v >> 2) + 4 * h + (v & 3)) * 32 + nl] = out[t][v];
+            __syncthreads();
+            if (kp == 0) {
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) {
+                        const uint8_t *src = region + (t * (MT * 32) + (8 * (v >> 2) + 4 * h + (v & 3)) * 32 + nl) * 4;
+                        float acc = *reinterpret_cast<const float *>(src);
+                        for (int q = 1; q < g.kw; ++q) acc += *reinterpret_cast<const float *>(src + q * Cfg<QT>::kRegion);
+                        out[t][v] = acc;
+                    }
             }
         }
-    }
-    if (kp == 0 && rows_ok) {
-        const int N = (int)w.N;
-        float *dst = g.n_chunks == 1 ? y : part + (size_t)c * g.M * N;
-        const int n = row0 + nl;
+        if (kp == 0 && rows_ok) {
+            float *dst = GROUPED || g.n_chunks == 1 ? y : part + (size_t)c * g.M * N;
+            const int n = row0 + nl;
 #pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int m = 8 * (v >> 2) + 4 * h + (v & 3);
-            if (m < g.M && n < N) dst[(size_t)m * N + n] = out[v];
+            for (int v = 0; v < NV; ++v) {
+                const int m = 8 * (v >> 2) + 4 * h + (v & 3);
+                float r = out[0][v];
+                if constexpr (SWIGLU) r = (r / (1.0f + expf(-r))) * out[NT - 1][v];
+                if (m < m_cnt && n < N) dst[(size_t)(GROUPED ? map[m] : m0 + m) * N + n] = r;
+            }
         }
     }
 }
@@ -519,10 +592,10 @@ __global__ __launch_bounds__(256) void sum_chunks_kernel(const MfmaArgs g) {
     }
 }
 
-template <int QT, int NI, int W>
+template <int QT, int NI, int W, int MODE>
 hipError_t launch_one(const MfmaArgs &g, hipStream_t s) {
     const Layout L = layout<QT, 8 * NI, W>(g.chunk_sb);
-    auto kern = gemv_mfma_kernel<QT, NI, W>;
+    auto kern = gemv_mfma_kernel<QT, NI, W, MODE>;
     static int allowed = 0;
     if (L.total > allowed) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -553,12 +626,13 @@ int waves_per_wg(int type) {
 struct Split {
     int n_chunks, chunk_sb, kw;
 };
-Split plan(int64_t K, int64_t M, int64_t total_rg, int W) {
+constexpr int kMaxSb16 = 16;   // super-blocks of 16 staged rows that fit LDS beside the wave regions (~66 KB)
+Split plan(int64_t K, int64_t M, int64_t total_rg, int W, int min_wgs = 200) {
     const int nb = (int)(K / 256);
-    const int max_sb = M <= 8 ? 32 : 16;  // staged activations stay under ~66 KB of LDS
+    const int max_sb = M <= 8 ? 2 * kMaxSb16 : kMaxSb16;
     Split p;
     p.kw = 1;
-    while (p.kw < W && p.kw * 2 <= nb && total_rg * p.kw / W < 200) p.kw *= 2;
+    while (p.kw < W && p.kw * 2 <= nb && total_rg * p.kw / W < min_wgs) p.kw *= 2;
     const int rw = W / p.kw;
     const int64_t wgs1 = (total_rg + rw - 1) / rw;
     int nc = (nb + max_sb - 1) / max_sb;
@@ -568,12 +642,19 @@ Split plan(int64_t K, int64_t M, int64_t total_rg, int W) {
     return p;
 }
 
-template <int QT, int NI>
+template <int QT, int NI, int MODE>
 hipError_t launch_w(const MfmaArgs &g, int W, hipStream_t s) {
-    if (W == 4) return launch_one<QT, NI, 4>(g, s);
+    if (W == 4) return launch_one<QT, NI, 4, MODE>(g, s);
     if constexpr (QT == kTypeQ4_K)
-        if (W == 16) return launch_one<QT, NI, 16>(g, s);
-    return launch_one<QT, NI, 8>(g, s);
+        if (W == 16) return launch_one<QT, NI, 16, MODE>(g, s);
+    return launch_one<QT, NI, 8, MODE>(g, s);
+}
+
+template <int MODE>
+hipError_t launch_typed(const MfmaArgs &g, int type, bool small, int W, hipStream_t s) {
+    if (type == kTypeQ4_K) return small ? launch_w<kTypeQ4_K, 1, MODE>(g, W, s) : launch_w<kTypeQ4_K, 2, MODE>(g, W, s);
+    if (type == kTypeQ6_K) return small ? launch_w<kTypeQ6_K, 1, MODE>(g, W, s) : launch_w<kTypeQ6_K, 2, MODE>(g, W, s);
+    return small ? launch_w<kTypeQ8_0, 1, MODE>(g, W, s) : launch_w<kTypeQ8_0, 2, MODE>(g, W, s);
 }
 
 }  // namespace
@@ -581,6 +662,11 @@ hipError_t launch_w(const MfmaArgs &g, int W, hipStream_t s) {
 bool mfma_gemv_fits(int type, int64_t M, int64_t K) {
     (void)type;
     return M >= 1 && M <= 16 && K % 256 == 0;
+}
+
+bool mfma_grouped_fits(int type, int64_t K) {
+    (void)type;
+    return K % 256 == 0 && K / 256 <= kMaxSb16;
 }
 
 size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, int64_t total_rg) {
@@ -593,6 +679,7 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s)
     g.n_targets = args.n_targets;
     g.a = args.a;
     g.M = args.M;
+    g.x_div = 1;
     int64_t total_rg = 0;
     for (int i = 0; i < args.n_targets; ++i) total_rg += (args.t[i].w.N + 31) / 32;
     const int W = waves_per_wg(args.t[0].w.type);
@@ -615,11 +702,44 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s)
     }
     g.n_wgs = wg;
     if (g.n_chunks > 1 && !scratch) return hipErrorInvalidValue;
-    const int type = args.t[0].w.type;
-    const bool small = args.M <= 8;
-    if (type == kTypeQ4_K) return small ? launch_w<kTypeQ4_K, 1>(g, W, s) : launch_w<kTypeQ4_K, 2>(g, W, s);
-    if (type == kTypeQ6_K) return small ? launch_w<kTypeQ6_K, 1>(g, W, s) : launch_w<kTypeQ6_K, 2>(g, W, s);
-    return small ? launch_w<kTypeQ8_0, 1>(g, W, s) : launch_w<kTypeQ8_0, 2>(g, W, s);
+    return launch_typed<kDense>(g, args.t[0].w.type, args.M <= 8, W, s);
+}
+
+// Expert-grouped form: args.order / args.offsets list each expert's pairs; `swiglu` takes tensors 0 and 1
+// as gate and up.  n_pairs only steers the launch shape (how many experts can be busy at once).
+hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool swiglu, hipStream_t s) {
+    MfmaArgs g{};
+    g.n_targets = swiglu ? 2 : 1;
+    g.a = args.a;
+    g.M = 0;
+    g.order = args.order;
+    g.offsets = args.offsets;
+    g.active = args.active;
+    g.x_div = args.x_div;
+    const WeightView &w = args.t[0].w;
+    const int type = w.type;
+    const int W = waves_per_wg(type);
+    const int64_t rg_e = (w.N + 31) / 32;
+    const bool small = n_pairs <= 4 * w.E;   // few pairs an expert: 8 staged rows a pass are enough
+    Split p = plan(w.K, small ? 8 : 16, std::min<int64_t>(w.E, n_pairs) * rg_e, W);
+    const int nb = (int)(w.K / 256);
+    if (p.n_chunks != 1) {   // the grouped form keeps K inside one workgroup
+        p.n_chunks = 1;
+        p.chunk_sb = nb;
+    }
+    g.n_chunks = 1;
+    g.chunk_sb = p.chunk_sb;
+    g.kw = p.kw;
+    g.rw = W / p.kw;
+    for (int i = 0; i < g.n_targets; ++i) {
+        g.t[i].w = args.t[i].w;
+        g.t[i].y = args.t[i].y;
+    }
+    g.wgs_per_expert = (int)((rg_e + g.rw - 1) / g.rw);
+    g.n_expert = (int)w.E;
+    g.n_wgs = (int)(std::min<int64_t>(w.E, n_pairs) * g.wgs_per_expert);
+    if (swiglu) return launch_typed<kGroupedSwiglu>(g, type, small, W, s);
+    return launch_typed<kGrouped>(g, type, small, W, s);
 }
 
 }  // namespace qproj

@@ -235,6 +235,11 @@ bool use_decode_kernel(int type, int64_t M, int64_t K) {
     return !off && M <= 4 && decode_kernel_fits(type, pow2_ceil(M), K);
 }
 
+bool use_mfma_grouped(int type, int64_t K) {
+    static const bool off = getenv("QPROJ_NO_MFMA_GEMV") != nullptr;
+    return !off && mfma_grouped_fits(type, K);
+}
+
 bool use_mfma_kernel(int type, int64_t M, int64_t K) {
     static const bool off = getenv("QPROJ_NO_MFMA_GEMV") != nullptr;
     static const int min_m = getenv("QPROJ_MFMA_MIN_M") ? atoi(getenv("QPROJ_MFMA_MIN_M")) : 3;
@@ -593,13 +598,15 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     const ActPlanes p = act_planes(act_kind_for(act, w->type), rows, K);
     const size_t off_order = p.total;
     const size_t off_offsets = off_order + align_up((size_t)n_pairs * 4);
-    const size_t total = off_offsets + align_up((size_t)(w->E + 1) * 4);
+    const size_t off_active = off_offsets + align_up((size_t)(w->E + 1) * 4);
+    const size_t total = off_active + align_up((size_t)(w->E + 1) * 4);
     int rc = ensure_ws(ctx, total);
     if (rc) return rc;
     QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, rows, K));
     int32_t *order = reinterpret_cast<int32_t *>(ctx->ws + off_order);
     int32_t *offsets = reinterpret_cast<int32_t *>(ctx->ws + off_offsets);
-    QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, w->E, order, offsets, ctx->flag_dev, ctx->stream));
+    int32_t *active = reinterpret_cast<int32_t *>(ctx->ws + off_active);
+    QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, w->E, order, offsets, active, ctx->flag_dev, ctx->stream));
     GemvArgs g{};
     g.n_targets = 1;
     g.t[0].w = w->view;
@@ -607,8 +614,12 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     g.a = act_view(p, ctx->ws, K);
     g.order = order;
     g.offsets = offsets;
+    g.active = active;
     g.x_div = nb1 == 1 ? (int)n_used : 1;
-    QP_HIP(ctx, launch_gemv_q8act(g, grouped_mt(n_pairs, w->E), (int)w->E, ctx->stream));
+    if (use_mfma_grouped(w->type, K))
+        QP_HIP(ctx, launch_gemv_mfma_grouped(g, n_pairs, false, ctx->stream));
+    else
+        QP_HIP(ctx, launch_gemv_q8act(g, grouped_mt(n_pairs, w->E), (int)w->E, ctx->stream));
     return QPROJ_OK;
 }
 
@@ -635,6 +646,8 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     off += align_up((size_t)n_pairs * 4);
     const size_t off_offsets = off;
     off += align_up((size_t)(E + 1) * 4);
+    const size_t off_active = off;
+    off += align_up((size_t)(E + 1) * 4);
     const size_t off_h = off;
     off += align_up((size_t)(n_pairs * d_ff) * 4);
     const size_t off_hq = off;
@@ -646,12 +659,13 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     uint8_t *ws = ctx->ws;
     int32_t *order = reinterpret_cast<int32_t *>(ws + off_order);
     int32_t *offsets = reinterpret_cast<int32_t *>(ws + off_offsets);
+    int32_t *active = reinterpret_cast<int32_t *>(ws + off_active);
     float *h = reinterpret_cast<float *>(ws + off_h);
     float *e = reinterpret_cast<float *>(ws + off_e);
     const int mt = grouped_mt(n_pairs, E);
 
     QP_HIP(ctx, run_quantize(ctx, px, ws, x_dev, B, d_model));
-    QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, E, order, offsets, ctx->flag_dev, ctx->stream));
+    QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, E, order, offsets, active, ctx->flag_dev, ctx->stream));
     GemvArgs g{};
     g.n_targets = 2;
     g.t[0].w = gate->view;
@@ -661,8 +675,12 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     g.a = act_view(px, ws, d_model);
     g.order = order;
     g.offsets = offsets;
+    g.active = active;
     g.x_div = (int)n_used;
-    QP_HIP(ctx, launch_moe_swiglu_gemv(g, mt, (int)E, ctx->stream));
+    if (use_mfma_grouped(gate->type, d_model))
+        QP_HIP(ctx, launch_gemv_mfma_grouped(g, n_pairs, true, ctx->stream));
+    else
+        QP_HIP(ctx, launch_moe_swiglu_gemv(g, mt, (int)E, ctx->stream));
     QP_HIP(ctx, run_quantize(ctx, ph, ws + off_hq, h, n_pairs, d_ff));
     GemvArgs gd{};
     gd.n_targets = 1;
@@ -671,8 +689,12 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     gd.a = act_view(ph, ws + off_hq, d_ff);
     gd.order = order;
     gd.offsets = offsets;
+    gd.active = active;
     gd.x_div = 1;
-    QP_HIP(ctx, launch_gemv_q8act(gd, mt, (int)E, ctx->stream));
+    if (use_mfma_grouped(down->type, d_ff))
+        QP_HIP(ctx, launch_gemv_mfma_grouped(gd, n_pairs, false, ctx->stream));
+    else
+        QP_HIP(ctx, launch_gemv_q8act(gd, mt, (int)E, ctx->stream));
     QP_HIP(ctx, launch_moe_combine(e, weights_dev, B, n_used, d_model, y_dev, ctx->stream));
     return QPROJ_OK;
 }

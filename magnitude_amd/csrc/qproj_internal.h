@@ -65,6 +65,7 @@ struct GemvArgs {
     // expert-grouped mode (MUL_MAT_ID); null order = dense
     const int32_t *order;   // pair indices sorted by expert
     const int32_t *offsets; // [E+1] ranges into order
+    const int32_t *active;  // [E+1] experts that have pairs, ascending; [E] = how many
     int x_div;              // activation row of pair p is p / x_div
 };
 
@@ -84,9 +85,12 @@ hipError_t launch_gemv_decode(const GemvArgs &args, int mt, bool fuse_quantize, 
 bool mfma_gemv_fits(int type, int64_t M, int64_t K);
 size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, int64_t total_row_groups);
 hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s);
+// expert-grouped form (args.order / args.offsets); K / 256 must not exceed 16 (mfma_grouped_fits)
+bool mfma_grouped_fits(int type, int64_t K);
+hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool swiglu, hipStream_t s);
 hipError_t launch_gemv_f32(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
 hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_expert, int32_t *order,
-                            int32_t *offsets, int32_t *error_flag, hipStream_t s);
+                            int32_t *offsets, int32_t *active, int32_t *error_flag, hipStream_t s);
 hipError_t launch_moe_swiglu_gemv(const GemvArgs &gate_up, int mt, int n_experts_grid, hipStream_t s);
 hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, int64_t n_used, int64_t N,
                               float *y, hipStream_t s);

@@ -292,10 +292,11 @@ class Context:
         return y
 
     def moe_ffn(self, gate: Weight, up: Weight, down: Weight, x: torch.Tensor, ids: torch.Tensor,
-                weights: torch.Tensor, act: int = ACT_GGML, sync: bool = True) -> torch.Tensor:
+                weights: torch.Tensor, act: int = ACT_GGML, out: torch.Tensor = None,
+                sync: bool = True) -> torch.Tensor:
         """y[b] = sum_j weights[b, j] * down_e(silu(gate_e x_b) * up_e x_b), e = ids[b, j]."""
         b, n_used = ids.shape
-        y = torch.empty((b, gate.K), dtype=torch.float32, device=x.device)
+        y = out if out is not None else torch.empty((b, gate.K), dtype=torch.float32, device=x.device)
         if sync:
             torch.cuda.current_stream().synchronize()
         self._check(self.lib.qproj_moe_ffn(self.handle, gate.handle, up.handle, down.handle,

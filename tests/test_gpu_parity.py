@@ -347,7 +347,7 @@ def test_moe_ffn_matches_oracle(ctx, orc, moe, B):
         ws = [ctx.upload(Q4_K, d_model, d_ff, moe["gate"][e]) for e in ids[0]]
         gsep = torch.cat([ctx.mul_mat(wv, dev(x), ACT_GGML) for wv in ws]).cpu().numpy()
         gid = ctx.mul_mat_id(g, dev(x[:, None, :]), dev(ids), ACT_GGML).cpu().numpy()[0]
-        assert np.array_equal(gsep, gid)
+        close(gsep, gid, 2e-5)   # decode kernel vs grouped matrix-core kernel: same integer dots, other fp32 order
 
 
 # ---------------------------------------------------------------- full benchmark sizes
