@@ -335,6 +335,36 @@ def main():
         out["prefill"] = {"act_format": "per-32 int8 + fp32 scale", "mfma": "v_mfma_i32_32x32x32_i8",
                           "headline_tops": head["gemm_tops"], "headline_frac_int8_peak": head["frac_int8_peak"],
                           "peak_tops": INT8_PEAK_TOPS, "shapes": res}
+        # the same shapes in the ggml activation format (Q8_K, one scale per 256): the reference's own arithmetic
+        resg = []
+        for (k, n) in ((4096, 14336), (14336, 4096), (4096, 4096)):
+            blocks = synth.random_weight(Q4_K, n, k, seed=77 + n, device=dev)
+            w = ctx.upload_from_device(Q4_K, k, n, blocks)
+            del blocks
+            for m in (512, 2048, 4096):
+                x = torch.randn((m, k), generator=g, device=dev)
+                yb = torch.empty((m, n), device=dev)
+                qb = torch.empty(int(lib.qproj_act_bytes(ACT_GGML, Q4_K, m, k)), dtype=torch.uint8, device=dev)
+                torch.cuda.synchronize()
+                fq = lambda: ctx.quantize_activations_raw(x, ACT_GGML, Q4_K, out=qb, sync=False)
+                fg = lambda: ctx.mul_mat_quantized([w], qb, ACT_GGML, m, [yb], sync=False)
+                fq(); fg(); ctx.sync()
+                it = 5 if m * n * k > 1e11 else 10
+                tq = timer.time_ms(fq, it)
+                tg = timer.time_ms(fg, it)
+                ops = 2.0 * m * n * k
+                resg.append({"M": m, "K": k, "N": n, "gemm_ms": tg, "quantize_ms": tq,
+                             "gemm_tops": ops / (tg * 1e-3) / 1e12,
+                             "frac_int8_peak": ops / (tg * 1e-3) / 1e12 / INT8_PEAK_TOPS})
+                log(f"[bench] prefill(ggml acts) M={m} K={k} N={n}: gemm {tg:.3f} ms = {resg[-1]['gemm_tops']:.1f} TOPS "
+                    f"({100 * resg[-1]['frac_int8_peak']:.1f}% of int8 peak), quantize {tq:.3f} ms")
+                del x, yb, qb
+            w.free()
+        headg = [r for r in resg if (r["M"], r["K"], r["N"]) == (4096, 4096, 14336)][0]
+        out["prefill_ggml_acts"] = {"act_format": "ggml Q8_K (int8 + fp32 scale per 256, block sums)",
+                                    "mfma": "2 x v_mfma_i32_32x32x32_i8 per sub-block (scale split in base 8)",
+                                    "headline_tops": headg["gemm_tops"], "headline_frac_int8_peak": headg["frac_int8_peak"],
+                                    "shapes": resg}
 
     # ------------------------------------------------------------------ MoE leg (config 5)
     if "moe" in legs:

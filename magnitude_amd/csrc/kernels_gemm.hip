@@ -247,6 +247,240 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// ggml activation format (Q8_K: one scale per 256) x Q4_K on the int8 matrix cores.
+//
+// With a single activation scale per super-block the integer sums of its eight sub-blocks may be
+// added before anything turns into floating point; only the 6-bit sub-block scale sc stands in the
+// way, and sc*q (up to 945) does not fit an int8 operand.  Written in base 8, sc = 8*sc_hi + sc_lo,
+// both products sc_lo*q and sc_hi*q stay below 106: the kernel keeps TWO int8 weight tiles in LDS
+// and runs two accumulation chains over the whole super-block entirely inside the matrix cores,
+//     I_lo = sum_k (sc_lo*q) * a,   I_hi = sum_k (sc_hi*q) * a,   sum_k sc*q*a = 8*I_hi + I_lo,
+// so the vector ALU only works once per 256 weights (shift-add, int->float, one fma with dx*d).
+// Twice the matrix instructions of the per-32 kernel, a sixth of its vector instructions.
+//
+// Tile 128 tokens x 128 weight rows, 8 waves of 32x64, K-steps of 64 (one 32-byte nibble group =
+// two sub-blocks), double-buffered, two workgroups per CU.  The min term is the same small fp16
+// product as above, fed with dx*bsum.
+constexpr int QBK = 64;
+constexpr int QLD = QBK + 16;   // LDS row stride in bytes
+
+struct Q8kStage {
+    int8_t a[BM * QLD];       // activations [m][k]
+    int8_t b_lo[BN * QLD];    // (sc & 7) * q   [n][k]
+    int8_t b_hi[BN * QLD];    // (sc >> 3) * q  [n][k]
+};
+struct Q8kSmem {
+    Q8kStage st[2];
+    float dx[2][BM];          // activation scale of the super-block, by super-block parity
+    float dn[2][BN];          // weight d of the super-block
+};
+
+typedef unsigned short v2us __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_mul_u16(uint32_t x, uint32_t s2) {
+    return __builtin_bit_cast(uint32_t, __builtin_bit_cast(v2us, x) * __builtin_bit_cast(v2us, s2));
+}
+
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const WeightView w, const ActView a, int64_t M,
+                                                                     float *__restrict__ y) {
+    extern __shared__ __align__(16) uint8_t smem_raw[];
+    Q8kSmem &sm = *reinterpret_cast<Q8kSmem *>(smem_raw);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;  // 4 x 2 waves
+    const int64_t n0 = (int64_t)blockIdx.x * BN, m0 = (int64_t)blockIdx.y * BM;
+    const int64_t N = w.N, K = w.K, nb = w.nb;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    int64_t ncol[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        int64_t n = n0 + wn * 64 + j * 32 + l32;
+        ncol[j] = n < N ? n : N - 1;
+    }
+
+    v16f acc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+    // ---------------------------------------------------------------- min term on the fp16 cores
+    {
+        const int64_t n_steps = (nb + 1) / 2;  // two super-blocks (16 sub-blocks) per product
+        for (int64_t s = 0; s < n_steps; ++s) {
+            v8h ah, al, bh[2], bl[2];
+            {
+                int64_t m = m0 + wm * 32 + l32;
+                int64_t sb = s * 2 + lh;
+                const bool live = m < M && sb < nb;
+                if (m >= M) m = M - 1;
+                if (sb >= nb) sb = nb - 1;
+                const float dx = a.d[m * nb + sb];
+                const uint4 *bp = reinterpret_cast<const uint4 *>(a.bsums + (m * nb + sb) * 16);
+                const uint4 b0 = bp[0], b1 = bp[1];
+                const uint32_t bw[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const int bs = (int)(int16_t)(bw[t] & 0xffff) + (int)(int16_t)(bw[t] >> 16);
+                    _Float16 h, l;
+                    split_h(live ? dx * (float)bs * kMinPrescale : 0.f, h, l);
+                    ah[t] = h;
+                    al[t] = l;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                int64_t sb = s * 2 + lh;
+                const bool live = sb < nb;
+                if (!live) sb = nb - 1;
+                const uint4 hd = *reinterpret_cast<const uint4 *>(w.q4k + (ncol[j] * nb + sb) * 144);
+                const ScalesK4 sc = unpack_scales_k4(hd.y, hd.z, hd.w);
+                const float dmin = live ? h2f(hd.x >> 16) : 0.f;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    _Float16 h, l;
+                    split_h(-(dmin * (float)min_k4(sc, t)), h, l);
+                    bh[j][t] = h;
+                    bl[j][t] = l;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j], acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[j], acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[j], acc[j], 0, 0, 0);
+            }
+        }
+        const float inv = 1.0f / kMinPrescale;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][v] *= inv;
+    }
+
+    // ---------------------------------------------------------------- main loop
+    // Global loads run THREE K-steps ahead of the arithmetic (a K-step is only eight matrix
+    // instructions per wave, far shorter than a trip to memory): four register sets, one per
+    // K-step of a super-block, so every index below is a compile-time constant.
+    struct Regs {
+        v4i act;
+        uint32_t wq0, wq1;
+    } regs[4];
+    v4i hdr = {0, 0, 0, 0};
+    float dx_next = 0.f;
+    const int wrow = tid >> 2, wpart = tid & 3;   // weight staging: row, 8-byte slice of the 32-byte group
+    int64_t wn_row = n0 + wrow;
+    if (wn_row >= N) wn_row = N - 1;
+    const uint8_t *wbase = w.q4k + wn_row * nb * 144;
+    const int arow = tid >> 2, aseg = tid & 3;    // activation staging: row, 16-byte segment of the 64
+    const int8_t *abase = a.qs + (m0 + arow < M ? m0 + arow : M - 1) * K + 16 * aseg;
+    const float *dxbase = a.d + (m0 + tid < M ? m0 + tid : M - 1) * nb;   // threads 0..127
+
+    auto load_stage = [&](Regs &r, int64_t sb, int g) {   // K-step g (0..3) of super-block sb
+        const uint8_t *blk = wbase + sb * 144;
+        const uint2 q2 = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * g + 8 * wpart);
+        r.wq0 = q2.x;
+        r.wq1 = q2.y;
+        if (g == 0) {
+            hdr = *reinterpret_cast<const v4i *>(blk);
+            if (tid < BM) dx_next = dxbase[sb];
+        }
+        r.act = *reinterpret_cast<const v4i *>(abase + sb * 256 + 64 * g);
+    };
+    ScalesK4 cur_sc{};
+    auto store_stage = [&](const Regs &r, Q8kStage &st, int64_t sb, int g) {
+        if (g == 0) {
+            cur_sc = unpack_scales_k4((uint32_t)hdr[1], (uint32_t)hdr[2], (uint32_t)hdr[3]);
+            if (wpart == 0) sm.dn[sb & 1][wrow] = h2f((uint32_t)hdr[0]);
+            if (tid < BM) sm.dx[sb & 1][tid] = dx_next;
+        }
+        const uint32_t s0 = scale_k4(cur_sc, 2 * g), s1 = scale_k4(cur_sc, 2 * g + 1);   // sub-blocks 2g (low nibbles), 2g+1
+        const uint32_t s0l = (s0 & 7) * 0x00010001u, s0h = (s0 >> 3) * 0x00010001u;
+        const uint32_t s1l = (s1 & 7) * 0x00010001u, s1h = (s1 >> 3) * 0x00010001u;
+        const uint32_t x0 = r.wq0 & 0x0f0f0f0fu, x1 = r.wq1 & 0x0f0f0f0fu;
+        const uint32_t z0 = (r.wq0 >> 4) & 0x0f0f0f0fu, z1 = (r.wq1 >> 4) & 0x0f0f0f0fu;
+        const int o = wrow * QLD + 8 * wpart;
+        *reinterpret_cast<uint2 *>(st.b_lo + o) = make_uint2(pk_mul_u16(x0, s0l), pk_mul_u16(x1, s0l));
+        *reinterpret_cast<uint2 *>(st.b_hi + o) = make_uint2(pk_mul_u16(x0, s0h), pk_mul_u16(x1, s0h));
+        *reinterpret_cast<uint2 *>(st.b_lo + o + 32) = make_uint2(pk_mul_u16(z0, s1l), pk_mul_u16(z1, s1l));
+        *reinterpret_cast<uint2 *>(st.b_hi + o + 32) = make_uint2(pk_mul_u16(z0, s1h), pk_mul_u16(z1, s1h));
+        *reinterpret_cast<v4i *>(st.a + arow * QLD + 16 * aseg) = r.act;
+    };
+
+    load_stage(regs[0], 0, 0);
+    load_stage(regs[1], 0, 1);
+    load_stage(regs[2], 0, 2);
+    store_stage(regs[0], sm.st[0], 0, 0);
+    __syncthreads();
+
+    const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    v16i ilo[2], ihi[2];
+    // one K-step: two sub-blocks, for each the low and the high chain of both column tiles
+    auto kstep = [&](const Q8kStage &st, bool first) {
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            const v4i af = *reinterpret_cast<const v4i *>(st.a + (wm * 32 + l32) * QLD + blk * 32 + 16 * lh);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int o = (wn * 64 + j * 32 + l32) * QLD + blk * 32 + 16 * lh;
+                const v4i bl = *reinterpret_cast<const v4i *>(st.b_lo + o);
+                const v4i bh = *reinterpret_cast<const v4i *>(st.b_hi + o);
+                if (first && blk == 0) {
+                    ilo[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bl, zi, 0, 0, 0);
+                    ihi[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bh, zi, 0, 0, 0);
+                } else {
+                    ilo[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bl, ilo[j], 0, 0, 0);
+                    ihi[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bh, ihi[j], 0, 0, 0);
+                }
+            }
+        }
+    };
+    for (int64_t sb = 0; sb < nb; ++sb) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            {   // K-step three ahead
+                // (past the end the last super-block is fetched again: an unconditional load keeps the
+                // count of loads in flight known, so the wait before the LDS store can leave them flying)
+                const int64_t sb3 = g == 0 ? sb : (sb + 1 < nb ? sb + 1 : nb - 1);
+                load_stage(regs[(g + 3) & 3], sb3, (g + 3) & 3);
+            }
+            kstep(sm.st[g & 1], g == 0);
+            if (g == 3) {   // the super-block is complete: 8*I_hi + I_lo, scaled by dx*d, joins the fp32 sum
+                const float *dxs = sm.dx[sb & 1];
+                float dxv[16];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float4 d4 = *reinterpret_cast<const float4 *>(dxs + wm * 32 + 8 * i + 4 * lh);
+                    dxv[4 * i] = d4.x; dxv[4 * i + 1] = d4.y; dxv[4 * i + 2] = d4.z; dxv[4 * i + 3] = d4.w;
+                }
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const float dn = sm.dn[sb & 1][wn * 64 + j * 32 + l32];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        acc[j][v] = fmaf((float)((ihi[j][v] << 3) + ilo[j][v]), dxv[v] * dn, acc[j][v]);
+                }
+            }
+            {   // next K-step into the other LDS stage
+                const int64_t sb1 = g < 3 ? sb : sb + 1;
+                if (sb1 < nb) store_stage(regs[(g + 1) & 3], sm.st[(g + 1) & 1], sb1, (g + 1) & 3);
+            }
+            __syncthreads();
+        }
+    }
+
+    // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int64_t n = n0 + wn * 64 + j * 32 + l32;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int64_t m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (m < M && n < N) y[m * N + n] = acc[j][v];
+        }
+    }
+}
+
 }  // namespace
 
 hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
@@ -256,6 +490,17 @@ hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, f
     if (attr != hipSuccess) return attr;
     const dim3 grid((unsigned)((w.N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
     hipLaunchKernelGGL(gemm_q4k_q8x32_kernel, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y);
+    return hipGetLastError();
+}
+
+// ggml-format activations (Q8_K planes in `a`), Q4_K weights, any M
+hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
+    if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || M <= 0) return hipErrorInvalidValue;
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Q8kSmem));
+    if (attr != hipSuccess) return attr;
+    const dim3 grid((unsigned)((w.N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
+    hipLaunchKernelGGL(gemm_q4k_q8k_kernel, grid, dim3(kGemmThreads), sizeof(Q8kSmem), s, w, a, M, y);
     return hipGetLastError();
 }
 

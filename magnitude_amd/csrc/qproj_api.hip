@@ -261,6 +261,11 @@ size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
 
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
                     float *const *y, float *scratch) {
+    static const int gemm_min_m = getenv("QPROJ_GEMM_MIN_M") ? atoi(getenv("QPROJ_GEMM_MIN_M")) : 48;
+    if (w[0]->type == kTypeQ4_K && M >= gemm_min_m) {   // prefill-sized batches: tiled product, weights reused across tokens
+        for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8k(w[i]->view, a, M, y[i], ctx->stream));
+        return QPROJ_OK;
+    }
     if (use_mfma_kernel(w[0]->type, M, w[0]->K)) {
         for (int64_t m0 = 0; m0 < M; m0 += 16) {
             const int64_t mc = std::min<int64_t>(16, M - m0);

@@ -95,5 +95,7 @@ hipError_t launch_moe_swiglu_gemv(const GemvArgs &gate_up, int mt, int n_experts
 hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, int64_t n_used, int64_t N,
                               float *y, hipStream_t s);
 hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
+// Q4_K weights x ggml Q8_K activations (`a`), large M
+hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
 
 }  // namespace qproj

@@ -196,6 +196,26 @@ def test_mul_mat_ggml_mode_matches_oracle(ctx, orc, qtype, m):
         w.free()
 
 
+@pytest.mark.parametrize("m,k,n", [(48, 4096, 256), (130, 768, 203), (200, 14336, 128), (333, 256, 40)])
+def test_mul_mat_ggml_mode_prefill_sized_batches(ctx, orc, m, k, n):
+    """Large M in the ggml activation format: the tiled matrix-core kernel (two int8 chains per
+    super-block) against the oracle's Q4_K x Q8_K integer arithmetic, ragged M and N included."""
+    from magnitude_amd import ACT_GGML
+    blocks = make_weight(orc, Q4_K, n, k, seed=1500 + k + n)
+    rng = np.random.default_rng(m + k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[:, rng.integers(0, k, 8)] *= 30.0          # outlier channels, as transformer activations have
+    w = ctx.upload(Q4_K, k, n, blocks)
+    got = ctx.mul_mat(w, dev(x), ACT_GGML).cpu().numpy()
+    want = orc.mul_mat(Q4_K, blocks, k, x, orc.ACT_GGML)
+    close(got, want, 2e-5)
+    gate(got, want)
+    # a row of the big batch is the small-batch kernel's row up to fp32 summation order
+    few = ctx.mul_mat(w, dev(x[:5]), ACT_GGML).cpu().numpy()
+    close(got[:5], few, 2e-5)
+    w.free()
+
+
 @pytest.mark.parametrize("qtype", TYPES)
 @pytest.mark.parametrize("m", [1, 3, 4, 6])
 def test_mul_mat_f32_mode_matches_fp64_dot(ctx, orc, qtype, m):
@@ -363,7 +383,7 @@ def test_full_size_against_device_fp64_of_proven_parts(ctx, qtype, k, n):
     w = ctx.upload_from_device(qtype, k, n, blocks)
     wd = ctx.dequantize(w).double()
     g = torch.Generator(device="cuda").manual_seed(1)
-    for m in (1, 4, 16):
+    for m in (1, 4, 16, 192):
         x = torch.randn((m, k), generator=g, device="cuda", dtype=torch.float32)
         y = ctx.mul_mat(w, x, ACT_GGML)
         a = ctx.quantize_activations(x, ACT_GGML, qtype)
