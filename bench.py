@@ -65,6 +65,20 @@ class Timer:
         b.synchronize()
         return a.elapsed_time(b) / iters
 
+    def samples_ms(self, fn, n):
+        """n separately timed calls (an event pair around each), for records that keep raw samples"""
+        t = self.torch
+        evs = []
+        with t.cuda.stream(self.stream):
+            for _ in range(n):
+                a, b = t.cuda.Event(enable_timing=True), t.cuda.Event(enable_timing=True)
+                a.record(self.stream)
+                fn()
+                b.record(self.stream)
+                evs.append((a, b))
+        evs[-1][1].synchronize()
+        return [a.elapsed_time(b) for a, b in evs]
+
 
 def capture(torch, stream, fn):
     """Captures fn() (launches on `stream` only) into a HIP graph; returns replay() or None."""
@@ -107,6 +121,8 @@ def main():
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (counter calibration for rocprofv3 --pmc)")
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
+    ap.add_argument("--evidence-sql", default=None,
+                    help="also write the per-kernel rows as test-backend-ops SQL INSERT lines to this file")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no sharding, no collectives); use --gpus 1", file=sys.stderr)
@@ -115,7 +131,7 @@ def main():
 
     import torch
 
-    from magnitude_amd import ACT_GGML, ACT_Q8X32, Context, synth
+    from magnitude_amd import ACT_GGML, ACT_Q8X32, Context, evidence, synth
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     dev = torch.device("cuda:0")
@@ -211,6 +227,7 @@ def main():
             f"{1.0 / dt:.0f} tok/s (projections only)")
 
     # ------------------------------------------------------------------ roofline leg: dominant kernel
+    ev_rows, ev_meas, ev_cal = [], [], []
     if "roofline" in legs:
         reps = max(5, args.steps)
         per = {}
@@ -225,13 +242,21 @@ def main():
             for _ in range(3):
                 run()
             torch.cuda.synchronize()
-            ms = timer.time_ms(run, reps) / L
+            samples = [s / L * 1e3 for s in timer.samples_ms(run, reps)]   # us per launch, one sample per replay
+            ms = sum(samples) / len(samples) * 1e-3
             nbytes = sum(gemv_bytes(lw_t, n, k) for nm, lw_t, n, k in LAYER_TENSORS if nm in grp[1]) \
                 - (len(grp[1]) - 1) * grp[2].numel() * 4      # the shared activation row is read once
             per[grp[0]] = {"us_per_launch": ms * 1e3, "bytes_per_launch": nbytes,
                            "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
             log(f"[bench] kernel {grp[0]:8s}: {ms * 1e3:7.2f} us  {per[grp[0]]['GBps']:6.0f} GB/s "
                 f"({100 * per[grp[0]]['frac_hbm_peak']:.1f}% of peak)")
+            qt0, rows, kk = [(t, sum(n for nm, _, n, _ in LAYER_TENSORS if nm in grp[1]), k)
+                             for nm, t, n, k in LAYER_TENSORS if nm == grp[1][0]][0]
+            ev_rows.append(evidence.backend_ops_row("MUL_MAT", evidence.mul_mat_params(qt0, rows, 1, kk), samples,
+                                                    flops=2.0 * rows * kk, bytes_moved=nbytes,
+                                                    memory_kb=nbytes // 1024, device=props.name))
+            ev_meas.append(evidence.measurement(f"decode.{grp[0]}.launch", "us", samples))
+            ev_cal.append(evidence.calibration_metric(qt0, False, nbytes, samples, launch_us=2.0))
         dom = per["gate_up"]
         out["roofline"] = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                            "frac": dom["frac_hbm_peak"], "traffic": measured_traffic(),
@@ -321,8 +346,14 @@ def main():
                 fq(); fg(); ctx.sync()
                 it = 5 if m * n * k > 1e11 else 10
                 tq = timer.time_ms(fq, it)
-                tg = timer.time_ms(fg, it)
+                sg = timer.samples_ms(fg, it)
+                tg = sum(sg) / len(sg)
                 ops = 2.0 * m * n * k
+                ev_rows.append(evidence.backend_ops_row("MUL_MAT", evidence.mul_mat_params(Q4_K, n, m, k) + ",act=q8x32",
+                                                        [s * 1e3 for s in sg], flops=ops,
+                                                        bytes_moved=gguf_bytes(Q4_K, n, k) + m * k + m * n * 4,
+                                                        memory_kb=(gguf_bytes(Q4_K, n, k) + m * n * 4) // 1024,
+                                                        device=props.name))
                 res.append({"M": m, "K": k, "N": n, "gemm_ms": tg, "quantize_ms": tq,
                             "gemm_tops": ops / (tg * 1e-3) / 1e12,
                             "end_to_end_tops": ops / ((tg + tq) * 1e-3) / 1e12,
@@ -351,8 +382,14 @@ def main():
                 fq(); fg(); ctx.sync()
                 it = 5 if m * n * k > 1e11 else 10
                 tq = timer.time_ms(fq, it)
-                tg = timer.time_ms(fg, it)
+                sg = timer.samples_ms(fg, it)
+                tg = sum(sg) / len(sg)
                 ops = 2.0 * m * n * k
+                ev_rows.append(evidence.backend_ops_row("MUL_MAT", evidence.mul_mat_params(Q4_K, n, m, k),
+                                                        [s * 1e3 for s in sg], flops=ops,
+                                                        bytes_moved=gguf_bytes(Q4_K, n, k) + m * k * 4 + m * n * 4,
+                                                        memory_kb=(gguf_bytes(Q4_K, n, k) + m * n * 4) // 1024,
+                                                        device=props.name))
                 resg.append({"M": m, "K": k, "N": n, "gemm_ms": tg, "quantize_ms": tq,
                              "gemm_tops": ops / (tg * 1e-3) / 1e12,
                              "frac_int8_peak": ops / (tg * 1e-3) / 1e12 / INT8_PEAK_TOPS})
@@ -387,8 +424,14 @@ def main():
             f(); ctx.sync()
             run = (None if args.no_graph else capture(torch, stream, f)) or f
             run(); torch.cuda.synchronize()
-            ms = timer.time_ms(run, 20)
+            sm_ = timer.samples_ms(run, 20)
+            ms = sum(sm_) / len(sm_)
             byts = distinct * per_expert + B * dm * 4 * 2
+            ev_rows.append(evidence.backend_ops_row("MUL_MAT_ID", evidence.mul_mat_id_params(Q4_K, dff, dm, E, top, B) +
+                                                    ",fused=moe_ffn(gate,up,swiglu,down,combine)", [s * 1e3 for s in sm_],
+                                                    flops=2.0 * B * top * 3 * dm * dff, bytes_moved=byts,
+                                                    memory_kb=byts // 1024, device=props.name))
+            ev_cal.append(evidence.calibration_metric(Q4_K, True, byts, [s * 1e3 for s in sm_], launch_us=2.0))
             res.append({"B": B, "distinct_experts": distinct, "ms": ms, "GBps": byts / (ms * 1e-3) / 1e9,
                         "frac_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
             log(f"[bench] moe B={B}: {ms * 1e3:.1f} us, {distinct} experts, {res[-1]['GBps']:.0f} GB/s")
@@ -415,12 +458,22 @@ def main():
                     spent += orc.time_mul_mat(qt, blocks, k, xs[k], orc.ACT_GGML, threads, 1)
             passes += 1
         cpu_gbs = passes * nl * LAYER_BYTES / spent / 1e9
+        one = 0.0                                  # one thread, one layer: the scalar figure beside the threaded one
+        for qt, n, k, blocks in host[0]:
+            one += orc.time_mul_mat(qt, blocks, k, xs[k], orc.ACT_GGML, 1, 1)
         out["cpu_baseline"] = {"value": cpu_gbs, "unit": "GB/s", "cores": threads, "kind": "port",
                                "sample": f"{passes} passes over {nl} of the same layers (7 projections each, M=1, "
                                          f"ggml activation mode), {spent:.1f} s of OpenMP C on the host",
-                               "host_cpus": os.cpu_count()}
+                               "host_cpus": os.cpu_count(),
+                               "one_thread_GBps": LAYER_BYTES / one / 1e9}
         log(f"[bench] cpu baseline: {cpu_gbs:.2f} GB/s on {threads} threads")
 
+    if ev_rows:
+        # the reference's own record shapes (test-backend-ops rows, parity measurements, fit calibration)
+        out["evidence"] = {"backend_ops": ev_rows, "measurements": ev_meas, "calibration": ev_cal}
+        if args.evidence_sql:
+            with open(args.evidence_sql, "w") as f:
+                f.write("\n".join(evidence.backend_ops_sql(r) for r in ev_rows) + "\n")
     print(json.dumps(out), flush=True)
     return 0
 
