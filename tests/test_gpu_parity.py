@@ -416,3 +416,38 @@ def test_full_size_prefill_gemm_against_device_fp64(ctx):
     ref = xq @ wd.T
     err = ((y.double() - ref).abs() / ref.abs().clamp(min=1.0)).max().item()
     assert err <= 5e-5, err
+
+
+# ---------------------------------------------------------------- GGUF file -> library
+
+def test_weights_read_from_a_gguf_file_give_the_same_products(ctx, orc, tmp_path):
+    """Tensors located by the GGUF reader and uploaded from the mapped file behave exactly like
+    the same blocks uploaded directly; an expert stack [K, N, E] keeps its expert-major rows."""
+    from magnitude_amd import ACT_GGML, gguf
+    k, n, E = 512, 96, 4
+    q4 = make_weight(orc, Q4_K, n, k, seed=8101)
+    q6 = make_weight(orc, Q6_K, n, k, seed=8102)
+    q8 = make_weight(orc, Q8_0, n, k, seed=8103)
+    ex = np.concatenate([make_weight(orc, Q4_K, n, k, seed=8110 + e).reshape(-1) for e in range(E)])
+    path = str(tmp_path / "model.gguf")
+    gguf.write(path, [("blk.0.attn_q.weight", (k, n), Q4_K, q4), ("blk.0.ffn_down.weight", (k, n), Q6_K, q6),
+                      ("output.weight", (k, n), Q8_0, q8), ("blk.0.ffn_up_exps.weight", (k, n, E), Q4_K, ex),
+                      ("blk.0.attn_norm.weight", (k,), 0, np.ones(k, np.float32))],
+               {"general.architecture": "llama", "general.file_type": 15})
+    x = dev(np.random.default_rng(3).standard_normal((3, k)).astype(np.float32))
+    with gguf.GgufFile(path) as g:
+        ws = g.upload_all(ctx)
+        assert set(ws) == {"blk.0.attn_q.weight", "blk.0.ffn_down.weight", "output.weight", "blk.0.ffn_up_exps.weight"}
+        with pytest.raises(gguf.GgufError):
+            g.upload(ctx, "blk.0.attn_norm.weight")
+    for name, qt, blk in (("blk.0.attn_q.weight", Q4_K, q4), ("blk.0.ffn_down.weight", Q6_K, q6), ("output.weight", Q8_0, q8)):
+        direct = ctx.upload(qt, k, n, blk)
+        assert torch.equal(ctx.mul_mat(ws[name], x, ACT_GGML), ctx.mul_mat(direct, x, ACT_GGML))
+        assert np.array_equal(ctx.download(ws[name]), np.asarray(blk).reshape(-1))
+    we = ws["blk.0.ffn_up_exps.weight"]
+    assert (we.K, we.N, we.E) == (k, n, E)
+    ids = dev(np.array([[2, 0]], dtype=np.int32))
+    got = ctx.mul_mat_id(we, x[:1, None, :].contiguous(), ids, ACT_GGML).cpu().numpy()[0]
+    for slot, e in enumerate((2, 0)):
+        one = ctx.upload(Q4_K, k, n, ex.reshape(E, -1)[e])
+        close(got[slot], ctx.mul_mat(one, x[:1], ACT_GGML).cpu().numpy()[0], 2e-5)
