@@ -319,6 +319,7 @@ __device__ __forceinline__ void compute(const uint8_t *region, const uint8_t *sm
 #pragma unroll
                     for (int v = 0; v < NV; ++v) isum[v] = __mul24(I[v], s) + isum[v];
                 }
+                __builtin_amdgcn_sched_barrier(0);   // keeps the four groups' operand loads from piling up in registers
             }
         // -32 * sum_j sc_j * bsum_j: block sums split as 64*hi + lo against the 16 scales
         const uint8_t *aux = smem + L.off_aux + (ks * MT + mrow) * 32;
