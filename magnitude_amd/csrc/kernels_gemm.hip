@@ -55,6 +55,22 @@ __device__ __forceinline__ void split_h(float v, _Float16 &hi, _Float16 &lo) {
     lo = (_Float16)(v - (float)hi);
 }
 
+// Workgroup -> tile.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its
+// own L2: every XCD gets one contiguous stretch of the tile order, and the order walks groups of 8
+// token tiles x all column tiles column by column, so the workgroups an XCD runs at the same time
+// share activation tiles AND weight tiles instead of streaming the whole weight matrix once per
+// row of tiles.
+__device__ __forceinline__ void tile_of_workgroup(int tiles_n, int tiles_m, int &tn, int &tm) {
+    constexpr int kXcds = 8, kGroupM = 8;
+    const int total = tiles_n * tiles_m, pid = (int)blockIdx.x;
+    const int x = pid % kXcds, base = total / kXcds, rem = total % kXcds;
+    const int q = x * base + min(x, rem) + pid / kXcds;
+    const int span = kGroupM * tiles_n, group = q / span, local = q - group * span;
+    const int first_m = group * kGroupM, gsz = min(tiles_m - first_m, kGroupM);
+    tm = first_m + local % gsz;
+    tn = local / gsz;
+}
+
 constexpr int kGemmThreads = 512;
 
 __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const WeightView w, const ActView a, int64_t M,
@@ -63,8 +79,10 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
     GemmSmem &sm = *reinterpret_cast<GemmSmem *>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;  // 4 x 2 waves
-    const int64_t n0 = (int64_t)blockIdx.x * BN, m0 = (int64_t)blockIdx.y * BM;
     const int64_t N = w.N, K = w.K;
+    int tile_n, tile_m;
+    tile_of_workgroup((int)((N + BN - 1) / BN), (int)((M + BM - 1) / BM), tile_n, tile_m);
+    const int64_t n0 = (int64_t)tile_n * BN, m0 = (int64_t)tile_m * BM;
     const int64_t kb32 = K / 32;
     const int l32 = lane & 31, lh = lane >> 5;
 
@@ -287,8 +305,10 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const Wei
     Q8kSmem &sm = *reinterpret_cast<Q8kSmem *>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;  // 4 x 2 waves
-    const int64_t n0 = (int64_t)blockIdx.x * BN, m0 = (int64_t)blockIdx.y * BM;
     const int64_t N = w.N, K = w.K, nb = w.nb;
+    int tile_n, tile_m;
+    tile_of_workgroup((int)((N + BN - 1) / BN), (int)((M + BM - 1) / BM), tile_n, tile_m);
+    const int64_t n0 = (int64_t)tile_n * BN, m0 = (int64_t)tile_m * BM;
     const int l32 = lane & 31, lh = lane >> 5;
 
     int64_t ncol[2];
@@ -488,7 +508,7 @@ hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, f
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8x32_kernel),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem));
     if (attr != hipSuccess) return attr;
-    const dim3 grid((unsigned)((w.N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
+    const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + BM - 1) / BM)));
     hipLaunchKernelGGL(gemm_q4k_q8x32_kernel, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y);
     return hipGetLastError();
 }
@@ -499,7 +519,7 @@ hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, flo
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_kernel),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Q8kSmem));
     if (attr != hipSuccess) return attr;
-    const dim3 grid((unsigned)((w.N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
+    const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + BM - 1) / BM)));
     hipLaunchKernelGGL(gemm_q4k_q8k_kernel, grid, dim3(kGemmThreads), sizeof(Q8kSmem), s, w, a, M, y);
     return hipGetLastError();
 }
