@@ -2,7 +2,7 @@
 """Benchmark of the quantized projection path on one MI355X.
 
 A "step" is one decoded token's pass over the projections of a 32-layer 8B-class dense model in
-Q4_K_M (config 2 of BASELINE.json, repeated over 32 DISTINCT layers = 4.41 GB of weights so that
+Q4_K_M (the 8B decode configuration, repeated over 32 DISTINCT layers = 4.41 GB of weights so that
 every step streams from HBM, not from the 256 MB Infinity Cache): per layer q/k/v (one launch),
 o, gate/up (one launch) in Q4_K and down in Q6_K, each preceded by the activation quantizer, in
 the ggml activation mode (the reference CPU path's arithmetic).  `value` is algorithmic GGUF bytes
