@@ -277,7 +277,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
 // so the vector ALU only works once per 256 weights (shift-add, int->float, one fma with dx*d).
 // Twice the matrix instructions of the per-32 kernel, a sixth of its vector instructions.
 //
-// Tile 128 tokens x 128 weight rows, 8 waves of 32x64, K-steps of 64 (one 32-byte nibble group =
+// Tile 128 tokens x 128 weight rows, 8 waves of 64 tokens x 32 rows, K-steps of 64 (one 32-byte nibble group =
 // two sub-blocks), double-buffered, two workgroups per CU.  The min term is the same small fp16
 // product as above, fed with dx*bsum.
 constexpr int QBK = 64;
@@ -304,19 +304,14 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const Wei
     extern __shared__ __align__(16) uint8_t smem_raw[];
     Q8kSmem &sm = *reinterpret_cast<Q8kSmem *>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;  // 4 x 2 waves
+    const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 waves, each 64 tokens x 32 weight rows: one B fragment pair feeds two products
     const int64_t N = w.N, K = w.K, nb = w.nb;
     int tile_n, tile_m;
     tile_of_workgroup((int)((N + BN - 1) / BN), (int)((M + BM - 1) / BM), tile_n, tile_m);
     const int64_t n0 = (int64_t)tile_n * BN, m0 = (int64_t)tile_m * BM;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    int64_t ncol[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        int64_t n = n0 + wn * 64 + j * 32 + l32;
-        ncol[j] = n < N ? n : N - 1;
-    }
+    const int64_t ncol = n0 + wn * 32 + l32 < N ? n0 + wn * 32 + l32 : N - 1;
 
     v16f acc[2];
 #pragma unroll
@@ -328,9 +323,10 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const Wei
     {
         const int64_t n_steps = (nb + 1) / 2;  // two super-blocks (16 sub-blocks) per product
         for (int64_t s = 0; s < n_steps; ++s) {
-            v8h ah, al, bh[2], bl[2];
-            {
-                int64_t m = m0 + wm * 32 + l32;
+            v8h ah[2], al[2], bh, bl;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                int64_t m = m0 + wm * 64 + i * 32 + l32;
                 int64_t sb = s * 2 + lh;
                 const bool live = m < M && sb < nb;
                 if (m >= M) m = M - 1;
@@ -344,31 +340,30 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const Wei
                     const int bs = (int)(int16_t)(bw[t] & 0xffff) + (int)(int16_t)(bw[t] >> 16);
                     _Float16 h, l;
                     split_h(live ? dx * (float)bs * kMinPrescale : 0.f, h, l);
-                    ah[t] = h;
-                    al[t] = l;
+                    ah[i][t] = h;
+                    al[i][t] = l;
                 }
             }
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            {
                 int64_t sb = s * 2 + lh;
                 const bool live = sb < nb;
                 if (!live) sb = nb - 1;
-                const uint4 hd = *reinterpret_cast<const uint4 *>(w.q4k + (ncol[j] * nb + sb) * 144);
+                const uint4 hd = *reinterpret_cast<const uint4 *>(w.q4k + (ncol * nb + sb) * 144);
                 const ScalesK4 sc = unpack_scales_k4(hd.y, hd.z, hd.w);
                 const float dmin = live ? h2f(hd.x >> 16) : 0.f;
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
                     _Float16 h, l;
                     split_h(-(dmin * (float)min_k4(sc, t)), h, l);
-                    bh[j][t] = h;
-                    bl[j][t] = l;
+                    bh[t] = h;
+                    bl[t] = l;
                 }
             }
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j], acc[j], 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[j], acc[j], 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[j], acc[j], 0, 0, 0);
+            for (int i = 0; i < 2; ++i) {
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bh, acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bl, acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[i], bh, acc[i], 0, 0, 0);
             }
         }
         const float inv = 1.0f / kMinPrescale;
@@ -394,7 +389,9 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const Wei
     const uint8_t *wbase = w.q4k + wn_row * nb * 144;
     const int arow = tid >> 2, aseg = tid & 3;    // activation staging: row, 16-byte segment of the 64
     const int8_t *abase = a.qs + (m0 + arow < M ? m0 + arow : M - 1) * K + 16 * aseg;
-    const float *dxbase = a.d + (m0 + tid < M ? m0 + tid : M - 1) * nb;   // threads 0..127
+    // every thread loads a scale (threads 128.. repeat rows 0..): a load under a branch would hide
+    // the number of loads in flight from the wait that precedes the LDS stores
+    const float *dxbase = a.d + (m0 + (tid & (BM - 1)) < M ? m0 + (tid & (BM - 1)) : M - 1) * nb;
 
     auto load_stage = [&](Regs &r, int64_t sb, int g) {   // K-step g (0..3) of super-block sb
         const uint8_t *blk = wbase + sb * 144;
@@ -403,7 +400,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const Wei
         r.wq1 = q2.y;
         if (g == 0) {
             hdr = *reinterpret_cast<const v4i *>(blk);
-            if (tid < BM) dx_next = dxbase[sb];
+            dx_next = dxbase[sb];
         }
         r.act = *reinterpret_cast<const v4i *>(abase + sb * 256 + 64 * g);
     };
@@ -435,16 +432,16 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const Wei
 
     const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     v16i ilo[2], ihi[2];
-    // one K-step: two sub-blocks, for each the low and the high chain of both column tiles
+    // one K-step: two sub-blocks, for each the low and the high chain of both token tiles
     auto kstep = [&](const Q8kStage &st, bool first) {
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
-            const v4i af = *reinterpret_cast<const v4i *>(st.a + (wm * 32 + l32) * QLD + blk * 32 + 16 * lh);
+            const int o = (wn * 32 + l32) * QLD + blk * 32 + 16 * lh;
+            const v4i bl = *reinterpret_cast<const v4i *>(st.b_lo + o);
+            const v4i bh = *reinterpret_cast<const v4i *>(st.b_hi + o);
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const int o = (wn * 64 + j * 32 + l32) * QLD + blk * 32 + 16 * lh;
-                const v4i bl = *reinterpret_cast<const v4i *>(st.b_lo + o);
-                const v4i bh = *reinterpret_cast<const v4i *>(st.b_hi + o);
+                const v4i af = *reinterpret_cast<const v4i *>(st.a + (wm * 64 + j * 32 + l32) * QLD + blk * 32 + 16 * lh);
                 if (first && blk == 0) {
                     ilo[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bl, zi, 0, 0, 0);
                     ihi[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bh, zi, 0, 0, 0);
@@ -467,15 +464,15 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const Wei
             kstep(sm.st[g & 1], g == 0);
             if (g == 3) {   // the super-block is complete: 8*I_hi + I_lo, scaled by dx*d, joins the fp32 sum
                 const float *dxs = sm.dx[sb & 1];
-                float dxv[16];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float4 d4 = *reinterpret_cast<const float4 *>(dxs + wm * 32 + 8 * i + 4 * lh);
-                    dxv[4 * i] = d4.x; dxv[4 * i + 1] = d4.y; dxv[4 * i + 2] = d4.z; dxv[4 * i + 3] = d4.w;
-                }
+                const float dn = sm.dn[sb & 1][wn * 32 + l32];
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
-                    const float dn = sm.dn[sb & 1][wn * 64 + j * 32 + l32];
+                    float dxv[16];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float4 d4 = *reinterpret_cast<const float4 *>(dxs + wm * 64 + j * 32 + 8 * i + 4 * lh);
+                        dxv[4 * i] = d4.x; dxv[4 * i + 1] = d4.y; dxv[4 * i + 2] = d4.z; dxv[4 * i + 3] = d4.w;
+                    }
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
                         acc[j][v] = fmaf((float)((ihi[j][v] << 3) + ilo[j][v]), dxv[v] * dn, acc[j][v]);
@@ -490,12 +487,12 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const Wei
     }
 
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
+    const int64_t n = n0 + wn * 32 + l32;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const int64_t n = n0 + wn * 64 + j * 32 + l32;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const int64_t m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            const int64_t m = m0 + wm * 64 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
             if (m < M && n < N) y[m * N + n] = acc[j][v];
         }
     }
