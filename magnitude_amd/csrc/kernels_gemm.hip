@@ -283,14 +283,15 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
 constexpr int QBK = 64;
 constexpr int QLD = QBK + 16;   // LDS row stride in bytes
 
-struct Q8kStage {
-    int8_t a[BM * QLD];       // activations [m][k]
-    int8_t b_lo[BN * QLD];    // (sc & 7) * q   [n][k]
-    int8_t b_hi[BN * QLD];    // (sc >> 3) * q  [n][k]
-};
+template <int WM>   // wave rows along the tokens: the tile is 64*WM tokens x 128 weight rows
 struct Q8kSmem {
-    Q8kStage st[2];
-    float dx[2][BM];          // activation scale of the super-block, by super-block parity
+    static constexpr int TM = 64 * WM;
+    struct Stage {
+        int8_t a[TM * QLD];       // activations [m][k]
+        int8_t b_lo[BN * QLD];    // (sc & 7) * q   [n][k]
+        int8_t b_hi[BN * QLD];    // (sc >> 3) * q  [n][k]
+    } st[2];
+    float dx[2][TM];          // activation scale of the super-block, by super-block parity
     float dn[2][BN];          // weight d of the super-block
 };
 
@@ -299,16 +300,21 @@ __device__ __forceinline__ uint32_t pk_mul_u16(uint32_t x, uint32_t s2) {
     return __builtin_bit_cast(uint32_t, __builtin_bit_cast(v2us, x) * __builtin_bit_cast(v2us, s2));
 }
 
-__global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const WeightView w, const ActView a, int64_t M,
-                                                                     float *__restrict__ y) {
+template <int WM>
+__global__ __launch_bounds__(256 * WM, 2) void gemm_q4k_q8k_kernel(const WeightView w, const ActView a, int64_t M,
+                                                                  float *__restrict__ y) {
+    using Smem = Q8kSmem<WM>;
+    using Q8kStage = typename Smem::Stage;
+    constexpr int NT = 256 * WM, TM = 64 * WM;
+    constexpr int WS = 2 / WM;   // 8-byte weight slices a thread converts per K-step
     extern __shared__ __align__(16) uint8_t smem_raw[];
-    Q8kSmem &sm = *reinterpret_cast<Q8kSmem *>(smem_raw);
+    Smem &sm = *reinterpret_cast<Smem *>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 waves, each 64 tokens x 32 weight rows: one B fragment pair feeds two products
     const int64_t N = w.N, K = w.K, nb = w.nb;
     int tile_n, tile_m;
-    tile_of_workgroup((int)((N + BN - 1) / BN), (int)((M + BM - 1) / BM), tile_n, tile_m);
-    const int64_t n0 = (int64_t)tile_n * BN, m0 = (int64_t)tile_m * BM;
+    tile_of_workgroup((int)((N + BN - 1) / BN), (int)((M + TM - 1) / TM), tile_n, tile_m);
+    const int64_t n0 = (int64_t)tile_n * BN, m0 = (int64_t)tile_m * TM;
     const int l32 = lane & 31, lh = lane >> 5;
 
     const int64_t ncol = n0 + wn * 32 + l32 < N ? n0 + wn * 32 + l32 : N - 1;
@@ -379,48 +385,61 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_q4k_q8k_kernel(const Wei
     // K-step of a super-block, so every index below is a compile-time constant.
     struct Regs {
         v4i act;
-        uint32_t wq0, wq1;
+        uint32_t wq[2 * WS];
     } regs[4];
-    v4i hdr = {0, 0, 0, 0};
+    v4i hdr[WS];
     float dx_next = 0.f;
-    const int wrow = tid >> 2, wpart = tid & 3;   // weight staging: row, 8-byte slice of the 32-byte group
-    int64_t wn_row = n0 + wrow;
-    if (wn_row >= N) wn_row = N - 1;
-    const uint8_t *wbase = w.q4k + wn_row * nb * 144;
+    // weight staging: slice id = tid + NT*j -> row id / 4, 8-byte part id % 4 of the 32-byte group
+    const uint8_t *wbase[WS];
+#pragma unroll
+    for (int j = 0; j < WS; ++j) {
+        int64_t r = n0 + ((tid + NT * j) >> 2);
+        if (r >= N) r = N - 1;
+        wbase[j] = w.q4k + r * nb * 144 + 8 * (tid & 3);
+    }
     const int arow = tid >> 2, aseg = tid & 3;    // activation staging: row, 16-byte segment of the 64
     const int8_t *abase = a.qs + (m0 + arow < M ? m0 + arow : M - 1) * K + 16 * aseg;
     // every thread loads a scale (threads 128.. repeat rows 0..): a load under a branch would hide
     // the number of loads in flight from the wait that precedes the LDS stores
-    const float *dxbase = a.d + (m0 + (tid & (BM - 1)) < M ? m0 + (tid & (BM - 1)) : M - 1) * nb;
+    const float *dxbase = a.d + (m0 + (tid & (TM - 1)) < M ? m0 + (tid & (TM - 1)) : M - 1) * nb;
 
     auto load_stage = [&](Regs &r, int64_t sb, int g) {   // K-step g (0..3) of super-block sb
-        const uint8_t *blk = wbase + sb * 144;
-        const uint2 q2 = *reinterpret_cast<const uint2 *>(blk + 16 + 32 * g + 8 * wpart);
-        r.wq0 = q2.x;
-        r.wq1 = q2.y;
+#pragma unroll
+        for (int j = 0; j < WS; ++j) {
+            const uint2 q2 = *reinterpret_cast<const uint2 *>(wbase[j] + sb * 144 + 16 + 32 * g);
+            r.wq[2 * j] = q2.x;
+            r.wq[2 * j + 1] = q2.y;
+        }
         if (g == 0) {
-            hdr = *reinterpret_cast<const v4i *>(blk);
+#pragma unroll
+            for (int j = 0; j < WS; ++j) hdr[j] = *reinterpret_cast<const v4i *>(wbase[j] - 8 * (tid & 3) + sb * 144);
             dx_next = dxbase[sb];
         }
         r.act = *reinterpret_cast<const v4i *>(abase + sb * 256 + 64 * g);
     };
-    ScalesK4 cur_sc{};
+    ScalesK4 cur_sc[WS];
     auto store_stage = [&](const Regs &r, Q8kStage &st, int64_t sb, int g) {
         if (g == 0) {
-            cur_sc = unpack_scales_k4((uint32_t)hdr[1], (uint32_t)hdr[2], (uint32_t)hdr[3]);
-            if (wpart == 0) sm.dn[sb & 1][wrow] = h2f((uint32_t)hdr[0]);
-            if (tid < BM) sm.dx[sb & 1][tid] = dx_next;
+#pragma unroll
+            for (int j = 0; j < WS; ++j) {
+                cur_sc[j] = unpack_scales_k4((uint32_t)hdr[j][1], (uint32_t)hdr[j][2], (uint32_t)hdr[j][3]);
+                if ((tid & 3) == 0) sm.dn[sb & 1][(tid + NT * j) >> 2] = h2f((uint32_t)hdr[j][0]);
+            }
+            if (tid < TM) sm.dx[sb & 1][tid] = dx_next;
         }
-        const uint32_t s0 = scale_k4(cur_sc, 2 * g), s1 = scale_k4(cur_sc, 2 * g + 1);   // sub-blocks 2g (low nibbles), 2g+1
-        const uint32_t s0l = (s0 & 7) * 0x00010001u, s0h = (s0 >> 3) * 0x00010001u;
-        const uint32_t s1l = (s1 & 7) * 0x00010001u, s1h = (s1 >> 3) * 0x00010001u;
-        const uint32_t x0 = r.wq0 & 0x0f0f0f0fu, x1 = r.wq1 & 0x0f0f0f0fu;
-        const uint32_t z0 = (r.wq0 >> 4) & 0x0f0f0f0fu, z1 = (r.wq1 >> 4) & 0x0f0f0f0fu;
-        const int o = wrow * QLD + 8 * wpart;
-        *reinterpret_cast<uint2 *>(st.b_lo + o) = make_uint2(pk_mul_u16(x0, s0l), pk_mul_u16(x1, s0l));
-        *reinterpret_cast<uint2 *>(st.b_hi + o) = make_uint2(pk_mul_u16(x0, s0h), pk_mul_u16(x1, s0h));
-        *reinterpret_cast<uint2 *>(st.b_lo + o + 32) = make_uint2(pk_mul_u16(z0, s1l), pk_mul_u16(z1, s1l));
-        *reinterpret_cast<uint2 *>(st.b_hi + o + 32) = make_uint2(pk_mul_u16(z0, s1h), pk_mul_u16(z1, s1h));
+#pragma unroll
+        for (int j = 0; j < WS; ++j) {
+            const uint32_t s0 = scale_k4(cur_sc[j], 2 * g), s1 = scale_k4(cur_sc[j], 2 * g + 1);   // sub-blocks 2g (low nibbles), 2g+1
+            const uint32_t s0l = (s0 & 7) * 0x00010001u, s0h = (s0 >> 3) * 0x00010001u;
+            const uint32_t s1l = (s1 & 7) * 0x00010001u, s1h = (s1 >> 3) * 0x00010001u;
+            const uint32_t x0 = r.wq[2 * j] & 0x0f0f0f0fu, x1 = r.wq[2 * j + 1] & 0x0f0f0f0fu;
+            const uint32_t z0 = (r.wq[2 * j] >> 4) & 0x0f0f0f0fu, z1 = (r.wq[2 * j + 1] >> 4) & 0x0f0f0f0fu;
+            const int o = ((tid + NT * j) >> 2) * QLD + 8 * (tid & 3);
+            *reinterpret_cast<uint2 *>(st.b_lo + o) = make_uint2(pk_mul_u16(x0, s0l), pk_mul_u16(x1, s0l));
+            *reinterpret_cast<uint2 *>(st.b_hi + o) = make_uint2(pk_mul_u16(x0, s0h), pk_mul_u16(x1, s0h));
+            *reinterpret_cast<uint2 *>(st.b_lo + o + 32) = make_uint2(pk_mul_u16(z0, s1l), pk_mul_u16(z1, s1l));
+            *reinterpret_cast<uint2 *>(st.b_hi + o + 32) = make_uint2(pk_mul_u16(z0, s1h), pk_mul_u16(z1, s1h));
+        }
         *reinterpret_cast<v4i *>(st.a + arow * QLD + 16 * aseg) = r.act;
     };
 
@@ -510,15 +529,27 @@ hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, f
     return hipGetLastError();
 }
 
+namespace {
+template <int WM>
+hipError_t launch_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
+    using Smem = Q8kSmem<WM>;
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_kernel<WM>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
+    if (attr != hipSuccess) return attr;
+    const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + Smem::TM - 1) / Smem::TM)));
+    hipLaunchKernelGGL(gemm_q4k_q8k_kernel<WM>, grid, dim3(256 * WM), sizeof(Smem), s, w, a, M, y);
+    return hipGetLastError();
+}
+}  // namespace
+
 // ggml-format activations (Q8_K planes in `a`), Q4_K weights, any M
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
     if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || M <= 0) return hipErrorInvalidValue;
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Q8kSmem));
-    if (attr != hipSuccess) return attr;
-    const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + BM - 1) / BM)));
-    hipLaunchKernelGGL(gemm_q4k_q8k_kernel, grid, dim3(kGemmThreads), sizeof(Q8kSmem), s, w, a, M, y);
-    return hipGetLastError();
+    // 128-token tiles when there are enough of them for 1.5 workgroups per compute unit (two fit),
+    // 64-token tiles below that
+    const int64_t tiles_n = (w.N + BN - 1) / BN;
+    if (tiles_n * ((M + 127) / 128) >= 384) return launch_q8k<2>(w, a, M, y, s);
+    return launch_q8k<1>(w, a, M, y, s);
 }
 
 }  // namespace qproj
