@@ -8,7 +8,7 @@ namespace qproj {
 
 __global__ __launch_bounds__(256) void quant_q8k_kernel(const float *__restrict__ x, int64_t n_super,
                                                         int8_t *__restrict__ qs, float *__restrict__ d,
-                                                        int16_t *__restrict__ bsums) {
+                                                        int16_t *__restrict__ bsums, uint16_t *__restrict__ msum) {
     const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (sb >= n_super) return;  // whole wave leaves together
@@ -19,6 +19,15 @@ __global__ __launch_bounds__(256) void quant_q8k_kernel(const float *__restrict_
     reinterpret_cast<uint32_t *>(qs + sb * 256)[lane] = packed;
     if ((lane & 3) == 0) bsums[sb * 16 + (lane >> 2)] = (int16_t)bsum;
     if (lane == 0) d[sb] = dd;
+    // d * (sum over a 32-wide sub-block), split into two fp16 parts, in the order the prefill
+    // kernel feeds them to the fp16 matrix instruction
+    const int pair = bsum + __shfl_xor(bsum, 4);
+    if ((lane & 7) == 0) {
+        const float v = dd * (float)pair * kMinPrescale;
+        const _Float16 hi = (_Float16)v, lo = (_Float16)(v - (float)hi);
+        msum[sb * 16 + (lane >> 3)] = __builtin_bit_cast(uint16_t, hi);
+        msum[sb * 16 + 8 + (lane >> 3)] = __builtin_bit_cast(uint16_t, lo);
+    }
 }
 
 // FP16_SCALE: ggml Q8_0 blocks (scale rounded through fp16).  Otherwise the prefill format:
@@ -47,13 +56,13 @@ __global__ __launch_bounds__(256) void quant_q8_32_kernel(const float *__restric
 }
 
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
-                               int16_t *bsums, int32_t *isum, hipStream_t s) {
+                               int16_t *bsums, uint16_t *msum, int32_t *isum, hipStream_t s) {
     const int64_t n = M * K;
     if (n == 0) return hipSuccess;
     const int64_t chunks = (n + 255) / 256;
     const dim3 grid((unsigned)((chunks + 3) / 4)), block(256);
     if (kind == kActKindQ8_K) {
-        hipLaunchKernelGGL(quant_q8k_kernel, grid, block, 0, s, x, n / 256, qs, d, bsums);
+        hipLaunchKernelGGL(quant_q8k_kernel, grid, block, 0, s, x, n / 256, qs, d, bsums, msum);
     } else if (kind == kActKindQ8_0) {
         hipLaunchKernelGGL(quant_q8_32_kernel<true>, grid, block, 0, s, x, chunks, n, qs, d, isum);
     } else if (kind == kActKindQ8X32) {

@@ -16,6 +16,7 @@
 //     header by that lane and held in registers for the 8 sub-blocks of a super-block;
 //   - LDS holds only the two int8 operand tiles and the transposed activation scales, double
 //     buffered over K-steps of 128 so that the global loads of step s+1 overlap step s.
+#include <cstdlib>
 #include "qproj_device.h"
 #include "qproj_internal.h"
 
@@ -30,7 +31,6 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr int BM = 128, BN = 128, BK = 128;
 constexpr int LDT = BK + 16;  // LDS row stride in bytes, padded against bank conflicts
-constexpr float kMinPrescale = 0.0625f;  // keeps da*isum inside fp16 range for |x| up to ~1e5
 
 struct GemmStage {
     int8_t a[BM * LDT];  // activations  [m][k]
@@ -334,21 +334,12 @@ __global__ __launch_bounds__(256 * WM, 2) void gemm_q4k_q8k_kernel(const WeightV
             for (int i = 0; i < 2; ++i) {
                 int64_t m = m0 + wm * 64 + i * 32 + l32;
                 int64_t sb = s * 2 + lh;
-                const bool live = m < M && sb < nb;
+                // rows past M are never stored and a super-block past the end meets zeroed mins
                 if (m >= M) m = M - 1;
                 if (sb >= nb) sb = nb - 1;
-                const float dx = a.d[m * nb + sb];
-                const uint4 *bp = reinterpret_cast<const uint4 *>(a.bsums + (m * nb + sb) * 16);
-                const uint4 b0 = bp[0], b1 = bp[1];
-                const uint32_t bw[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const int bs = (int)(int16_t)(bw[t] & 0xffff) + (int)(int16_t)(bw[t] >> 16);
-                    _Float16 h, l;
-                    split_h(live ? dx * (float)bs * kMinPrescale : 0.f, h, l);
-                    ah[i][t] = h;
-                    al[i][t] = l;
-                }
+                const v8h *mp = reinterpret_cast<const v8h *>(a.msum + (m * nb + sb) * 16);
+                ah[i] = mp[0];
+                al[i] = mp[1];
             }
             {
                 int64_t sb = s * 2 + lh;
@@ -517,6 +508,210 @@ __global__ __launch_bounds__(256 * WM, 2) void gemm_q4k_q8k_kernel(const WeightV
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same arithmetic with the weights kept out of LDS.  Inside a super-block the order of the 256
+// products is free (both chains run over all of it), so a lane may feed the matrix instruction
+// with whichever 16 weights it likes as long as the activation operand carries the matching 16:
+// lane (row l%32, half l/32) loads the 64 contiguous nibble bytes [64*half, 64*half+64) of its
+// own weight row = sub-blocks 4*half .. 4*half+3, expands and scales them in registers, and reads
+// the activations of exactly those sub-blocks from LDS.  Each of the NW waves owns 32 weight rows
+// of the tile and all of its 64 tokens; LDS carries only the activation tile (one super-block,
+// double-buffered), so there is one workgroup barrier per 256 weights, no weight stores to LDS and
+// half the LDS reads of the tiled kernel above.
+constexpr int DLA = 256 + 16;   // LDS row stride of the activation tile in bytes
+
+struct DirectSmem {
+    int8_t a[2][64 * DLA];
+    float dx[2][64];
+};
+
+struct DirectB {     // one super-block of the lane's weight row as it comes from memory
+    v4i hdr;         // d, dmin, 12 bytes of 6-bit scales and mins
+    v4i q[4];        // 64 nibble bytes: q[2*gg + half] = bytes 16*half.. of the 32-byte group 2*(l/32) + gg
+};
+
+__device__ __forceinline__ uint32_t byte_to_u16x2(uint32_t word, int i) {
+    // byte i of word -> both 16-bit halves (v_perm_b32: selector 0x0c yields a zero byte)
+    return __builtin_amdgcn_perm(0u, word, 0x0c000c00u | (uint32_t)(i << 16) | (uint32_t)i);
+}
+
+template <int NW>
+__global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const WeightView w, const ActView a, int64_t M,
+                                                                        float *__restrict__ y) {
+    constexpr int NT = 64 * NW, TN = 32 * NW;
+    constexpr int PA = 1024 / NT;   // 16-byte activation pieces a thread moves per super-block
+    extern __shared__ __align__(16) uint8_t smem_raw[];
+    DirectSmem &sm = *reinterpret_cast<DirectSmem *>(smem_raw);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t N = w.N, K = w.K, nb = w.nb;
+    int tile_n, tile_m;
+    tile_of_workgroup((int)((N + TN - 1) / TN), (int)((M + 63) / 64), tile_n, tile_m);
+    const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * 64;
+    const int l32 = lane & 31, lh = lane >> 5;
+    const int64_t ncol = n0 + wave * 32 + l32 < N ? n0 + wave * 32 + l32 : N - 1;
+
+    v16f acc[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+    // ---------------------------------------------------------------- min term on the fp16 cores
+    {
+        const int64_t n_steps = (nb + 1) / 2;  // two super-blocks (16 sub-blocks) per product
+        for (int64_t s = 0; s < n_steps; ++s) {
+            v8h ah[2], al[2], bh, bl;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                int64_t m = m0 + i * 32 + l32;
+                int64_t sb = s * 2 + lh;
+                // rows past M are never stored and a super-block past the end meets zeroed mins
+                if (m >= M) m = M - 1;
+                if (sb >= nb) sb = nb - 1;
+                const v8h *mp = reinterpret_cast<const v8h *>(a.msum + (m * nb + sb) * 16);
+                ah[i] = mp[0];
+                al[i] = mp[1];
+            }
+            {
+                int64_t sb = s * 2 + lh;
+                const bool live = sb < nb;
+                if (!live) sb = nb - 1;
+                const v4i hd = *reinterpret_cast<const v4i *>(w.q4k + (ncol * nb + sb) * 144);
+                const ScalesK4 sc = unpack_scales_k4((uint32_t)hd[1], (uint32_t)hd[2], (uint32_t)hd[3]);
+                const float dmin = live ? h2f((uint32_t)hd[0] >> 16) : 0.f;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    _Float16 h, l;
+                    split_h(-(dmin * (float)min_k4(sc, t)), h, l);
+                    bh[t] = h;
+                    bl[t] = l;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bh, acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bl, acc[i], 0, 0, 0);
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[i], bh, acc[i], 0, 0, 0);
+            }
+        }
+        const float inv = 1.0f / kMinPrescale;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][v] *= inv;
+    }
+
+    // ---------------------------------------------------------------- main loop over super-blocks
+    const uint8_t *wrow = w.q4k + ncol * nb * 144;
+    const int8_t *arow[PA];
+    int aoff[PA];
+#pragma unroll
+    for (int p = 0; p < PA; ++p) {
+        const int id = tid + NT * p, row = id >> 4, seg = id & 15;
+        arow[p] = a.qs + (m0 + row < M ? m0 + row : M - 1) * K + 16 * seg;
+        aoff[p] = row * DLA + 16 * seg;
+    }
+    const float *dxrow = a.d + (m0 + (tid & 63) < M ? m0 + (tid & 63) : M - 1) * nb;
+
+    auto load_b = [&](DirectB &b, int64_t sb) {
+        const uint8_t *blk = wrow + sb * 144;
+        b.hdr = *reinterpret_cast<const v4i *>(blk);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) b.q[i] = *reinterpret_cast<const v4i *>(blk + 16 + 64 * lh + 16 * i);
+    };
+    v4i areg[PA];
+    float dxreg;
+    auto load_a = [&](int64_t sb) {
+#pragma unroll
+        for (int p = 0; p < PA; ++p) areg[p] = *reinterpret_cast<const v4i *>(arow[p] + sb * 256);
+        dxreg = dxrow[sb];
+    };
+    auto store_a = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < PA; ++p) *reinterpret_cast<v4i *>(sm.a[buf] + aoff[p]) = areg[p];
+        sm.dx[buf][tid & 63] = dxreg;   // every thread stores (threads 64.. repeat tokens 0..): no branch, no load sunk into it
+    };
+
+    const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    auto superblock = [&](const DirectB &b, int buf) {
+        // the lane's four sub-block scales, split in base 8 and spread over both 16-bit halves
+        const ScalesK4 sc = unpack_scales_k4((uint32_t)b.hdr[1], (uint32_t)b.hdr[2], (uint32_t)b.hdr[3]);
+        const uint32_t scw = lh ? sc.sc_hi : sc.sc_lo;
+        const uint32_t lo_w = scw & 0x07070707u, hi_w = (scw >> 3) & 0x07070707u;
+        const int8_t *ap = sm.a[buf] + l32 * DLA + 128 * lh;
+        v16i ilo[2], ihi[2];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int gg = t >> 2, nib = (t >> 1) & 1, half = t & 1, i = 2 * gg + nib;
+            const uint32_t sl = byte_to_u16x2(lo_w, i), sh = byte_to_u16x2(hi_w, i);
+            const v4i raw = b.q[2 * gg + half];
+            v4i bl, bh;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t x = nib ? ((uint32_t)raw[c] >> 4) & 0x0f0f0f0fu : (uint32_t)raw[c] & 0x0f0f0f0fu;
+                bl[c] = (int)pk_mul_u16(x, sl);
+                bh[c] = (int)pk_mul_u16(x, sh);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const v4i af = *reinterpret_cast<const v4i *>(ap + j * 32 * DLA + 32 * i + 16 * half);
+                ilo[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bl, t == 0 ? zi : ilo[j], 0, 0, 0);
+                ihi[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bh, t == 0 ? zi : ihi[j], 0, 0, 0);
+            }
+        }
+        const float dn = h2f((uint32_t)b.hdr[0] & 0xffffu);
+        const float *dxs = sm.dx[buf];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            float dxv[16];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float4 d4 = *reinterpret_cast<const float4 *>(dxs + j * 32 + 8 * i + 4 * lh);
+                dxv[4 * i] = d4.x; dxv[4 * i + 1] = d4.y; dxv[4 * i + 2] = d4.z; dxv[4 * i + 3] = d4.w;
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                acc[j][v] = fmaf((float)((ihi[j][v] << 3) + ilo[j][v]), dxv[v] * dn, acc[j][v]);
+        }
+    };
+
+    DirectB b0, b1;
+    load_b(b0, 0);
+    load_a(0);
+    store_a(0);
+    __syncthreads();
+    // two super-blocks per trip so that the two weight register sets keep their names; loads past
+    // the end fetch the last super-block again (an unconditional load keeps the wait counters exact)
+    for (int64_t sb = 0; sb < nb; sb += 2) {
+        const int64_t s1 = sb + 1 < nb ? sb + 1 : nb - 1, s2 = sb + 2 < nb ? sb + 2 : nb - 1;
+        load_b(b1, s1);
+        load_a(s1);
+        __builtin_amdgcn_sched_barrier(0);   // the loads stay ahead of the arithmetic they overlap with
+        superblock(b0, 0);
+        store_a(1);
+        __syncthreads();
+        if (sb + 1 < nb) {
+            load_b(b0, s2);
+            load_a(s2);
+            __builtin_amdgcn_sched_barrier(0);
+            superblock(b1, 1);
+            store_a(0);
+            __syncthreads();
+        }
+    }
+
+    // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
+    const int64_t n = n0 + wave * 32 + l32;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (m < M && n < N) y[m * N + n] = acc[j][v];
+        }
+    }
+}
+
 }  // namespace
 
 hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
@@ -540,11 +735,20 @@ hipError_t launch_q8k(const WeightView &w, const ActView &a, int64_t M, float *y
     hipLaunchKernelGGL(gemm_q4k_q8k_kernel<WM>, grid, dim3(256 * WM), sizeof(Smem), s, w, a, M, y);
     return hipGetLastError();
 }
+template <int NW>
+hipError_t launch_q8k_direct(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
+    const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64)));
+    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(DirectSmem), s, w, a, M, y);
+    return hipGetLastError();
+}
 }  // namespace
 
 // ggml-format activations (Q8_K planes in `a`), Q4_K weights, any M
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
     if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || M <= 0) return hipErrorInvalidValue;
+    static const int variant = [] { const char *e = getenv("QPROJ_GEMM_Q8K_VARIANT"); return e ? atoi(e) : 0; }();
+    if (variant == 8) return launch_q8k_direct<8>(w, a, M, y, s);
+    if (variant == 4) return launch_q8k_direct<4>(w, a, M, y, s);
     // 128-token tiles when there are enough of them for 1.5 workgroups per compute unit (two fit),
     // 64-token tiles below that
     const int64_t tiles_n = (w.N + BN - 1) / BN;

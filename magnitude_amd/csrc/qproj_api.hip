@@ -78,7 +78,7 @@ int ensure_ws(qproj_ctx *ctx, size_t bytes) {
 
 // planes of a quantized-activation buffer, in the order the header documents
 struct ActPlanes {
-    size_t off_qs = 0, off_d = 0, off_aux = 0, total = 0;
+    size_t off_qs = 0, off_d = 0, off_aux = 0, off_msum = 0, total = 0;
     int kind = 0;
 };
 
@@ -97,7 +97,8 @@ ActPlanes act_planes(int kind, int64_t M, int64_t K) {
     size_t aux = 0;
     if (kind == kActKindQ8_K) aux = (size_t)(M * (K / 16)) * 2;
     if (kind == kActKindQ8X32) aux = (size_t)(M * (K / 32)) * 4;
-    p.total = p.off_aux + align_up(aux);
+    p.off_msum = p.off_aux + align_up(aux);
+    p.total = p.off_msum + (kind == kActKindQ8_K ? align_up((size_t)(M * (K / 256)) * 32) : 0);
     return p;
 }
 
@@ -108,6 +109,7 @@ ActView act_view(const ActPlanes &p, uint8_t *base, int64_t K) {
     a.qs = reinterpret_cast<const int8_t *>(base + p.off_qs);
     a.d = reinterpret_cast<const float *>(base + p.off_d);
     a.bsums = p.kind == kActKindQ8_K ? reinterpret_cast<const int16_t *>(base + p.off_aux) : nullptr;
+    a.msum = p.kind == kActKindQ8_K ? reinterpret_cast<const uint16_t *>(base + p.off_msum) : nullptr;
     a.isum = p.kind == kActKindQ8X32 ? reinterpret_cast<const int32_t *>(base + p.off_aux) : nullptr;
     return a;
 }
@@ -116,6 +118,7 @@ hipError_t run_quantize(qproj_ctx *ctx, const ActPlanes &p, uint8_t *base, const
     return launch_quantize_act(p.kind, x, M, K, reinterpret_cast<int8_t *>(base + p.off_qs),
                                reinterpret_cast<float *>(base + p.off_d),
                                reinterpret_cast<int16_t *>(base + p.off_aux),
+                               reinterpret_cast<uint16_t *>(base + p.off_msum),
                                reinterpret_cast<int32_t *>(base + p.off_aux), ctx->stream);
 }
 
@@ -125,6 +128,7 @@ ActView act_rows(const ActView &a, int64_t m0) {
     r.qs = a.qs + m0 * a.K;
     r.d = a.d + m0 * (a.K / dblk);
     if (a.bsums) r.bsums = a.bsums + m0 * (a.K / 16);
+    if (a.msum) r.msum = a.msum + m0 * (a.K / 16);
     if (a.isum) r.isum = a.isum + m0 * (a.K / 32);
     return r;
 }

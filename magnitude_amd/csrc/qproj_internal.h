@@ -41,8 +41,11 @@ struct ActView {
     const int8_t *qs;      // [rows][K]
     const float *d;        // [rows][K/32] (Q8_0, Q8X32) or [rows][K/256] (Q8_K)
     const int16_t *bsums;  // Q8_K: [rows][K/16]
+    const uint16_t *msum;  // Q8_K: [rows][K/256][16] fp16: d * (sum of 32 codes) * kMinPrescale for the 8
+                           //       sub-blocks, high parts, then the 8 low parts (v - high); prefill min term
     const int32_t *isum;   // Q8X32: [rows][K/32]
 };
+constexpr float kMinPrescale = 0.0625f;  // keeps d * sum inside fp16 range for |x| up to ~1e5
 constexpr int kActKindQ8_0 = 0;
 constexpr int kActKindQ8_K = 1;
 constexpr int kActKindQ8X32 = 2;
@@ -75,7 +78,7 @@ hipError_t launch_repack_to_planes(int type, const uint8_t *gguf, uint8_t *plane
                                    int64_t n_blocks, hipStream_t s);
 hipError_t launch_repack_to_gguf(int type, const WeightView &w, uint8_t *gguf, int64_t n_blocks, hipStream_t s);
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
-                               int16_t *bsums, int32_t *isum, hipStream_t s);
+                               int16_t *bsums, uint16_t *msum, int32_t *isum, hipStream_t s);
 hipError_t launch_gemv_q8act(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
 // persistent decode kernel (mt <= 4 rows); fuse_quantize: args.x holds fp32 rows, else args.a
 bool decode_kernel_fits(int type, int mt, int64_t K);

@@ -144,6 +144,14 @@ def test_quantize_q8_K_bit_exact(ctx, orc):
     assert np.array_equal(got["qs"].cpu().numpy(), want_q)
     assert np.array_equal(got["d"].cpu().numpy().view(np.uint32), want_d.view(np.uint32))
     assert np.array_equal(got["bsums"].cpu().numpy(), want_b)
+    # the prefill kernel's extra plane: d * (sum of each 32 codes) / 16, as an fp16 high part and
+    # the fp16 of what the high part leaves (numpy's float16 rounds to nearest even like the device)
+    v = want_d[:, :, None] * want_b.reshape(m, k // 256, 8, 2).sum(-1).astype(np.float32) * np.float32(0.0625)
+    hi = v.astype(np.float16)
+    lo = (v - hi.astype(np.float32)).astype(np.float16)
+    ms = got["msum"].cpu().numpy()
+    assert np.array_equal(ms[:, :, 0].view(np.uint16), hi.view(np.uint16))
+    assert np.array_equal(ms[:, :, 1].view(np.uint16), lo.view(np.uint16))
 
 
 def test_quantize_q8_0_activations_bit_exact(ctx, orc):
