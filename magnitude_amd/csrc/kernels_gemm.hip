@@ -16,7 +16,6 @@
 //     header by that lane and held in registers for the 8 sub-blocks of a super-block;
 //   - LDS holds only the two int8 operand tiles and the transposed activation scales, double
 //     buffered over K-steps of 128 so that the global loads of step s+1 overlap step s.
-#include <cstdlib>
 #include "qproj_device.h"
 #include "qproj_internal.h"
 
@@ -271,261 +270,45 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
 // With a single activation scale per super-block the integer sums of its eight sub-blocks may be
 // added before anything turns into floating point; only the 6-bit sub-block scale sc stands in the
 // way, and sc*q (up to 945) does not fit an int8 operand.  Written in base 8, sc = 8*sc_hi + sc_lo,
-// both products sc_lo*q and sc_hi*q stay below 106: the kernel keeps TWO int8 weight tiles in LDS
-// and runs two accumulation chains over the whole super-block entirely inside the matrix cores,
+// both products sc_lo*q and sc_hi*q stay below 106: two int8 weight operands and two accumulation
+// chains over the whole super-block run entirely inside the matrix cores,
 //     I_lo = sum_k (sc_lo*q) * a,   I_hi = sum_k (sc_hi*q) * a,   sum_k sc*q*a = 8*I_hi + I_lo,
 // so the vector ALU only works once per 256 weights (shift-add, int->float, one fma with dx*d).
-// Twice the matrix instructions of the per-32 kernel, a sixth of its vector instructions.
-//
-// Tile 128 tokens x 128 weight rows, 8 waves of 64 tokens x 32 rows, K-steps of 64 (one 32-byte nibble group =
-// two sub-blocks), double-buffered, two workgroups per CU.  The min term is the same small fp16
-// product as above, fed with dx*bsum.
-constexpr int QBK = 64;
-constexpr int QLD = QBK + 16;   // LDS row stride in bytes
-
-template <int WM>   // wave rows along the tokens: the tile is 64*WM tokens x 128 weight rows
-struct Q8kSmem {
-    static constexpr int TM = 64 * WM;
-    struct Stage {
-        int8_t a[TM * QLD];       // activations [m][k]
-        int8_t b_lo[BN * QLD];    // (sc & 7) * q   [n][k]
-        int8_t b_hi[BN * QLD];    // (sc >> 3) * q  [n][k]
-    } st[2];
-    float dx[2][TM];          // activation scale of the super-block, by super-block parity
-    float dn[2][BN];          // weight d of the super-block
-};
-
+// Twice the matrix instructions of the per-32 kernel, a third of its vector instructions.
 typedef unsigned short v2us __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pk_mul_u16(uint32_t x, uint32_t s2) {
     return __builtin_bit_cast(uint32_t, __builtin_bit_cast(v2us, x) * __builtin_bit_cast(v2us, s2));
 }
 
-template <int WM>
-__global__ __launch_bounds__(256 * WM, 2) void gemm_q4k_q8k_kernel(const WeightView w, const ActView a, int64_t M,
-                                                                  float *__restrict__ y) {
-    using Smem = Q8kSmem<WM>;
-    using Q8kStage = typename Smem::Stage;
-    constexpr int NT = 256 * WM, TM = 64 * WM;
-    constexpr int WS = 2 / WM;   // 8-byte weight slices a thread converts per K-step
-    extern __shared__ __align__(16) uint8_t smem_raw[];
-    Smem &sm = *reinterpret_cast<Smem *>(smem_raw);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 waves, each 64 tokens x 32 weight rows: one B fragment pair feeds two products
-    const int64_t N = w.N, K = w.K, nb = w.nb;
-    int tile_n, tile_m;
-    tile_of_workgroup((int)((N + BN - 1) / BN), (int)((M + TM - 1) / TM), tile_n, tile_m);
-    const int64_t n0 = (int64_t)tile_n * BN, m0 = (int64_t)tile_m * TM;
-    const int l32 = lane & 31, lh = lane >> 5;
-
-    const int64_t ncol = n0 + wn * 32 + l32 < N ? n0 + wn * 32 + l32 : N - 1;
-
-    v16f acc[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
-
-    // ---------------------------------------------------------------- min term on the fp16 cores
-    {
-        const int64_t n_steps = (nb + 1) / 2;  // two super-blocks (16 sub-blocks) per product
-        for (int64_t s = 0; s < n_steps; ++s) {
-            v8h ah[2], al[2], bh, bl;
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                int64_t m = m0 + wm * 64 + i * 32 + l32;
-                int64_t sb = s * 2 + lh;
-                // rows past M are never stored and a super-block past the end meets zeroed mins
-                if (m >= M) m = M - 1;
-                if (sb >= nb) sb = nb - 1;
-                const v8h *mp = reinterpret_cast<const v8h *>(a.msum + (m * nb + sb) * 16);
-                ah[i] = mp[0];
-                al[i] = mp[1];
-            }
-            {
-                int64_t sb = s * 2 + lh;
-                const bool live = sb < nb;
-                if (!live) sb = nb - 1;
-                const uint4 hd = *reinterpret_cast<const uint4 *>(w.q4k + (ncol * nb + sb) * 144);
-                const ScalesK4 sc = unpack_scales_k4(hd.y, hd.z, hd.w);
-                const float dmin = live ? h2f(hd.x >> 16) : 0.f;
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    _Float16 h, l;
-                    split_h(-(dmin * (float)min_k4(sc, t)), h, l);
-                    bh[t] = h;
-                    bl[t] = l;
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bh, acc[i], 0, 0, 0);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bl, acc[i], 0, 0, 0);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[i], bh, acc[i], 0, 0, 0);
-            }
-        }
-        const float inv = 1.0f / kMinPrescale;
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][v] *= inv;
-    }
-
-    // ---------------------------------------------------------------- main loop
-    // Global loads run THREE K-steps ahead of the arithmetic (a K-step is only eight matrix
-    // instructions per wave, far shorter than a trip to memory): four register sets, one per
-    // K-step of a super-block, so every index below is a compile-time constant.
-    struct Regs {
-        v4i act;
-        uint32_t wq[2 * WS];
-    } regs[4];
-    v4i hdr[WS];
-    float dx_next = 0.f;
-    // weight staging: slice id = tid + NT*j -> row id / 4, 8-byte part id % 4 of the 32-byte group
-    const uint8_t *wbase[WS];
-#pragma unroll
-    for (int j = 0; j < WS; ++j) {
-        int64_t r = n0 + ((tid + NT * j) >> 2);
-        if (r >= N) r = N - 1;
-        wbase[j] = w.q4k + r * nb * 144 + 8 * (tid & 3);
-    }
-    const int arow = tid >> 2, aseg = tid & 3;    // activation staging: row, 16-byte segment of the 64
-    const int8_t *abase = a.qs + (m0 + arow < M ? m0 + arow : M - 1) * K + 16 * aseg;
-    // every thread loads a scale (threads 128.. repeat rows 0..): a load under a branch would hide
-    // the number of loads in flight from the wait that precedes the LDS stores
-    const float *dxbase = a.d + (m0 + (tid & (TM - 1)) < M ? m0 + (tid & (TM - 1)) : M - 1) * nb;
-
-    auto load_stage = [&](Regs &r, int64_t sb, int g) {   // K-step g (0..3) of super-block sb
-#pragma unroll
-        for (int j = 0; j < WS; ++j) {
-            const uint2 q2 = *reinterpret_cast<const uint2 *>(wbase[j] + sb * 144 + 16 + 32 * g);
-            r.wq[2 * j] = q2.x;
-            r.wq[2 * j + 1] = q2.y;
-        }
-        if (g == 0) {
-#pragma unroll
-            for (int j = 0; j < WS; ++j) hdr[j] = *reinterpret_cast<const v4i *>(wbase[j] - 8 * (tid & 3) + sb * 144);
-            dx_next = dxbase[sb];
-        }
-        r.act = *reinterpret_cast<const v4i *>(abase + sb * 256 + 64 * g);
-    };
-    ScalesK4 cur_sc[WS];
-    auto store_stage = [&](const Regs &r, Q8kStage &st, int64_t sb, int g) {
-        if (g == 0) {
-#pragma unroll
-            for (int j = 0; j < WS; ++j) {
-                cur_sc[j] = unpack_scales_k4((uint32_t)hdr[j][1], (uint32_t)hdr[j][2], (uint32_t)hdr[j][3]);
-                if ((tid & 3) == 0) sm.dn[sb & 1][(tid + NT * j) >> 2] = h2f((uint32_t)hdr[j][0]);
-            }
-            if (tid < TM) sm.dx[sb & 1][tid] = dx_next;
-        }
-#pragma unroll
-        for (int j = 0; j < WS; ++j) {
-            const uint32_t s0 = scale_k4(cur_sc[j], 2 * g), s1 = scale_k4(cur_sc[j], 2 * g + 1);   // sub-blocks 2g (low nibbles), 2g+1
-            const uint32_t s0l = (s0 & 7) * 0x00010001u, s0h = (s0 >> 3) * 0x00010001u;
-            const uint32_t s1l = (s1 & 7) * 0x00010001u, s1h = (s1 >> 3) * 0x00010001u;
-            const uint32_t x0 = r.wq[2 * j] & 0x0f0f0f0fu, x1 = r.wq[2 * j + 1] & 0x0f0f0f0fu;
-            const uint32_t z0 = (r.wq[2 * j] >> 4) & 0x0f0f0f0fu, z1 = (r.wq[2 * j + 1] >> 4) & 0x0f0f0f0fu;
-            const int o = ((tid + NT * j) >> 2) * QLD + 8 * (tid & 3);
-            *reinterpret_cast<uint2 *>(st.b_lo + o) = make_uint2(pk_mul_u16(x0, s0l), pk_mul_u16(x1, s0l));
-            *reinterpret_cast<uint2 *>(st.b_hi + o) = make_uint2(pk_mul_u16(x0, s0h), pk_mul_u16(x1, s0h));
-            *reinterpret_cast<uint2 *>(st.b_lo + o + 32) = make_uint2(pk_mul_u16(z0, s1l), pk_mul_u16(z1, s1l));
-            *reinterpret_cast<uint2 *>(st.b_hi + o + 32) = make_uint2(pk_mul_u16(z0, s1h), pk_mul_u16(z1, s1h));
-        }
-        *reinterpret_cast<v4i *>(st.a + arow * QLD + 16 * aseg) = r.act;
-    };
-
-    load_stage(regs[0], 0, 0);
-    load_stage(regs[1], 0, 1);
-    load_stage(regs[2], 0, 2);
-    store_stage(regs[0], sm.st[0], 0, 0);
-    __syncthreads();
-
-    const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    v16i ilo[2], ihi[2];
-    // one K-step: two sub-blocks, for each the low and the high chain of both token tiles
-    auto kstep = [&](const Q8kStage &st, bool first) {
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-            const int o = (wn * 32 + l32) * QLD + blk * 32 + 16 * lh;
-            const v4i bl = *reinterpret_cast<const v4i *>(st.b_lo + o);
-            const v4i bh = *reinterpret_cast<const v4i *>(st.b_hi + o);
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                const v4i af = *reinterpret_cast<const v4i *>(st.a + (wm * 64 + j * 32 + l32) * QLD + blk * 32 + 16 * lh);
-                if (first && blk == 0) {
-                    ilo[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bl, zi, 0, 0, 0);
-                    ihi[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bh, zi, 0, 0, 0);
-                } else {
-                    ilo[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bl, ilo[j], 0, 0, 0);
-                    ihi[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bh, ihi[j], 0, 0, 0);
-                }
-            }
-        }
-    };
-    for (int64_t sb = 0; sb < nb; ++sb) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            {   // K-step three ahead
-                // (past the end the last super-block is fetched again: an unconditional load keeps the
-                // count of loads in flight known, so the wait before the LDS store can leave them flying)
-                const int64_t sb3 = g == 0 ? sb : (sb + 1 < nb ? sb + 1 : nb - 1);
-                load_stage(regs[(g + 3) & 3], sb3, (g + 3) & 3);
-            }
-            kstep(sm.st[g & 1], g == 0);
-            if (g == 3) {   // the super-block is complete: 8*I_hi + I_lo, scaled by dx*d, joins the fp32 sum
-                const float *dxs = sm.dx[sb & 1];
-                const float dn = sm.dn[sb & 1][wn * 32 + l32];
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    float dxv[16];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const float4 d4 = *reinterpret_cast<const float4 *>(dxs + wm * 64 + j * 32 + 8 * i + 4 * lh);
-                        dxv[4 * i] = d4.x; dxv[4 * i + 1] = d4.y; dxv[4 * i + 2] = d4.z; dxv[4 * i + 3] = d4.w;
-                    }
-#pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        acc[j][v] = fmaf((float)((ihi[j][v] << 3) + ilo[j][v]), dxv[v] * dn, acc[j][v]);
-                }
-            }
-            {   // next K-step into the other LDS stage
-                const int64_t sb1 = g < 3 ? sb : sb + 1;
-                if (sb1 < nb) store_stage(regs[(g + 1) & 3], sm.st[(g + 1) & 1], sb1, (g + 1) & 3);
-            }
-            __syncthreads();
-        }
-    }
-
-    // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
-    const int64_t n = n0 + wn * 32 + l32;
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int64_t m = m0 + wm * 64 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < M && n < N) y[m * N + n] = acc[j][v];
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
-// The same arithmetic with the weights kept out of LDS.  Inside a super-block the order of the 256
-// products is free (both chains run over all of it), so a lane may feed the matrix instruction
-// with whichever 16 weights it likes as long as the activation operand carries the matching 16:
-// lane (row l%32, half l/32) loads the 64 contiguous nibble bytes [64*half, 64*half+64) of its
-// own weight row = sub-blocks 4*half .. 4*half+3, expands and scales them in registers, and reads
-// the activations of exactly those sub-blocks from LDS.  Each of the NW waves owns 32 weight rows
-// of the tile and all of its 64 tokens; LDS carries only the activation tile (one super-block,
-// double-buffered), so there is one workgroup barrier per 256 weights, no weight stores to LDS and
-// half the LDS reads of the tiled kernel above.
+// The weights never become an LDS tile: they are converted in registers.  Inside a super-block
+// the order of the 256 products is free (both chains run over all of it), so a lane may feed the matrix
+// instruction with whichever 16 weights it likes as long as the activation operand carries the
+// matching 16: lane (row l%32, half l/32) takes the 64 contiguous nibble bytes [64*half, 64*half+64)
+// of its own weight row = sub-blocks 4*half .. 4*half+3, expands and scales them in registers, and
+// reads the activations of exactly those sub-blocks from LDS.  Each of the NW waves owns 32 weight
+// rows of the tile and all of its 64 tokens.
+//
+// Memory side: a lane-per-row load touches 64 cache lines per instruction and the vector memory
+// pipeline, not the arithmetic, becomes the limit.  So every wave fetches its 32 raw 144-byte blocks
+// with consecutive lanes on consecutive 16-byte pieces (288 pieces, five loads), parks them in a
+// wave-private LDS strip exactly as they lie in memory (a row stride of 144 bytes is conflict-free
+// for 16-byte reads) and picks its row's header and nibbles out of the strip.  The min term rides
+// along: the activation quantizer has already written d*(sub-block sum)/16 as fp16 pairs, the tile
+// of those is staged with the activations, and two fp16 matrix instructions per super-block and
+// token tile (operand [high | low] against [-dmin*min high | same], then [high | low] against
+// [-dmin*min low | 0]) add it to the accumulators, which therefore run in units of 1/16 until the
+// final store.  One workgroup barrier per 256 weights.
 constexpr int DLA = 256 + 16;   // LDS row stride of the activation tile in bytes
 
+template <int NW>
 struct DirectSmem {
-    int8_t a[2][64 * DLA];
-    float dx[2][64];
+    int8_t a[2][64 * DLA];           // activations of one super-block [token][256 + pad]
+    uint16_t ms[2][64 * 16];         // min-term operand [token][8 high | 8 low] (fp16 bits)
+    float dx[2][64];                 // activation scale of the super-block
+    uint8_t park[NW][32 * 144];      // per wave: the raw blocks of its 32 weight rows
 };
 
-struct DirectB {     // one super-block of the lane's weight row as it comes from memory
+struct DirectB {     // one super-block of the lane's weight row
     v4i hdr;         // d, dmin, 12 bytes of 6-bit scales and mins
     v4i q[4];        // 64 nibble bytes: q[2*gg + half] = bytes 16*half.. of the 32-byte group 2*(l/32) + gg
 };
@@ -541,14 +324,13 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const W
     constexpr int NT = 64 * NW, TN = 32 * NW;
     constexpr int PA = 1024 / NT;   // 16-byte activation pieces a thread moves per super-block
     extern __shared__ __align__(16) uint8_t smem_raw[];
-    DirectSmem &sm = *reinterpret_cast<DirectSmem *>(smem_raw);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    DirectSmem<NW> &sm = *reinterpret_cast<DirectSmem<NW> *>(smem_raw);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t N = w.N, K = w.K, nb = w.nb;
     int tile_n, tile_m;
     tile_of_workgroup((int)((N + TN - 1) / TN), (int)((M + 63) / 64), tile_n, tile_m);
     const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * 64;
     const int l32 = lane & 31, lh = lane >> 5;
-    const int64_t ncol = n0 + wave * 32 + l32 < N ? n0 + wave * 32 + l32 : N - 1;
 
     v16f acc[2];
 #pragma unroll
@@ -556,86 +338,83 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const W
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
 
-    // ---------------------------------------------------------------- min term on the fp16 cores
-    {
-        const int64_t n_steps = (nb + 1) / 2;  // two super-blocks (16 sub-blocks) per product
-        for (int64_t s = 0; s < n_steps; ++s) {
-            v8h ah[2], al[2], bh, bl;
+    // ---- global -> register -> LDS plumbing.  Every address is a wave-uniform base plus a 32-bit
+    // lane offset; rows past the edge of the matrix repeat the last valid row (never stored).
+    // weights: piece p = lane + 64*c of the wave's 288 -> row p / 9, 16-byte part p % 9
+    const int64_t wave_row0 = n0 + wave * 32 < N ? n0 + wave * 32 : N - 1;
+    const int wrow_cap = (int)(N - 1 - wave_row0 < 31 ? N - 1 - wave_row0 : 31);
+    const uint8_t *wbase = w.q4k + wave_row0 * nb * 144;
+    uint32_t woff[5];
+    int wpark[5];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                int64_t m = m0 + i * 32 + l32;
-                int64_t sb = s * 2 + lh;
-                // rows past M are never stored and a super-block past the end meets zeroed mins
-                if (m >= M) m = M - 1;
-                if (sb >= nb) sb = nb - 1;
-                const v8h *mp = reinterpret_cast<const v8h *>(a.msum + (m * nb + sb) * 16);
-                ah[i] = mp[0];
-                al[i] = mp[1];
-            }
-            {
-                int64_t sb = s * 2 + lh;
-                const bool live = sb < nb;
-                if (!live) sb = nb - 1;
-                const v4i hd = *reinterpret_cast<const v4i *>(w.q4k + (ncol * nb + sb) * 144);
-                const ScalesK4 sc = unpack_scales_k4((uint32_t)hd[1], (uint32_t)hd[2], (uint32_t)hd[3]);
-                const float dmin = live ? h2f((uint32_t)hd[0] >> 16) : 0.f;
-#pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    _Float16 h, l;
-                    split_h(-(dmin * (float)min_k4(sc, t)), h, l);
-                    bh[t] = h;
-                    bl[t] = l;
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bh, acc[i], 0, 0, 0);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[i], bl, acc[i], 0, 0, 0);
-                acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[i], bh, acc[i], 0, 0, 0);
-            }
-        }
-        const float inv = 1.0f / kMinPrescale;
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][v] *= inv;
+    for (int c = 0; c < 5; ++c) {
+        const int p = lane + 64 * c < 287 ? lane + 64 * c : 287;
+        const int r = p / 9 < wrow_cap ? p / 9 : wrow_cap;
+        woff[c] = (uint32_t)(r * (int)nb * 144 + 16 * (p % 9));
+        wpark[c] = 16 * p;
     }
-
-    // ---------------------------------------------------------------- main loop over super-blocks
-    const uint8_t *wrow = w.q4k + ncol * nb * 144;
-    const int8_t *arow[PA];
-    int aoff[PA];
+    // activations: piece id = tid + NT*p -> token id / 16, 16-byte segment id % 16
+    const int mrow_cap = (int)(M - 1 - m0 < 63 ? M - 1 - m0 : 63);
+    const int8_t *abase = a.qs + m0 * K;
+    uint32_t aoffg[PA];
+    int aoffl[PA];
 #pragma unroll
     for (int p = 0; p < PA; ++p) {
         const int id = tid + NT * p, row = id >> 4, seg = id & 15;
-        arow[p] = a.qs + (m0 + row < M ? m0 + row : M - 1) * K + 16 * seg;
-        aoff[p] = row * DLA + 16 * seg;
+        aoffg[p] = (uint32_t)((row < mrow_cap ? row : mrow_cap) * (int)K + 16 * seg);
+        aoffl[p] = row * DLA + 16 * seg;
     }
-    const float *dxrow = a.d + (m0 + (tid & 63) < M ? m0 + (tid & 63) : M - 1) * nb;
+    // min-term operand: 64 tokens x 32 bytes, thread t (mod 128) moves 16 bytes; scale: thread t (mod 64)
+    const uint8_t *msbase = reinterpret_cast<const uint8_t *>(a.msum) + m0 * nb * 32;
+    const int msrow = (tid & 127) >> 1;
+    const uint32_t msoffg = (uint32_t)((msrow < mrow_cap ? msrow : mrow_cap) * (int)nb * 32 + 16 * (tid & 1));
+    const float *dxbase = a.d + m0 * nb;
+    const uint32_t dxoffg = (uint32_t)(((tid & 63) < mrow_cap ? (tid & 63) : mrow_cap) * (int)nb);
 
-    auto load_b = [&](DirectB &b, int64_t sb) {
-        const uint8_t *blk = wrow + sb * 144;
-        b.hdr = *reinterpret_cast<const v4i *>(blk);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) b.q[i] = *reinterpret_cast<const v4i *>(blk + 16 + 64 * lh + 16 * i);
-    };
-    v4i areg[PA];
+    v4i stg[5], areg[PA], msreg;
     float dxreg;
-    auto load_a = [&](int64_t sb) {
+    auto load_next = [&](int64_t sb) {   // activations first: they are wanted at the end of this trip already
 #pragma unroll
-        for (int p = 0; p < PA; ++p) areg[p] = *reinterpret_cast<const v4i *>(arow[p] + sb * 256);
-        dxreg = dxrow[sb];
+        for (int p = 0; p < PA; ++p) areg[p] = *reinterpret_cast<const v4i *>(abase + sb * 256 + aoffg[p]);
+        msreg = *reinterpret_cast<const v4i *>(msbase + sb * 32 + msoffg);
+        dxreg = dxbase[sb + dxoffg];
+#pragma unroll
+        for (int c = 0; c < 5; ++c) stg[c] = *reinterpret_cast<const v4i *>(wbase + sb * 144 + woff[c]);
     };
-    auto store_a = [&](int buf) {
+    uint8_t *park = sm.park[wave];
+    auto store_next = [&](int buf) {
 #pragma unroll
-        for (int p = 0; p < PA; ++p) *reinterpret_cast<v4i *>(sm.a[buf] + aoff[p]) = areg[p];
-        sm.dx[buf][tid & 63] = dxreg;   // every thread stores (threads 64.. repeat tokens 0..): no branch, no load sunk into it
+        for (int p = 0; p < PA; ++p) *reinterpret_cast<v4i *>(sm.a[buf] + aoffl[p]) = areg[p];
+        // threads beyond the first 128 / 64 repeat a store of the same value: no branch, no load sunk into one
+        *reinterpret_cast<v4i *>(reinterpret_cast<uint8_t *>(sm.ms[buf]) + 16 * (tid & 127)) = msreg;
+        sm.dx[buf][tid & 63] = dxreg;
+#pragma unroll
+        for (int c = 0; c < 5; ++c) *reinterpret_cast<v4i *>(park + wpark[c]) = stg[c];
     };
 
     const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     auto superblock = [&](const DirectB &b, int buf) {
-        // the lane's four sub-block scales, split in base 8 and spread over both 16-bit halves
         const ScalesK4 sc = unpack_scales_k4((uint32_t)b.hdr[1], (uint32_t)b.hdr[2], (uint32_t)b.hdr[3]);
+        // ---- min term: -dmin*min of the 8 sub-blocks as fp16 high and low parts
+        {
+            const float ndmin = -h2f((uint32_t)b.hdr[0] >> 16);
+            v8h bh, bl;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                _Float16 h, l;
+                split_h(ndmin * (float)min_k4(sc, t), h, l);
+                bh[t] = h;
+                bl[t] = lh ? (_Float16)0.f : l;
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const v8h am = *reinterpret_cast<const v8h *>(reinterpret_cast<const uint8_t *>(sm.ms[buf]) +
+                                                             (j * 32 + l32) * 32 + 16 * lh);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, bh, acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, bl, acc[j], 0, 0, 0);
+            }
+        }
+        // ---- the lane's four sub-block scales, split in base 8 and spread over both 16-bit halves
         const uint32_t scw = lh ? sc.sc_hi : sc.sc_lo;
         const uint32_t lo_w = scw & 0x07070707u, hi_w = (scw >> 3) & 0x07070707u;
         const int8_t *ap = sm.a[buf] + l32 * DLA + 128 * lh;
@@ -659,7 +438,7 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const W
                 ihi[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bh, t == 0 ? zi : ihi[j], 0, 0, 0);
             }
         }
-        const float dn = h2f((uint32_t)b.hdr[0] & 0xffffu);
+        const float dn = h2f((uint32_t)b.hdr[0] & 0xffffu) * kMinPrescale;   // exact: a power of two
         const float *dxs = sm.dx[buf];
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -675,39 +454,32 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const W
         }
     };
 
-    DirectB b0, b1;
-    load_b(b0, 0);
-    load_a(0);
-    store_a(0);
+    load_next(0);
+    store_next(0);
     __syncthreads();
-    // two super-blocks per trip so that the two weight register sets keep their names; loads past
-    // the end fetch the last super-block again (an unconditional load keeps the wait counters exact)
-    for (int64_t sb = 0; sb < nb; sb += 2) {
-        const int64_t s1 = sb + 1 < nb ? sb + 1 : nb - 1, s2 = sb + 2 < nb ? sb + 2 : nb - 1;
-        load_b(b1, s1);
-        load_a(s1);
+    for (int64_t sb = 0; sb < nb; ++sb) {
+        const int buf = (int)(sb & 1);
+        DirectB b;   // out of the strip: header of row l%32, then the lane's 64 nibble bytes
+        b.hdr = *reinterpret_cast<const v4i *>(park + l32 * 144);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) b.q[i] = *reinterpret_cast<const v4i *>(park + l32 * 144 + 16 + 64 * lh + 16 * i);
+        // past the end the last super-block is fetched again: unconditional loads keep the wait counters exact
+        load_next(sb + 1 < nb ? sb + 1 : nb - 1);
         __builtin_amdgcn_sched_barrier(0);   // the loads stay ahead of the arithmetic they overlap with
-        superblock(b0, 0);
-        store_a(1);
+        superblock(b, buf);
+        store_next(buf ^ 1);
         __syncthreads();
-        if (sb + 1 < nb) {
-            load_b(b0, s2);
-            load_a(s2);
-            __builtin_amdgcn_sched_barrier(0);
-            superblock(b1, 1);
-            store_a(0);
-            __syncthreads();
-        }
     }
 
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
     const int64_t n = n0 + wave * 32 + l32;
+    const float inv = 1.0f / kMinPrescale;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < M && n < N) y[m * N + n] = acc[j][v];
+            if (m < M && n < N) y[m * N + n] = acc[j][v] * inv;
         }
     }
 }
@@ -724,36 +496,17 @@ hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, f
     return hipGetLastError();
 }
 
-namespace {
-template <int WM>
-hipError_t launch_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
-    using Smem = Q8kSmem<WM>;
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_kernel<WM>),
+// ggml-format activations (Q8_K planes in `a`, including the min-term plane), Q4_K weights, any M
+hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
+    if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || !a.msum || M <= 0) return hipErrorInvalidValue;
+    constexpr int NW = 4;   // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit
+    using Smem = DirectSmem<NW>;
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_direct_kernel<NW>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
     if (attr != hipSuccess) return attr;
-    const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + Smem::TM - 1) / Smem::TM)));
-    hipLaunchKernelGGL(gemm_q4k_q8k_kernel<WM>, grid, dim3(256 * WM), sizeof(Smem), s, w, a, M, y);
-    return hipGetLastError();
-}
-template <int NW>
-hipError_t launch_q8k_direct(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
     const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64)));
-    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(DirectSmem), s, w, a, M, y);
+    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, w, a, M, y);
     return hipGetLastError();
-}
-}  // namespace
-
-// ggml-format activations (Q8_K planes in `a`), Q4_K weights, any M
-hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
-    if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || M <= 0) return hipErrorInvalidValue;
-    static const int variant = [] { const char *e = getenv("QPROJ_GEMM_Q8K_VARIANT"); return e ? atoi(e) : 0; }();
-    if (variant == 8) return launch_q8k_direct<8>(w, a, M, y, s);
-    if (variant == 4) return launch_q8k_direct<4>(w, a, M, y, s);
-    // 128-token tiles when there are enough of them for 1.5 workgroups per compute unit (two fit),
-    // 64-token tiles below that
-    const int64_t tiles_n = (w.N + BN - 1) / BN;
-    if (tiles_n * ((M + 127) / 128) >= 384) return launch_q8k<2>(w, a, M, y, s);
-    return launch_q8k<1>(w, a, M, y, s);
 }
 
 }  // namespace qproj
