@@ -367,17 +367,18 @@ def main():
                           "headline_tops": head["gemm_tops"], "headline_frac_int8_peak": head["frac_int8_peak"],
                           "peak_tops": INT8_PEAK_TOPS, "shapes": res}
         # the same shapes in the ggml activation format (Q8_K, one scale per 256): the reference's own arithmetic
+        # (plus the layer's Q6_K down projection, which a Q4_K_M model runs through the same operator)
         resg = []
-        for (k, n) in ((4096, 14336), (14336, 4096), (4096, 4096)):
-            blocks = synth.random_weight(Q4_K, n, k, seed=77 + n, device=dev)
-            w = ctx.upload_from_device(Q4_K, k, n, blocks)
+        for (qt, k, n) in ((Q4_K, 4096, 14336), (Q4_K, 14336, 4096), (Q4_K, 4096, 4096), (Q6_K, 14336, 4096)):
+            blocks = synth.random_weight(qt, n, k, seed=77 + n, device=dev)
+            w = ctx.upload_from_device(qt, k, n, blocks)
             del blocks
             for m in (512, 2048, 4096):
                 x = torch.randn((m, k), generator=g, device=dev)
                 yb = torch.empty((m, n), device=dev)
-                qb = torch.empty(int(lib.qproj_act_bytes(ACT_GGML, Q4_K, m, k)), dtype=torch.uint8, device=dev)
+                qb = torch.empty(int(lib.qproj_act_bytes(ACT_GGML, qt, m, k)), dtype=torch.uint8, device=dev)
                 torch.cuda.synchronize()
-                fq = lambda: ctx.quantize_activations_raw(x, ACT_GGML, Q4_K, out=qb, sync=False)
+                fq = lambda: ctx.quantize_activations_raw(x, ACT_GGML, qt, out=qb, sync=False)
                 fg = lambda: ctx.mul_mat_quantized([w], qb, ACT_GGML, m, [yb], sync=False)
                 fq(); fg(); ctx.sync()
                 it = 5 if m * n * k > 1e11 else 10
@@ -385,21 +386,23 @@ def main():
                 sg = timer.samples_ms(fg, it)
                 tg = sum(sg) / len(sg)
                 ops = 2.0 * m * n * k
-                ev_rows.append(evidence.backend_ops_row("MUL_MAT", evidence.mul_mat_params(Q4_K, n, m, k),
+                ev_rows.append(evidence.backend_ops_row("MUL_MAT", evidence.mul_mat_params(qt, n, m, k),
                                                         [s * 1e3 for s in sg], flops=ops,
-                                                        bytes_moved=gguf_bytes(Q4_K, n, k) + m * k * 4 + m * n * 4,
-                                                        memory_kb=(gguf_bytes(Q4_K, n, k) + m * n * 4) // 1024,
+                                                        bytes_moved=gguf_bytes(qt, n, k) + m * k * 4 + m * n * 4,
+                                                        memory_kb=(gguf_bytes(qt, n, k) + m * n * 4) // 1024,
                                                         device=props.name))
-                resg.append({"M": m, "K": k, "N": n, "gemm_ms": tg, "quantize_ms": tq,
+                tname = "Q4_K" if qt == Q4_K else "Q6_K"
+                resg.append({"type": tname, "M": m, "K": k, "N": n, "gemm_ms": tg, "quantize_ms": tq,
                              "gemm_tops": ops / (tg * 1e-3) / 1e12,
                              "frac_int8_peak": ops / (tg * 1e-3) / 1e12 / INT8_PEAK_TOPS})
-                log(f"[bench] prefill(ggml acts) M={m} K={k} N={n}: gemm {tg:.3f} ms = {resg[-1]['gemm_tops']:.1f} TOPS "
+                log(f"[bench] prefill(ggml acts) {tname} M={m} K={k} N={n}: gemm {tg:.3f} ms = {resg[-1]['gemm_tops']:.1f} TOPS "
                     f"({100 * resg[-1]['frac_int8_peak']:.1f}% of int8 peak), quantize {tq:.3f} ms")
                 del x, yb, qb
             w.free()
-        headg = [r for r in resg if (r["M"], r["K"], r["N"]) == (4096, 4096, 14336)][0]
+        headg = [r for r in resg if (r["type"], r["M"], r["K"], r["N"]) == ("Q4_K", 4096, 4096, 14336)][0]
         out["prefill_ggml_acts"] = {"act_format": "ggml Q8_K (int8 + fp32 scale per 256, block sums)",
-                                    "mfma": "2 x v_mfma_i32_32x32x32_i8 per sub-block (scale split in base 8)",
+                                    "mfma": "Q4_K: 2 x v_mfma_i32_32x32x32_i8 per sub-block (scale split in base 8); "
+                                            "Q6_K: v_mfma_i32_32x32x16_i8 per sub-block, integer scale on the vector ALU",
                                     "headline_tops": headg["gemm_tops"], "headline_frac_int8_peak": headg["frac_int8_peak"],
                                     "shapes": resg}
 

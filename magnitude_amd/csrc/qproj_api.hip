@@ -266,8 +266,18 @@ size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
                     float *const *y, float *scratch) {
     static const int gemm_min_m = getenv("QPROJ_GEMM_MIN_M") ? atoi(getenv("QPROJ_GEMM_MIN_M")) : 48;
-    if (w[0]->type == kTypeQ4_K && M >= gemm_min_m) {   // prefill-sized batches: tiled product, weights reused across tokens
-        for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8k(w[i]->view, a, M, y[i], ctx->stream));
+    // prefill-sized batches: tiled product, weights reused across 64 tokens.  The Q6_K kernel is slow
+    // per workgroup (a vector multiply-add per output and sub-block): below 128 tiles of 64 x 128 it
+    // only pays from 112 tokens on, under that the small-batch kernel in steps of 16 is quicker.
+    const auto tiled = [&](const qproj_weight *t) {
+        if (M < gemm_min_m) return false;
+        if (t->type == kTypeQ4_K) return true;
+        return t->type == kTypeQ6_K && (M >= 112 || ((M + 63) / 64) * ((t->N + 127) / 128) >= 128);
+    };
+    if (tiled(w[0])) {
+        for (int i = 0; i < n; ++i)
+            QP_HIP(ctx, w[0]->type == kTypeQ4_K ? launch_gemm_q8k(w[i]->view, a, M, y[i], ctx->stream)
+                                                : launch_gemm_q6k_q8k(w[i]->view, a, M, y[i], ctx->stream));
         return QPROJ_OK;
     }
     if (use_mfma_kernel(w[0]->type, M, w[0]->K)) {

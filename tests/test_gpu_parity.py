@@ -204,18 +204,20 @@ def test_mul_mat_ggml_mode_matches_oracle(ctx, orc, qtype, m):
         w.free()
 
 
+@pytest.mark.parametrize("qtype", [Q4_K, Q6_K])
 @pytest.mark.parametrize("m,k,n", [(48, 4096, 256), (130, 768, 203), (200, 14336, 128), (333, 256, 40)])
-def test_mul_mat_ggml_mode_prefill_sized_batches(ctx, orc, m, k, n):
-    """Large M in the ggml activation format: the tiled matrix-core kernel (two int8 chains per
-    super-block) against the oracle's Q4_K x Q8_K integer arithmetic, ragged M and N included."""
+def test_mul_mat_ggml_mode_prefill_sized_batches(ctx, orc, qtype, m, k, n):
+    """Large M in the ggml activation format: the prefill matrix-core kernels (Q4_K: two int8 chains
+    per super-block; Q6_K: one K=16 product per sub-block, integer scale on the vector ALU) against
+    the oracle's integer arithmetic with Q8_K activations, ragged M and N included."""
     from magnitude_amd import ACT_GGML
-    blocks = make_weight(orc, Q4_K, n, k, seed=1500 + k + n)
+    blocks = make_weight(orc, qtype, n, k, seed=1500 + k + n)
     rng = np.random.default_rng(m + k)
     x = rng.standard_normal((m, k)).astype(np.float32)
     x[:, rng.integers(0, k, 8)] *= 30.0          # outlier channels, as transformer activations have
-    w = ctx.upload(Q4_K, k, n, blocks)
+    w = ctx.upload(qtype, k, n, blocks)
     got = ctx.mul_mat(w, dev(x), ACT_GGML).cpu().numpy()
-    want = orc.mul_mat(Q4_K, blocks, k, x, orc.ACT_GGML)
+    want = orc.mul_mat(qtype, blocks, k, x, orc.ACT_GGML)
     close(got, want, 2e-5)
     gate(got, want)
     # a row of the big batch is the small-batch kernel's row up to fp32 summation order
