@@ -9,7 +9,7 @@ the ggml activation mode (the reference CPU path's arithmetic).  `value` is algo
 per step / time.  Extra legs report the dominant kernel against the HBM roofline, the int8-MFMA
 prefill GEMM (config 4), the MoE feed-forward (config 5) and the CPU oracle on the host cores.
 
-    python bench.py --gpus 1 --steps 20 --warmup 3 [--legs step,roofline,verify,q8_0,prefill,moe,cpu]
+    python bench.py --gpus 1 --steps 20 --warmup 3 [--legs step,roofline,verify,q8_0,prefill,moe,llama_bench,cpu]
 """
 from __future__ import annotations
 
@@ -114,7 +114,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=32)
-    ap.add_argument("--legs", default="step,roofline,verify,q8_0,prefill,moe,cpu")
+    ap.add_argument("--legs", default="step,roofline,verify,q8_0,prefill,moe,llama_bench,cpu")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--split-quantize", action="store_true",
                     help="run the activation quantizer as a separate launch instead of inside the projection kernel")
@@ -157,7 +157,7 @@ def main():
     # ------------------------------------------------------------------ weights
     L = args.layers
     layers = []
-    need_layers = bool(legs & {"step", "roofline", "verify", "cpu"})
+    need_layers = bool(legs & {"step", "roofline", "verify", "cpu", "llama_bench"})
     if need_layers:
         t0 = time.time()
         for l in range(L):
@@ -470,6 +470,44 @@ def main():
                                "host_cpus": os.cpu_count(),
                                "one_thread_GBps": LAYER_BYTES / one / 1e9}
         log(f"[bench] cpu baseline: {cpu_gbs:.2f} GB/s on {threads} threads")
+
+    # ------------------------------------------------------------------ llama-bench style leg
+    # pp512 / tg128 over the projections of all layers (no attention, norms or sampling): the prompt
+    # pass is one 512-token batch per layer tensor group, generation is 128 single-token steps.
+    if "llama_bench" in legs:
+        n_prompt, n_gen, reps = 512, 128, 5
+        xs = {kk: torch.randn((n_prompt, kk), generator=g, device=dev) for kk in (D_MODEL, D_FF)}
+        yp = {name: torch.empty((n_prompt, n), device=dev) for name, _, n, _ in LAYER_TENSORS}
+
+        def prompt_pass():
+            for lw in layers:
+                for _, names, x1, _ in groups:
+                    ctx.mul_mat_multi([lw[nm] for nm in names], xs[x1.shape[1]], ACT_GGML,
+                                      outs=[yp[nm] for nm in names], sync=False)
+
+        def timed(fn):
+            fn(); ctx.sync(); torch.cuda.synchronize()
+            t0 = time.perf_counter_ns()
+            fn(); ctx.sync(); torch.cuda.synchronize()
+            return time.perf_counter_ns() - t0
+
+        def generate():
+            for _ in range(n_gen):
+                step()
+                ctx.sync()            # llama-bench synchronizes after every generated token
+
+        cfg = {"batch_size": n_prompt, "ubatch_size": n_prompt, "n_gpu_layers": L, "split_mode": "none", "main_gpu": 0,
+               "flash_attention": False, "warmup": True, "actual_backends": ["qproj-hip"],
+               "scope": "projection operators only (q,k,v,o,gate,up Q4_K; down Q6_K), ggml activation format"}
+        devs = [{"name": props.name, "backend": "ROCm", "index": 0}]
+        pp = [timed(prompt_pass) for _ in range(reps)]
+        tg = [timed(generate) for _ in range(reps)]
+        rec_pp = evidence.llama_bench_record("llama-bench.prompt-processing", n_prompt, 1, 0, 0, pp, cfg, devs)
+        rec_tg = evidence.llama_bench_record("llama-bench.token-generation", 0, 0, n_gen, n_gen, tg, cfg, devs)
+        out["llama_bench"] = [rec_pp, rec_tg]
+        med = lambda v: sorted(v)[len(v) // 2]
+        log(f"[bench] llama-bench style, projections only: pp{n_prompt} {n_prompt * 1e9 / med(pp):.0f} tok/s "
+            f"({med(pp) / 1e6:.2f} ms), tg{n_gen} {n_gen * 1e9 / med(tg):.0f} tok/s ({med(tg) / 1e6:.1f} ms)")
 
     if ev_rows:
         # the reference's own record shapes (test-backend-ops rows, parity measurements, fit calibration)

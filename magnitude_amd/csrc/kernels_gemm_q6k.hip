@@ -263,10 +263,9 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
 
 }  // namespace
 
-// ggml-format activations (Q8_K planes in `a`), Q6_K weights, any M
-hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
-    if (w.type != kTypeQ6_K || a.kind != kActKindQ8_K || !a.bsums || M <= 0) return hipErrorInvalidValue;
-    constexpr int NW = 4;   // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit
+namespace {
+template <int NW>
+hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
     using Smem = Q6Smem<NW>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q6k_q8k_kernel<NW>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
@@ -274,6 +273,15 @@ hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M,
     const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64)));
     hipLaunchKernelGGL(gemm_q6k_q8k_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, w, a, M, y);
     return hipGetLastError();
+}
+}  // namespace
+
+// ggml-format activations (Q8_K planes in `a`), Q6_K weights, any M
+hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
+    if (w.type != kTypeQ6_K || a.kind != kActKindQ8_K || !a.bsums || M <= 0) return hipErrorInvalidValue;
+    // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit (64 x 64 tiles for
+    // grids that leave compute units idle were measured slower: 0.30 against 0.25 ms at M=512)
+    return launch_q6k<4>(w, a, M, y, s);
 }
 
 }  // namespace qproj

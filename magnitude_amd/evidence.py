@@ -8,6 +8,10 @@
 * `calibration_metric`: one entry of the hardware calibration the engine's performance estimator
   consumes (inference/crates/icn-server/src/main.rs:1313-1325; `estimate_generation_performance`,
   icn-hardware/src/lib.rs:1508): bytes per second and launch overhead per tensor type.
+* `llama_bench_record`: the result object of the engine's llama-bench style probe
+  (inference/crates/icn-engine/src/parity_probe.rs:1352-1424: operation names :53-56, prompt loop
+  :1427-1469, generation loop :1471-1504), for a driver that runs the same prompt-processing /
+  token-generation schedule over the projections only.
 """
 from __future__ import annotations
 
@@ -88,4 +92,51 @@ def calibration_metric(tensor_type: int, routed: bool, bytes_per_launch: float, 
         "sample_count": len(samples_us),
         "measured_microseconds": int(round(sum(samples_us))),
         "stable": bool(spread < 0.10),
+    }
+
+
+LLAMA_BENCH_OPERATIONS = ("llama-bench.prompt-processing", "llama-bench.token-generation",
+                          "llama-bench.prompt-generation")
+
+
+def llama_bench_record(operation: str, prompt_tokens: int, prompt_calls: int, generation_tokens: int,
+                       generation_calls: int, durations_ns, effective_configuration: dict, devices,
+                       producer: str = "magnitude_amd/projection-only") -> dict:
+    """One record per measured case; every repetition keeps its own duration and tokens/s sample
+    (the probe measures one repetition per call, a harness collects them)."""
+    if operation not in LLAMA_BENCH_OPERATIONS:
+        raise ValueError(f"unknown operation {operation!r}")
+    durations_ns = [float(d) for d in durations_ns]
+    if not durations_ns or min(durations_ns) <= 0:
+        raise ValueError("measured duration was zero")
+    tokens = int(prompt_tokens) + int(generation_tokens)
+    shape_ok = {"llama-bench.prompt-processing": prompt_tokens > 0 and generation_tokens == 0,
+                "llama-bench.token-generation": prompt_tokens == 0 and generation_tokens > 0,
+                "llama-bench.prompt-generation": prompt_tokens > 0 and generation_tokens > 0}[operation]
+    if not shape_ok:
+        raise ValueError(f"token counts do not fit {operation}")
+    cfg = dict(effective_configuration)
+    cfg.setdefault("n_prompt", int(prompt_tokens))
+    cfg.setdefault("n_gen", int(generation_tokens))
+    return {
+        "schemaVersion": 1,
+        "output": {
+            "operation": operation,
+            "measuredPromptTokens": int(prompt_tokens),
+            "measuredPromptDecodeCalls": int(prompt_calls),
+            "measuredGenerationTokens": int(generation_tokens),
+            "measuredGenerationDecodeCalls": int(generation_calls),
+            "preparedContextDepthTokens": 0,
+            "preparedContextDepthDecodeCalls": 0,
+            "measurementRepetitions": len(durations_ns),
+            "measuredTokens": tokens,
+            "tokenSchedule": "synthetic-activations",   # projections see activations, never token ids
+        },
+        "measurements": [
+            measurement("duration", "ns", durations_ns),
+            measurement("tokens_per_second", "tokens/s", [tokens * 1e9 / d for d in durations_ns]),
+        ],
+        "effectiveConfiguration": cfg,
+        "devices": list(devices),
+        "producerVersion": producer,
     }

@@ -42,3 +42,30 @@ def test_calibration_metric_fields():
                       "launch_microseconds", "relative_spread", "sample_count", "measured_microseconds", "stable"}
     assert c["bytes_per_second"] == pytest.approx(66_191_360 / 15.5e-6)
     assert c["sample_count"] == 3 and c["stable"] and c["relative_spread"] == pytest.approx(1.0 / 15.5)
+
+
+def test_llama_bench_record_has_the_probe_result_shape():
+    """Field names and nesting of inference/crates/icn-engine/src/parity_probe.rs:1395-1424; one
+    duration and one tokens/s sample per repetition, tokens/s = tokens * 1e9 / ns (:1357)."""
+    from magnitude_amd import evidence
+    rec = evidence.llama_bench_record("llama-bench.prompt-processing", 512, 1, 0, 0, [2.0e6, 4.0e6],
+                                      {"batch_size": 512}, [{"name": "gpu"}])
+    assert rec["schemaVersion"] == 1
+    assert set(rec) == {"schemaVersion", "output", "measurements", "effectiveConfiguration", "devices", "producerVersion"}
+    out = rec["output"]
+    assert out["operation"] == "llama-bench.prompt-processing"
+    assert (out["measuredPromptTokens"], out["measuredPromptDecodeCalls"]) == (512, 1)
+    assert (out["measuredGenerationTokens"], out["measuredGenerationDecodeCalls"]) == (0, 0)
+    assert out["measuredTokens"] == 512 and out["measurementRepetitions"] == 2
+    names = [(m["name"], m["unit"]) for m in rec["measurements"]]
+    assert names == [("duration", "ns"), ("tokens_per_second", "tokens/s")]
+    assert rec["measurements"][1]["samples"] == [512 * 1e9 / 2.0e6, 512 * 1e9 / 4.0e6]
+    assert rec["effectiveConfiguration"]["n_prompt"] == 512 and rec["effectiveConfiguration"]["n_gen"] == 0
+    tg = evidence.llama_bench_record("llama-bench.token-generation", 0, 0, 128, 128, [1.0e8], {}, [])
+    assert tg["output"]["measuredTokens"] == 128 and tg["measurements"][1]["samples"] == [1280.0]
+    with pytest.raises(ValueError):
+        evidence.llama_bench_record("llama-bench.token-generation", 512, 1, 0, 0, [1.0], {}, [])   # wrong shape for the operation
+    with pytest.raises(ValueError):
+        evidence.llama_bench_record("llama-bench.prompt-processing", 512, 1, 0, 0, [0.0], {}, [])  # zero duration
+    with pytest.raises(ValueError):
+        evidence.llama_bench_record("decode", 1, 1, 0, 0, [1.0], {}, [])
