@@ -34,14 +34,14 @@ constexpr int LA = 256 + 16;   // activation row stride in LDS (bytes)
 constexpr int SQL = 128 + 8;   // strip row strides: conflict-free for 8-byte reads by consecutive rows
 constexpr int SQH = 64 + 8;
 
-template <int NW>
+template <int NW, int JT>   // NW waves of 32 weight rows each, JT token tiles of 32
 struct Q6Smem {
     // activations of one super-block, per token: the first eight bytes of the 16 sub-blocks, then
     // the second eight bytes of the 16 sub-blocks (a lane's operands of two neighbouring
     // sub-blocks are then one 16-byte read)
-    int8_t a[2][64 * LA];
-    int16_t bs[2][64 * 16];   // activation block sums per 16
-    float dx[2][64];
+    int8_t a[2][32 * JT * LA];
+    int16_t bs[2][32 * JT * 16];   // activation block sums per 16
+    float dx[2][32 * JT];
     uint8_t ql[NW][32 * SQL];
     uint8_t qh[NW][32 * SQH];
     int8_t sc[NW][32 * 16];
@@ -49,23 +49,24 @@ struct Q6Smem {
 
 __device__ __forceinline__ long as_i64(uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); }
 
-template <int NW>
+template <int NW, int JT>
 __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightView w, const ActView a, int64_t M,
                                                                  float *__restrict__ y) {
-    constexpr int NT = 64 * NW, TN = 32 * NW;
-    constexpr int PA = 1024 / NT;   // 16-byte activation pieces a thread moves per super-block
+    constexpr int NT = 64 * NW, TN = 32 * NW, TM = 32 * JT;
+    constexpr int PA = TM * 16 / NT;   // 16-byte activation pieces a thread moves per super-block
+    static_assert(PA >= 1 && TM * 2 <= NT, "tile does not fit the staging scheme");
     extern __shared__ __align__(16) uint8_t smem_raw[];
-    Q6Smem<NW> &sm = *reinterpret_cast<Q6Smem<NW> *>(smem_raw);
+    Q6Smem<NW, JT> &sm = *reinterpret_cast<Q6Smem<NW, JT> *>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t N = w.N, K = w.K, nb = w.nb;
     int tile_n, tile_m;
-    tile_of_workgroup((int)((N + TN - 1) / TN), (int)((M + 63) / 64), tile_n, tile_m);
-    const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * 64;
+    tile_of_workgroup((int)((N + TN - 1) / TN), (int)((M + TM - 1) / TM), tile_n, tile_m);
+    const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * TM;
     const int l32 = lane & 31, lh = lane >> 5;
 
-    v16f acc[2];
+    v16f acc[JT];
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < JT; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
 
@@ -95,7 +96,7 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
     const uint32_t scoff = (uint32_t)(myrow * (int)nb * 16);   // 32 pieces of scales: row l%32 (both halves store)
     const uint32_t doff = (uint32_t)(myrow * (int)nb);
     // activations: piece id = tid + NT*p -> token id / 16, sub-block id % 16
-    const int mrow_cap = (int)(M - 1 - m0 < 63 ? M - 1 - m0 : 63);
+    const int mrow_cap = (int)(M - 1 - m0 < TM - 1 ? M - 1 - m0 : TM - 1);
     const int8_t *abase = a.qs + m0 * K;
     uint32_t aoffg[PA];
     int aoffl[PA];
@@ -105,12 +106,12 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
         aoffg[p] = (uint32_t)((row < mrow_cap ? row : mrow_cap) * (int)K + 16 * seg);
         aoffl[p] = row * LA + 8 * seg;
     }
-    // block sums: 64 tokens x 32 bytes, thread t (mod 128) moves 16 bytes; scale: thread t (mod 64)
+    // block sums: TM tokens x 32 bytes, thread t (mod 2*TM) moves 16 bytes; scale: thread t (mod TM)
     const uint8_t *bsbase = reinterpret_cast<const uint8_t *>(a.bsums) + m0 * nb * 32;
-    const int bsrow = (tid & 127) >> 1;
+    const int bsrow = (tid & (2 * TM - 1)) >> 1;
     const uint32_t bsoffg = (uint32_t)((bsrow < mrow_cap ? bsrow : mrow_cap) * (int)nb * 32 + 16 * (tid & 1));
     const float *dxbase = a.d + m0 * nb;
-    const uint32_t dxoffg = (uint32_t)(((tid & 63) < mrow_cap ? (tid & 63) : mrow_cap) * (int)nb);
+    const uint32_t dxoffg = (uint32_t)(((tid & (TM - 1)) < mrow_cap ? (tid & (TM - 1)) : mrow_cap) * (int)nb);
 
     v4i sql[4], sqh[2], ssc, areg[PA], bsreg;
     float dxreg;
@@ -135,9 +136,9 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
             *reinterpret_cast<v2i *>(sm.a[buf] + aoffl[p]) = areg[p].xy;
             *reinterpret_cast<v2i *>(sm.a[buf] + aoffl[p] + 128) = areg[p].zw;
         }
-        // threads beyond the first 128 / 64 repeat a store of the same value: no branch, no load sunk into one
-        *reinterpret_cast<v4i *>(reinterpret_cast<uint8_t *>(sm.bs[buf]) + 16 * (tid & 127)) = bsreg;
-        sm.dx[buf][tid & 63] = dxreg;
+        // threads beyond the first 2*TM / TM repeat a store of the same value: no branch, no load sunk into one
+        *reinterpret_cast<v4i *>(reinterpret_cast<uint8_t *>(sm.bs[buf]) + 16 * (tid & (2 * TM - 1))) = bsreg;
+        sm.dx[buf][tid & (TM - 1)] = dxreg;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             *reinterpret_cast<v2i *>(pql + qlpark[c]) = sql[c].xy;
@@ -156,12 +157,12 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
     auto superblock = [&](int buf, uint32_t dbits) {
         const v4i scv = *reinterpret_cast<const v4i *>(psc + l32 * 16);   // the 16 scales of the lane's row
         const int8_t *ap = sm.a[buf] + l32 * LA + 128 * lh;
-        v16i isum[2];
+        v16i isum[JT];
         // ---- -32 * sum_s sc_s * bsum_s: block sums as 64*hi + lo against the scales of k-half l/32
         {
             const long bsc = lh ? as_i64((uint32_t)scv[2], (uint32_t)scv[3]) : as_i64((uint32_t)scv[0], (uint32_t)scv[1]);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
+            for (int j = 0; j < JT; ++j) {
                 const v4i b = *reinterpret_cast<const v4i *>(reinterpret_cast<const uint8_t *>(sm.bs[buf]) +
                                                            (j * 32 + l32) * 32 + 16 * lh);
                 uint32_t lo[4], hi[4];
@@ -206,7 +207,7 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
                 const int s0 = (int)(int8_t)((uint32_t)scv[sb0 >> 2] >> (8 * (sb0 & 3)));
                 const int s1 = (int)(int8_t)((uint32_t)scv[(sb0 + 1) >> 2] >> (8 * ((sb0 + 1) & 3)));
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
+                for (int j = 0; j < JT; ++j) {
                     const v4i av = *reinterpret_cast<const v4i *>(ap + j * 32 * LA + 8 * sb0);
                     const v16i i0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64((uint32_t)av[0], (uint32_t)av[1]),
                                                                           as_i64(wl[0][k], wh[0][k]), zi, 0, 0, 0);
@@ -222,7 +223,7 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
         const float dn = h2f(dbits);
         const float *dxs = sm.dx[buf];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < JT; ++j) {
             float dxv[16];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -252,7 +253,7 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
     const int64_t n = n0 + wave * 32 + l32;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < JT; ++j) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
@@ -264,14 +265,15 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
 }  // namespace
 
 namespace {
-template <int NW>
+template <int NW, int JT>
 hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
-    using Smem = Q6Smem<NW>;
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q6k_q8k_kernel<NW>),
+    using Smem = Q6Smem<NW, JT>;
+    const auto kern = &gemm_q6k_q8k_kernel<NW, JT>;
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
     if (attr != hipSuccess) return attr;
-    const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64)));
-    hipLaunchKernelGGL(gemm_q6k_q8k_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, w, a, M, y);
+    const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 32 * JT - 1) / (32 * JT))));
+    hipLaunchKernelGGL(kern, grid, dim3(64 * NW), sizeof(Smem), s, w, a, M, y);
     return hipGetLastError();
 }
 }  // namespace
@@ -279,9 +281,10 @@ hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y
 // ggml-format activations (Q8_K planes in `a`), Q6_K weights, any M
 hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
     if (w.type != kTypeQ6_K || a.kind != kActKindQ8_K || !a.bsums || M <= 0) return hipErrorInvalidValue;
-    // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit (64 x 64 tiles for
-    // grids that leave compute units idle were measured slower: 0.30 against 0.25 ms at M=512)
-    return launch_q6k<4>(w, a, M, y, s);
+    // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit; 32-token tiles when
+    // the grid of 64-token tiles would leave compute units idle
+    if (((w.N + 127) / 128) * ((M + 63) / 64) >= 384) return launch_q6k<4, 2>(w, a, M, y, s);
+    return launch_q6k<4, 1>(w, a, M, y, s);
 }
 
 }  // namespace qproj

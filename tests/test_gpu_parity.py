@@ -393,7 +393,7 @@ def test_full_size_against_device_fp64_of_proven_parts(ctx, qtype, k, n):
     w = ctx.upload_from_device(qtype, k, n, blocks)
     wd = ctx.dequantize(w).double()
     g = torch.Generator(device="cuda").manual_seed(1)
-    for m in (1, 4, 16, 192, 512):   # 192 and 512 take the 64- and the 128-token tiles of the Q4_K prefill kernel
+    for m in (1, 4, 16, 192, 1024):   # 192 and 1024: the 32- and the 64-token tiles of the Q6_K prefill kernel
         x = torch.randn((m, k), generator=g, device="cuda", dtype=torch.float32)
         y = ctx.mul_mat(w, x, ACT_GGML)
         a = ctx.quantize_activations(x, ACT_GGML, qtype)
