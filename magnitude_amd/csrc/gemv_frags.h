@@ -230,8 +230,10 @@ template <> struct Dot<kTypeQ4_K> {
             sl = dot4(f.lo[i], xl[i], sl);
             sh = dot4(f.hi[i], xh[i], sh);
         }
-        const int isum = f.sc0 * sl + f.sc1 * sh;
-        const int msum = f.m0 * bl + f.m1 * bh;
+        // every factor fits 24 bits (6-bit scales and mins, sums of 32 products of a nibble and an int8):
+        // the full-rate 24-bit multiply instead of the quarter-rate 32-bit one
+        const int isum = __mul24(f.sc0, sl) + __mul24(f.sc1, sh);
+        const int msum = __mul24(f.m0, bl) + __mul24(f.m1, bh);
         return fmaf(f.d * xd, (float)isum, -((f.dmin * xd) * (float)msum));
     }
 };
@@ -259,7 +261,7 @@ template <> struct Dot<kTypeQ6_K> {
             int s = 0;
 #pragma unroll
             for (int t = 0; t < 4; ++t) s = dot4(f.q[g][t], xg[g][t], s);
-            isum += f.sc[g] * (s - 32 * bs[g]);  // weights are stored +32
+            isum += __mul24(f.sc[g], s - 32 * bs[g]);  // weights are stored +32; both factors fit 24 bits
         }
         return (f.d * xd) * (float)isum;
     }

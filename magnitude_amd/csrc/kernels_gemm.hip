@@ -484,6 +484,7 @@ hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, f
 // ggml-format activations (Q8_K planes in `a`, including the min-term plane), Q4_K weights, any M
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
     if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || !a.msum || M <= 0) return hipErrorInvalidValue;
+    if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 64 token rows of K bytes, 32 weight rows of K*144/256
     constexpr int NW = 4;   // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit
     using Smem = DirectSmem<NW>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_direct_kernel<NW>),

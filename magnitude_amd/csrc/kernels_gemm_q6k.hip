@@ -281,6 +281,7 @@ hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y
 // ggml-format activations (Q8_K planes in `a`), Q6_K weights, any M
 hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
     if (w.type != kTypeQ6_K || a.kind != kActKindQ8_K || !a.bsums || M <= 0) return hipErrorInvalidValue;
+    if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 64 token rows of K bytes, 32 weight rows of K/2
     // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit; 32-token tiles when
     // the grid of 64-token tiles would leave compute units idle
     if (((w.N + 127) / 128) * ((M + 63) / 64) >= 384) return launch_q6k<4, 2>(w, a, M, y, s);
