@@ -367,9 +367,11 @@ def main():
                           "headline_tops": head["gemm_tops"], "headline_frac_int8_peak": head["frac_int8_peak"],
                           "peak_tops": INT8_PEAK_TOPS, "shapes": res}
         # the same shapes in the ggml activation format (Q8_K, one scale per 256): the reference's own arithmetic
-        # (plus the layer's Q6_K down projection, which a Q4_K_M model runs through the same operator)
+        # (plus the layer's Q6_K down projection, which a Q4_K_M model runs through the same operator, and
+        # config 1's Q8_0 matrix with ggml's Q8_0 activation blocks)
         resg = []
-        for (qt, k, n) in ((Q4_K, 4096, 14336), (Q4_K, 14336, 4096), (Q4_K, 4096, 4096), (Q6_K, 14336, 4096)):
+        for (qt, k, n) in ((Q4_K, 4096, 14336), (Q4_K, 14336, 4096), (Q4_K, 4096, 4096), (Q6_K, 14336, 4096),
+                           (Q8_0, 4096, 4096)):
             blocks = synth.random_weight(qt, n, k, seed=77 + n, device=dev)
             w = ctx.upload_from_device(qt, k, n, blocks)
             del blocks
@@ -391,7 +393,7 @@ def main():
                                                         bytes_moved=gguf_bytes(qt, n, k) + m * k * 4 + m * n * 4,
                                                         memory_kb=(gguf_bytes(qt, n, k) + m * n * 4) // 1024,
                                                         device=props.name))
-                tname = "Q4_K" if qt == Q4_K else "Q6_K"
+                tname = {Q4_K: "Q4_K", Q6_K: "Q6_K", Q8_0: "Q8_0"}[qt]
                 resg.append({"type": tname, "M": m, "K": k, "N": n, "gemm_ms": tg, "quantize_ms": tq,
                              "gemm_tops": ops / (tg * 1e-3) / 1e12,
                              "frac_int8_peak": ops / (tg * 1e-3) / 1e12 / INT8_PEAK_TOPS})
@@ -402,7 +404,8 @@ def main():
         headg = [r for r in resg if (r["type"], r["M"], r["K"], r["N"]) == ("Q4_K", 4096, 4096, 14336)][0]
         out["prefill_ggml_acts"] = {"act_format": "ggml Q8_K (int8 + fp32 scale per 256, block sums)",
                                     "mfma": "Q4_K: 2 x v_mfma_i32_32x32x32_i8 per sub-block (scale split in base 8); "
-                                            "Q6_K: v_mfma_i32_32x32x16_i8 per sub-block, integer scale on the vector ALU",
+                                            "Q6_K: v_mfma_i32_32x32x16_i8 per sub-block, integer scale on the vector ALU; "
+                                            "Q8_0: v_mfma_i32_32x32x32_i8 per block, fp32 scales",
                                     "headline_tops": headg["gemm_tops"], "headline_frac_int8_peak": headg["frac_int8_peak"],
                                     "shapes": resg}
 

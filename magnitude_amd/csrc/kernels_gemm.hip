@@ -46,7 +46,7 @@ struct GemmSmem {
 // registers one thread carries from global memory to LDS for one K-step
 struct StageRegs {
     uint4 act[2];
-    uint4 wq;
+    uint4 wq, wq2;   // wq2: Q8_0 only (its rows are 128 bytes per K-step, Q4_K's 64)
     float4 ad;  // threads 0..127: activation scales; threads 128..255: block header of a weight row
 };
 
@@ -57,8 +57,13 @@ __device__ __forceinline__ void split_h(float v, _Float16 &hi, _Float16 &lo) {
 
 constexpr int kGemmThreads = 512;
 
-__global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const WeightView w, const ActView a, int64_t M,
-                                                               float *__restrict__ y) {
+// QT = Q4_K: per-32 int8 activations with fp32 scales and block sums (the prefill format).
+// QT = Q8_0: ggml's Q8_0 activation blocks against Q8_0 weights: the same product without nibbles,
+// without a min term, and with a weight scale per 32 instead of d*sc per sub-block.
+template <int QT>
+__global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const WeightView w, const ActView a, int64_t M,
+                                                                   float *__restrict__ y) {
+    constexpr bool kQ4 = QT == kTypeQ4_K;
     extern __shared__ __align__(16) uint8_t smem_raw[];
     GemmSmem &sm = *reinterpret_cast<GemmSmem *>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -86,7 +91,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
 
     // ---------------------------------------------------------------- min term on the fp16 cores
     // acc = -(1/prescale) * sum_kb A[m][kb] * B[n][kb] is built as +sum with negated B and scaled later
-    {
+    if constexpr (kQ4) {
         const int64_t n_steps = (kb32 + 15) / 16;  // 16 sub-blocks = two super-blocks per product
         for (int64_t s = 0; s < n_steps; ++s) {
             v8h ah, al, bh[2], bl[2];
@@ -151,21 +156,34 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
             r.act[i] = make_uint4(0, 0, 0, 0);
             if (m < M) r.act[i] = *reinterpret_cast<const uint4 *>(a.qs + m * K + k0 + 16 * seg);
         }
-        {  // weights: 128 rows x 64 packed bytes (two 64-weight chunks of the super-block)
+        if constexpr (kQ4) {  // weights: 128 rows x 64 packed bytes (two 64-weight chunks of the super-block)
             const int row = tid >> 2, part = tid & 3;
             int64_t n = n0 + row;
             if (n >= N) n = N - 1;
             const int c2 = (int)((k0 & 255) >> 5);  // 32-byte chunk pair index * 2
             const uint8_t *blk = w.q4k + (n * w.nb + (k0 >> 8)) * 144 + 16 + 16 * c2 + 16 * part;
             r.wq = *reinterpret_cast<const uint4 *>(blk);
+        } else {              // weights: 128 rows x 128 int8
+            const int row = tid >> 2, part = tid & 3;
+            int64_t n = n0 + row;
+            if (n >= N) n = N - 1;
+            const int8_t *src = w.q8_qs + n * K + k0 + 32 * part;
+            r.wq = *reinterpret_cast<const uint4 *>(src);
+            r.wq2 = *reinterpret_cast<const uint4 *>(src + 16);
         }
         r.ad = make_float4(0.f, 0.f, 0.f, 0.f);
         if (tid < BM) {
             if (m0 + tid < M) r.ad = *reinterpret_cast<const float4 *>(a.d + (m0 + tid) * kb32 + (k0 >> 5));
-        } else if (tid < BM + BN && (k0 & 255) == 0) {  // a new super-block starts: its header
+        } else if (tid < BM + BN && (!kQ4 || (k0 & 255) == 0)) {
             int64_t n = n0 + (tid - BM);
             if (n >= N) n = N - 1;
-            r.ad = *reinterpret_cast<const float4 *>(w.q4k + (n * w.nb + (k0 >> 8)) * 144);
+            if constexpr (kQ4) {   // a new super-block starts: its header
+                r.ad = *reinterpret_cast<const float4 *>(w.q4k + (n * w.nb + (k0 >> 8)) * 144);
+            } else {               // the four fp16 scales of this K-step
+                const uint2 d4 = *reinterpret_cast<const uint2 *>(w.q8_d + n * w.nb + (k0 >> 5));
+                r.ad.x = __uint_as_float(d4.x);
+                r.ad.y = __uint_as_float(d4.y);
+            }
         }
     };
     auto store_stage = [&](const StageRegs &r, GemmStage &st, int64_t k0) {
@@ -175,7 +193,11 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
             const int row = idx >> 3, seg = idx & 7;
             *reinterpret_cast<uint4 *>(st.a + row * LDT + 16 * seg) = r.act[i];
         }
-        {
+        if constexpr (!kQ4) {
+            const int row = tid >> 2, part = tid & 3;
+            *reinterpret_cast<uint4 *>(st.b + row * LDT + 32 * part) = r.wq;
+            *reinterpret_cast<uint4 *>(st.b + row * LDT + 32 * part + 16) = r.wq2;
+        } else {
             // 16 packed bytes = bytes 16*(part&1).. of chunk (part>>1): low nibbles -> sub-block 2c, high -> 2c+1
             const int row = tid >> 2, part = tid & 3, ch = part >> 1, half = part & 1;
             int8_t *base = st.b + row * LDT + 64 * ch + 16 * half;
@@ -188,13 +210,22 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
             st.a_d[1][tid] = r.ad.y;
             st.a_d[2][tid] = r.ad.z;
             st.a_d[3][tid] = r.ad.w;
-        } else if (tid < BM + BN && (k0 & 255) == 0) {
-            const uint32_t h0 = __float_as_uint(r.ad.x);
-            const ScalesK4 sc = unpack_scales_k4(__float_as_uint(r.ad.y), __float_as_uint(r.ad.z), __float_as_uint(r.ad.w));
-            const float d = h2f(h0);
-            float *dst = &sm.w_s[0][tid - BM];
+        } else if (tid < BM + BN && (!kQ4 || (k0 & 255) == 0)) {
+            if constexpr (kQ4) {
+                const uint32_t h0 = __float_as_uint(r.ad.x);
+                const ScalesK4 sc = unpack_scales_k4(__float_as_uint(r.ad.y), __float_as_uint(r.ad.z), __float_as_uint(r.ad.w));
+                const float d = h2f(h0);
+                float *dst = &sm.w_s[0][tid - BM];
 #pragma unroll
-            for (int t = 0; t < 8; ++t) dst[t * BN] = d * (float)scale_k4(sc, t);
+                for (int t = 0; t < 8; ++t) dst[t * BN] = d * (float)scale_k4(sc, t);
+            } else {   // scale slots 0..3 and 4..7 alternate with the K-steps, like the operand stages
+                const uint32_t lo = __float_as_uint(r.ad.x), hi = __float_as_uint(r.ad.y);
+                float *dst = &sm.w_s[(int)((k0 / BK) & 1) * 4][tid - BM];
+                dst[0] = h2f(lo & 0xffffu);
+                dst[BN] = h2f(lo >> 16);
+                dst[2 * BN] = h2f(hi & 0xffffu);
+                dst[3 * BN] = h2f(hi >> 16);
+            }
         }
     };
 
@@ -208,7 +239,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
         const int64_t k0 = ks * BK;
         const GemmStage &st = sm.st[ks & 1];
         if (ks + 1 < n_ksteps) load_stage(regs, k0 + BK);  // in flight during the arithmetic below
-        const float *wsp = &sm.w_s[(k0 & 255) >> 5][wn * 64 + l32];
+        const float *wsp = &sm.w_s[kQ4 ? (int)((k0 & 255) >> 5) : (int)(ks & 1) * 4][wn * 64 + l32];
 #pragma unroll 1
         for (int kb = 0; kb < 4; ++kb) {
             const v4i af = *reinterpret_cast<const v4i *>(st.a + (wm * 32 + l32) * LDT + kb * 32 + 16 * lh);
@@ -232,7 +263,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_q4k_q8x32_kernel(const W
             for (int v = 0; v < 16; ++v) acc[1][v] = fmaf((float)I1[v], ad[v] * w1, acc[1][v]);
         }
         // the next step starts a new super-block: its scales replace the ones other waves may still read
-        if (((k0 + BK) & 255) == 0) __syncthreads();
+        if (kQ4 && ((k0 + BK) & 255) == 0) __syncthreads();
         if (ks + 1 < n_ksteps) store_stage(regs, sm.st[(ks + 1) & 1], k0 + BK);
         __syncthreads();
     }
@@ -473,11 +504,24 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const W
 
 hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
     if (w.type != kTypeQ4_K || w.K % 256 != 0 || M <= 0) return hipErrorInvalidValue;
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8x32_kernel),
+    const auto kern = &gemm_per32_kernel<kTypeQ4_K>;
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem));
     if (attr != hipSuccess) return attr;
     const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + BM - 1) / BM)));
-    hipLaunchKernelGGL(gemm_q4k_q8x32_kernel, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y);
+    hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y);
+    return hipGetLastError();
+}
+
+// Q8_0 weights x ggml Q8_0 activation blocks (planes in `a`), K a multiple of 128
+hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
+    if (w.type != kTypeQ8_0 || a.kind != kActKindQ8_0 || w.K % BK != 0 || M <= 0) return hipErrorInvalidValue;
+    const auto kern = &gemm_per32_kernel<kTypeQ8_0>;
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem));
+    if (attr != hipSuccess) return attr;
+    const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + BM - 1) / BM)));
+    hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y);
     return hipGetLastError();
 }
 

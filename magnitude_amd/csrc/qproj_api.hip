@@ -272,12 +272,16 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
     const auto tiled = [&](const qproj_weight *t) {
         if (M < gemm_min_m) return false;
         if (t->type == kTypeQ4_K) return true;
+        if (t->type == kTypeQ8_0) return t->K % 128 == 0 && M >= 64;
         return t->type == kTypeQ6_K && (M >= 112 || ((M + 63) / 64) * ((t->N + 127) / 128) >= 128);
     };
     if (tiled(w[0])) {
-        for (int i = 0; i < n; ++i)
-            QP_HIP(ctx, w[0]->type == kTypeQ4_K ? launch_gemm_q8k(w[i]->view, a, M, y[i], ctx->stream)
-                                                : launch_gemm_q6k_q8k(w[i]->view, a, M, y[i], ctx->stream));
+        for (int i = 0; i < n; ++i) {
+            const int t = w[0]->type;
+            QP_HIP(ctx, t == kTypeQ4_K   ? launch_gemm_q8k(w[i]->view, a, M, y[i], ctx->stream)
+                        : t == kTypeQ6_K ? launch_gemm_q6k_q8k(w[i]->view, a, M, y[i], ctx->stream)
+                                         : launch_gemm_q8_0(w[i]->view, a, M, y[i], ctx->stream));
+        }
         return QPROJ_OK;
     }
     if (use_mfma_kernel(w[0]->type, M, w[0]->K)) {

@@ -100,6 +100,7 @@ hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, i
 hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
 // Q4_K weights x ggml Q8_K activations (`a`), large M
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
+hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
 hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
 
 }  // namespace qproj

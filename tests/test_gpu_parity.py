@@ -204,12 +204,13 @@ def test_mul_mat_ggml_mode_matches_oracle(ctx, orc, qtype, m):
         w.free()
 
 
-@pytest.mark.parametrize("qtype", [Q4_K, Q6_K])
+@pytest.mark.parametrize("qtype", [Q4_K, Q6_K, Q8_0])
 @pytest.mark.parametrize("m,k,n", [(48, 4096, 256), (130, 768, 203), (200, 14336, 128), (333, 256, 40)])
 def test_mul_mat_ggml_mode_prefill_sized_batches(ctx, orc, qtype, m, k, n):
     """Large M in the ggml activation format: the prefill matrix-core kernels (Q4_K: two int8 chains
-    per super-block; Q6_K: one K=16 product per sub-block, integer scale on the vector ALU) against
-    the oracle's integer arithmetic with Q8_K activations, ragged M and N included."""
+    per super-block; Q6_K: one K=16 product per sub-block, integer scale on the vector ALU; Q8_0: one
+    product per block of 32, both scales applied in fp32) against the oracle's integer arithmetic
+    with ggml's activation blocks, ragged M and N included."""
     from magnitude_amd import ACT_GGML
     blocks = make_weight(orc, qtype, n, k, seed=1500 + k + n)
     rng = np.random.default_rng(m + k)
