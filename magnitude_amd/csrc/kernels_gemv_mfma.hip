@@ -28,6 +28,7 @@
 
 #include "qproj_device.h"
 #include "qproj_internal.h"
+#include "actquant_device.h"
 
 namespace qproj {
 
@@ -49,6 +50,7 @@ struct MfmaArgs {
     int n_targets;
     MfmaTarget t[kMaxTargets];
     ActView a;
+    const float *x;        // non-null: fp32 activation rows [rows][K], quantized by every workgroup in its prologue
     int M, n_chunks, chunk_sb, kw, rw, n_wgs;
     // expert-grouped mode (MUL_MAT_ID): activation rows of expert e are the pairs order[offsets[e]..offsets[e+1])
     const int32_t *order;
@@ -427,6 +429,61 @@ __device__ __forceinline__ void stage_activations(const MfmaArgs &g, uint8_t *sm
     }
 }
 
+// The same LDS image made from fp32 rows: each wave quantizes whole 256-element chunks (ggml's
+// quantize_row_q8_K, or eight quantize_row_q8_0 blocks for Q8_0 weights) exactly as the standalone
+// quantizer kernels do, so both routes stage identical bytes.  Two chunks are in flight per wave.
+template <int QT, int MT, int kThreads, bool MAPPED>
+__device__ __forceinline__ void stage_quantize(const MfmaArgs &g, uint8_t *smem, const Layout &L, int c0, int nsb,
+                                               int n_rows, int m0) {
+    constexpr int NWAVES = kThreads / 64;
+    const int lane = threadIdx.x & 63, wave = uniform(threadIdx.x >> 6);
+    const int *map = reinterpret_cast<const int *>(smem + L.off_map);
+    auto src_row = [&](int m) -> size_t { return MAPPED ? (size_t)(map[m] / g.x_div) : (size_t)(m0 + m); };
+    float *dxs = reinterpret_cast<float *>(smem + L.off_dx);
+    const int total = n_rows * nsb;
+    for (int base = 0; base < total; base += 2 * NWAVES) {
+        float4 v[2];
+        int mm[2], ss[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int idx = min(base + u * NWAVES + wave, total - 1);
+            mm[u] = idx / nsb;
+            ss[u] = idx - mm[u] * nsb;
+            v[u] = *reinterpret_cast<const float4 *>(g.x + src_row(mm[u]) * (size_t)g.a.K + (size_t)(c0 + ss[u]) * 256 + 4 * lane);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            if (base + u * NWAVES + wave >= total) continue;   // wave-uniform
+            const int m = mm[u], sb = ss[u];
+            uint32_t *dst = reinterpret_cast<uint32_t *>(smem + m * L.lda + sb * 256 + 4 * lane);
+            if constexpr (QT == kTypeQ8_0) {
+                int s;
+                float dd;
+                *dst = wave_quantize_q8_32(v[u], s, dd);
+                if ((lane & 7) == 0) dxs[(sb * 8 + (lane >> 3)) * MT + m] = h2f(f2h(dd));
+            } else {
+                int bsum;
+                float dd;
+                *dst = wave_quantize_q8k(v[u], lane, bsum, dd);
+                if (lane == 0) dxs[sb * MT + m] = dd;
+                uint8_t *aux = smem + L.off_aux + (sb * MT + m) * Cfg<QT>::kAux;
+                if constexpr (QT == kTypeQ4_K) {   // sums of 32: bytes 0..7 high parts, 8..15 low parts
+                    const int s32 = bsum + __shfl_xor(bsum, 4);
+                    if ((lane & 7) == 0) {
+                        aux[lane >> 3] = (uint8_t)((s32 >> 6) & 0xff);
+                        aux[8 + (lane >> 3)] = (uint8_t)(s32 & 63);
+                    }
+                } else {                           // sums of 16: bytes 0..15 high parts, 16..31 low parts
+                    if ((lane & 3) == 0) {
+                        aux[lane >> 2] = (uint8_t)((bsum >> 6) & 0xff);
+                        aux[16 + (lane >> 2)] = (uint8_t)(bsum & 63);
+                    }
+                }
+            }
+        }
+    }
+}
+
 constexpr int kDense = 0, kGrouped = 1, kGroupedSwiglu = 2;
 
 // MODE kDense: y[m][n] for the M rows of `a`.  kGrouped: the workgroup's expert e multiplies its
@@ -516,7 +573,10 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
                 map[threadIdx.x] = (int)threadIdx.x < m_cnt ? g.order[pair0 + m0 + (int)threadIdx.x] : 0;
             __syncthreads();
         }
-        stage_activations<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
+        if (g.x)
+            stage_quantize<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
+        else
+            stage_activations<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
         __syncthreads();
 
         float out[NT][NV];
@@ -679,6 +739,7 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s)
     MfmaArgs g{};
     g.n_targets = args.n_targets;
     g.a = args.a;
+    g.x = args.x;
     g.M = args.M;
     g.x_div = 1;
     int64_t total_rg = 0;
@@ -712,6 +773,7 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
     MfmaArgs g{};
     g.n_targets = swiglu ? 2 : 1;
     g.a = args.a;
+    g.x = args.x;
     g.M = 0;
     g.order = args.order;
     g.offsets = args.offsets;

@@ -263,8 +263,18 @@ size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
     return need;
 }
 
+// true when mul_mat of M fp32 rows goes to the small-batch kernel with the quantizer fused into its
+// prologue.  Off unless asked for: every one of the ~200 workgroups repeats the quantization of all M
+// rows, which costs more than the separate quantizer launch saves (gate+up, M = 4 / 8 / 16: 22.1 /
+// 26.9 / 38.5 us fused against 20.5 / 20.8 / 22.7 us).
+bool dense_fuses_quantizer(const qproj_weight *w, int64_t M) {
+    static const bool on = getenv("QPROJ_FUSED_QUANT_DENSE") && atoi(getenv("QPROJ_FUSED_QUANT_DENSE"));
+    return on && M <= 16 && use_mfma_kernel(w->type, M, w->K);
+}
+
+// x_f32: non-null when `a` carries no planes and the kernel quantizes these rows itself (small batches only)
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
-                    float *const *y, float *scratch) {
+                    float *const *y, float *scratch, const float *x_f32 = nullptr) {
     static const int gemm_min_m = getenv("QPROJ_GEMM_MIN_M") ? atoi(getenv("QPROJ_GEMM_MIN_M")) : 48;
     // prefill-sized batches: tiled product, weights reused across 64 tokens.  The Q6_K kernel is slow
     // per workgroup (a vector multiply-add per output and sub-block): below 128 tiles of 64 x 128 it
@@ -293,7 +303,8 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
                 g.t[i].w = w[i]->view;
                 g.t[i].y = y[i] + m0 * w[i]->N;
             }
-            g.a = act_rows(a, m0);
+            g.a = x_f32 ? a : act_rows(a, m0);
+            g.x = x_f32;   // (only with M <= 16: a single pass)
             g.M = (int)mc;
             g.x_div = 1;
             QP_HIP(ctx, launch_gemv_mfma(g, scratch, ctx->stream));
@@ -327,6 +338,14 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
         QP_HIP(ctx, launch_gemv_q8act(g, pow2_ceil(mc), 1, ctx->stream));
     }
     return QPROJ_OK;
+}
+
+// the grouped matrix-core kernel quantizes its own activation rows when an expert has few of them
+// (every workgroup of the expert repeats that work): two launches less per MoE layer, 40.5 -> 33.7 us
+// at one token, 73 -> 68 us at eight, no difference any more at four pairs an expert
+bool grouped_fuses_quantizer(int type, int64_t K, int64_t n_pairs, int64_t E) {
+    static const bool on = !(getenv("QPROJ_NO_FUSED_QUANT") && atoi(getenv("QPROJ_NO_FUSED_QUANT")));
+    return on && use_mfma_grouped(type, K) && n_pairs <= 2 * E;
 }
 
 int grouped_mt(int64_t n_pairs, int64_t E) {
@@ -545,6 +564,14 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
     if (act == kActGGML || act == kActQ8X32) {
         if (act == kActQ8X32 && w[0]->type != kTypeQ4_K)
             return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat: the per-32 int8 path is built for Q4_K weights");
+        if (act == kActGGML && dense_fuses_quantizer(w[0], M)) {
+            int rc = ensure_ws(ctx, dense_scratch_bytes(n, w, M));
+            if (rc) return rc;
+            ActView a{};
+            a.kind = act_kind_for(act, w[0]->type);
+            a.K = K;
+            return run_dense_q8act(ctx, n, w, a, M, y_dev, reinterpret_cast<float *>(ctx->ws), x_dev);
+        }
         const ActPlanes p = act_planes(act_kind_for(act, w[0]->type), M, K);
         const size_t extra = act == kActGGML ? dense_scratch_bytes(n, w, M) : 0;
         int rc = ensure_ws(ctx, p.total + extra);
@@ -625,7 +652,9 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     const size_t total = off_active + align_up((size_t)(w->E + 1) * 4);
     int rc = ensure_ws(ctx, total);
     if (rc) return rc;
-    QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, rows, K));
+    // few pairs an expert: the grouped kernel quantizes the rows it needs in its prologue
+    const bool fuse = grouped_fuses_quantizer(w->type, K, n_pairs, w->E);
+    if (!fuse) QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, rows, K));
     int32_t *order = reinterpret_cast<int32_t *>(ctx->ws + off_order);
     int32_t *offsets = reinterpret_cast<int32_t *>(ctx->ws + off_offsets);
     int32_t *active = reinterpret_cast<int32_t *>(ctx->ws + off_active);
@@ -635,6 +664,7 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     g.t[0].w = w->view;
     g.t[0].y = y_dev;
     g.a = act_view(p, ctx->ws, K);
+    g.x = fuse ? x_dev : nullptr;
     g.order = order;
     g.offsets = offsets;
     g.active = active;
@@ -687,7 +717,9 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     float *e = reinterpret_cast<float *>(ws + off_e);
     const int mt = grouped_mt(n_pairs, E);
 
-    QP_HIP(ctx, run_quantize(ctx, px, ws, x_dev, B, d_model));
+    const bool fuse_x = grouped_fuses_quantizer(gate->type, d_model, n_pairs, E);
+    const bool fuse_h = grouped_fuses_quantizer(down->type, d_ff, n_pairs, E);
+    if (!fuse_x) QP_HIP(ctx, run_quantize(ctx, px, ws, x_dev, B, d_model));
     QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, E, order, offsets, active, ctx->flag_dev, ctx->stream));
     GemvArgs g{};
     g.n_targets = 2;
@@ -696,6 +728,7 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     g.t[1].w = up->view;
     g.t[1].y = h;
     g.a = act_view(px, ws, d_model);
+    g.x = fuse_x ? x_dev : nullptr;
     g.order = order;
     g.offsets = offsets;
     g.active = active;
@@ -704,12 +737,13 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
         QP_HIP(ctx, launch_gemv_mfma_grouped(g, n_pairs, true, ctx->stream));
     else
         QP_HIP(ctx, launch_moe_swiglu_gemv(g, mt, (int)E, ctx->stream));
-    QP_HIP(ctx, run_quantize(ctx, ph, ws + off_hq, h, n_pairs, d_ff));
+    if (!fuse_h) QP_HIP(ctx, run_quantize(ctx, ph, ws + off_hq, h, n_pairs, d_ff));
     GemvArgs gd{};
     gd.n_targets = 1;
     gd.t[0].w = down->view;
     gd.t[0].y = e;
     gd.a = act_view(ph, ws + off_hq, d_ff);
+    gd.x = fuse_h ? h : nullptr;
     gd.order = order;
     gd.offsets = offsets;
     gd.active = active;
