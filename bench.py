@@ -430,8 +430,8 @@ def main():
             f(); ctx.sync()
             run = (None if args.no_graph else capture(torch, stream, f)) or f
             run(); torch.cuda.synchronize()
-            sm_ = timer.samples_ms(run, 20)
-            ms = sum(sm_) / len(sm_)
+            sm_ = timer.samples_ms(run, 20)          # raw samples for the records (an event pair around each call)
+            ms = timer.time_ms(run, 100)             # the figure: 100 calls back to back between one event pair
             byts = distinct * per_expert + B * dm * 4 * 2
             ev_rows.append(evidence.backend_ops_row("MUL_MAT_ID", evidence.mul_mat_id_params(Q4_K, dff, dm, E, top, B) +
                                                     ",fused=moe_ffn(gate,up,swiglu,down,combine)", [s * 1e3 for s in sm_],
@@ -442,7 +442,9 @@ def main():
                         "frac_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
             log(f"[bench] moe B={B}: {ms * 1e3:.1f} us, {distinct} experts, {res[-1]['GBps']:.0f} GB/s")
         out["moe"] = {"experts": E, "top": top, "d_model": dm, "d_ff": dff, "batches": res,
-                      "note": "6 launches per call (quantize, group, gate/up+SwiGLU, quantize, down, combine), replayed as a HIP graph; "
+                      "note": "3 to 6 launches per call ([quantize,] [group,] gate/up+SwiGLU, [quantize,] down, combine: the grouped "
+                              "kernel quantizes its own rows when experts have few pairs, and skips the grouping pass for "
+                              "up to 16 pairs), replayed as a HIP graph, 100 calls back to back; "
                               "the same experts every replay, so weights may sit in the Infinity Cache"}
         for w in exps.values():
             w.free()

@@ -59,6 +59,10 @@ struct MfmaArgs {
     int n_expert;
     int x_div;             // activation row of pair p is p / x_div
     int wgs_per_expert;
+    // pair mode (ids non-null): workgroup set s serves pair s alone with expert ids[s]; no order / offsets / active
+    const int32_t *ids;
+    int n_pairs;
+    int32_t *error_flag;
 };
 
 template <int QT>
@@ -506,11 +510,22 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
     if constexpr (GROUPED) {
         const int slot = (int)blockIdx.x / g.wgs_per_expert;   // the grid covers min(E, pairs) experts
         rs = (int)blockIdx.x - slot * g.wgs_per_expert;
-        if (slot >= g.active[g.n_expert]) return;
-        expert = g.active[slot];
-        pair0 = g.offsets[expert];
-        n_rows = g.offsets[expert + 1] - pair0;
-        if (n_rows <= 0) return;
+        if (g.ids) {   // a workgroup set per pair
+            if (slot >= g.n_pairs) return;
+            expert = g.ids[slot];
+            if (expert < 0 || expert >= g.n_expert) {   // the pair is left out, as the grouping pass would
+                if (rs == 0 && threadIdx.x == 0) atomicOr(g.error_flag, 1);
+                return;
+            }
+            pair0 = slot;
+            n_rows = 1;
+        } else {
+            if (slot >= g.active[g.n_expert]) return;
+            expert = g.active[slot];
+            pair0 = g.offsets[expert];
+            n_rows = g.offsets[expert + 1] - pair0;
+            if (n_rows <= 0) return;
+        }
     } else {
         int ti = 0;
 #pragma unroll
@@ -570,7 +585,9 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
         if constexpr (GROUPED) {
             if (m0 > 0) __syncthreads();   // the previous pass is done with the staged rows and the regions
             if ((int)threadIdx.x < MT)
-                map[threadIdx.x] = (int)threadIdx.x < m_cnt ? g.order[pair0 + m0 + (int)threadIdx.x] : 0;
+                map[threadIdx.x] = (int)threadIdx.x >= m_cnt ? 0
+                                   : g.ids      ? pair0 + m0 + (int)threadIdx.x
+                                                : g.order[pair0 + m0 + (int)threadIdx.x];
             __syncthreads();
         }
         if (g.x)
@@ -800,7 +817,10 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
     }
     g.wgs_per_expert = (int)((rg_e + g.rw - 1) / g.rw);
     g.n_expert = (int)w.E;
-    g.n_wgs = (int)(std::min<int64_t>(w.E, n_pairs) * g.wgs_per_expert);
+    g.ids = args.ids;
+    g.n_pairs = args.n_pairs;
+    g.error_flag = args.error_flag;
+    g.n_wgs = (int)((args.ids ? n_pairs : std::min<int64_t>(w.E, n_pairs)) * g.wgs_per_expert);
     if (swiglu) return launch_typed<kGroupedSwiglu>(g, type, small, W, s);
     return launch_typed<kGrouped>(g, type, small, W, s);
 }

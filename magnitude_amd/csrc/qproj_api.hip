@@ -348,6 +348,13 @@ bool grouped_fuses_quantizer(int type, int64_t K, int64_t n_pairs, int64_t E) {
     return on && use_mfma_grouped(type, K) && n_pairs <= 2 * E;
 }
 
+// a handful of pairs (one or two decode tokens): no grouping pass, a set of workgroups per pair; an expert
+// that does come twice is simply read twice
+bool grouped_pair_mode(int type, int64_t K, int64_t n_pairs, int64_t E) {
+    static const bool on = !(getenv("QPROJ_NO_PAIR_MODE") && atoi(getenv("QPROJ_NO_PAIR_MODE")));
+    return on && grouped_fuses_quantizer(type, K, n_pairs, E) && n_pairs <= 16;
+}
+
 int grouped_mt(int64_t n_pairs, int64_t E) {
     if (n_pairs * 4 <= E) return 1;
     if (n_pairs <= E) return 2;
@@ -658,11 +665,18 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     int32_t *order = reinterpret_cast<int32_t *>(ctx->ws + off_order);
     int32_t *offsets = reinterpret_cast<int32_t *>(ctx->ws + off_offsets);
     int32_t *active = reinterpret_cast<int32_t *>(ctx->ws + off_active);
-    QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, w->E, order, offsets, active, ctx->flag_dev, ctx->stream));
+    const bool pair_mode = grouped_pair_mode(w->type, K, n_pairs, w->E);
+    if (!pair_mode)
+        QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, w->E, order, offsets, active, ctx->flag_dev, ctx->stream));
     GemvArgs g{};
     g.n_targets = 1;
     g.t[0].w = w->view;
     g.t[0].y = y_dev;
+    if (pair_mode) {
+        g.ids = ids_dev;
+        g.n_pairs = (int)n_pairs;
+        g.error_flag = ctx->flag_dev;
+    }
     g.a = act_view(p, ctx->ws, K);
     g.x = fuse ? x_dev : nullptr;
     g.order = order;
@@ -720,8 +734,16 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     const bool fuse_x = grouped_fuses_quantizer(gate->type, d_model, n_pairs, E);
     const bool fuse_h = grouped_fuses_quantizer(down->type, d_ff, n_pairs, E);
     if (!fuse_x) QP_HIP(ctx, run_quantize(ctx, px, ws, x_dev, B, d_model));
-    QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, E, order, offsets, active, ctx->flag_dev, ctx->stream));
+    const bool pair_mode = grouped_pair_mode(gate->type, d_model, n_pairs, E) &&
+                           grouped_pair_mode(down->type, d_ff, n_pairs, E);
+    if (!pair_mode)
+        QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, E, order, offsets, active, ctx->flag_dev, ctx->stream));
     GemvArgs g{};
+    if (pair_mode) {
+        g.ids = ids_dev;
+        g.n_pairs = (int)n_pairs;
+        g.error_flag = ctx->flag_dev;
+    }
     g.n_targets = 2;
     g.t[0].w = gate->view;
     g.t[0].y = h;
@@ -739,6 +761,11 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
         QP_HIP(ctx, launch_moe_swiglu_gemv(g, mt, (int)E, ctx->stream));
     if (!fuse_h) QP_HIP(ctx, run_quantize(ctx, ph, ws + off_hq, h, n_pairs, d_ff));
     GemvArgs gd{};
+    if (pair_mode) {
+        gd.ids = ids_dev;
+        gd.n_pairs = (int)n_pairs;
+        gd.error_flag = ctx->flag_dev;
+    }
     gd.n_targets = 1;
     gd.t[0].w = down->view;
     gd.t[0].y = e;

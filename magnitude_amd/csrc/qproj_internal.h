@@ -70,6 +70,11 @@ struct GemvArgs {
     const int32_t *offsets; // [E+1] ranges into order
     const int32_t *active;  // [E+1] experts that have pairs, ascending; [E] = how many
     int x_div;              // activation row of pair p is p / x_div
+    // pair mode of the grouped matrix-core kernel (a handful of pairs, no grouping pass): a set of
+    // workgroups per pair p multiplies row p / x_div by expert ids[p]; ids outside [0, E) raise *error_flag
+    const int32_t *ids;
+    int n_pairs;
+    int32_t *error_flag;
 };
 
 // ---- launchers (each returns the hipError_t of the launch) ----
