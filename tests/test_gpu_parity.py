@@ -328,7 +328,9 @@ def routing(rng, B, top, E):
     return ids, (e / e.sum(axis=1, keepdims=True)).astype(np.float32)
 
 
-@pytest.mark.parametrize("B", [1, 8, 64])
+# B = 1: a workgroup set per pair (no grouping pass); B = 3: grouped, activations quantized in the
+# kernel prologue; B = 8, 64: grouped, separate quantizer launch
+@pytest.mark.parametrize("B", [1, 3, 8, 64])
 def test_mul_mat_id_matches_oracle(ctx, orc, moe, B):
     from magnitude_amd import ACT_GGML
     E, k, n, top = moe["E"], moe["d_model"], moe["d_ff"], 8
@@ -354,9 +356,17 @@ def test_mul_mat_id_reports_bad_expert_ids(ctx, orc, moe):
         ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML)
     ids[0, 1] = 1                                            # the context stays usable
     ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML)
+    # the same through the grouping pass (more than 16 pairs)
+    ids = np.tile(np.arange(8, dtype=np.int32), (3, 1))
+    ids[2, 5] = -1
+    x = np.zeros((3, 1, k), np.float32)
+    with pytest.raises(QprojError):
+        ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML)
+    ids[2, 5] = 5
+    ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML)
 
 
-@pytest.mark.parametrize("B", [1, 8, 64])
+@pytest.mark.parametrize("B", [1, 3, 8, 64])
 def test_moe_ffn_matches_oracle(ctx, orc, moe, B):
     from magnitude_amd import ACT_GGML
     E, d_model, d_ff, top = moe["E"], moe["d_model"], moe["d_ff"], 8
