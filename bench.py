@@ -145,7 +145,8 @@ def main():
         "metric": "Q4_K GEMV achieved HBM GB/s (% peak) + prefill GEMM TOPS, 8B shapes",
         "value": None, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 x int4/int6 weights -> int32 dot, fp32 scale (u8 bytes streamed)",
+        "dtype": "int8",
+        "dtype_note": "int8 activations x int4/int6/int8 weight codes -> int32 dots, fp32 scales (u8 bytes streamed)",
         "data": "synthetic: N(0,0.02) weights quantized to GGUF Q4_K/Q6_K on the device, N(0,1) fp32 activations",
         "config": {"workload": "configs[1]: Q4_K_M decode projections (q,k,v,o,gate,up Q4_K; down Q6_K), batch 1, "
                                f"d_model 4096, FFN 14336, {args.layers} distinct layers per step",
