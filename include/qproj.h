@@ -102,7 +102,7 @@ int qproj_dequantize(qproj_ctx *ctx, const qproj_weight *w, float *out_dev);
  *   Q8_K  : int8 qs[M][K] | f32 d[M][K/256] | int16 bsums[M][K/16] | f16 msum[M][K/256][16]
  *           (msum: d * (sum of the 32 codes of a sub-block) / 16 as an fp16 pair, the 8 high parts of
  *           a super-block, then the 8 low parts; operand of the prefill kernel's min term)
- *   Q8X32 : int8 qs[M][K] | f32 d[M][K/32]  | int32 isum[M][K/32]
+ *   Q8X32 : int8 qs[M][K] | f32 d[M][K/32]  | int32 isum[M][K/32] | f16 msum[M][K/256][16] (as above)
  * each plane starting at a 256-byte aligned offset, in that order. */
 size_t qproj_act_bytes(int kind, int wtype, int64_t M, int64_t K);
 int qproj_quantize_activations(qproj_ctx *ctx, int kind, int wtype, const float *x_dev, int64_t M,

@@ -35,7 +35,8 @@ __global__ __launch_bounds__(256) void quant_q8k_kernel(const float *__restrict_
 template <bool FP16_SCALE>
 __global__ __launch_bounds__(256) void quant_q8_32_kernel(const float *__restrict__ x, int64_t n_chunks256,
                                                           int64_t n_elems, int8_t *__restrict__ qs,
-                                                          float *__restrict__ d, int32_t *__restrict__ isum) {
+                                                          float *__restrict__ d, int32_t *__restrict__ isum,
+                                                          uint16_t *__restrict__ msum) {
     const int64_t ch = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (ch >= n_chunks256) return;
@@ -51,7 +52,15 @@ __global__ __launch_bounds__(256) void quant_q8_32_kernel(const float *__restric
     if ((lane & 7) == 0) {
         const int64_t b = e0 >> 5;
         d[b] = FP16_SCALE ? h2f(f2h(dd)) : dd;
-        if (!FP16_SCALE) isum[b] = s;
+        if (!FP16_SCALE) {
+            isum[b] = s;
+            // d * (sum of the block's codes), split into two fp16 parts, in the order the prefill kernel
+            // feeds them to the fp16 matrix instruction: per 256 elements 8 high parts, then 8 low parts
+            const float v = dd * (float)s * kMinPrescale;
+            const _Float16 hi = (_Float16)v, lo = (_Float16)(v - (float)hi);
+            msum[ch * 16 + (lane >> 3)] = __builtin_bit_cast(uint16_t, hi);
+            msum[ch * 16 + 8 + (lane >> 3)] = __builtin_bit_cast(uint16_t, lo);
+        }
     }
 }
 
@@ -64,9 +73,9 @@ hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, i
     if (kind == kActKindQ8_K) {
         hipLaunchKernelGGL(quant_q8k_kernel, grid, block, 0, s, x, n / 256, qs, d, bsums, msum);
     } else if (kind == kActKindQ8_0) {
-        hipLaunchKernelGGL(quant_q8_32_kernel<true>, grid, block, 0, s, x, chunks, n, qs, d, isum);
+        hipLaunchKernelGGL(quant_q8_32_kernel<true>, grid, block, 0, s, x, chunks, n, qs, d, isum, msum);
     } else if (kind == kActKindQ8X32) {
-        hipLaunchKernelGGL(quant_q8_32_kernel<false>, grid, block, 0, s, x, chunks, n, qs, d, isum);
+        hipLaunchKernelGGL(quant_q8_32_kernel<false>, grid, block, 0, s, x, chunks, n, qs, d, isum, msum);
     } else {
         return hipErrorInvalidValue;
     }

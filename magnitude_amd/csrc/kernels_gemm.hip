@@ -90,53 +90,76 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const Weigh
         for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
 
     // ---------------------------------------------------------------- min term on the fp16 cores
-    // acc = -(1/prescale) * sum_kb A[m][kb] * B[n][kb] is built as +sum with negated B and scaled later
+    // acc = -(1/prescale) * sum_kb A[m][kb] * B[n][kb] is built as +sum with negated B and scaled later.
+    // The activation side (d * block sum, as fp16 high and low parts) comes ready from the quantizer.  The
+    // weight side (-dmin * min of every sub-block, split the same way) is worked out once per workgroup,
+    // 16 super-blocks at a time, into the LDS the main loop will use afterwards: two planes
+    // [super-block][row][8 x fp16], so that every wave only reads operands and issues matrix instructions.
     if constexpr (kQ4) {
-        const int64_t n_steps = (kb32 + 15) / 16;  // 16 sub-blocks = two super-blocks per product
-        for (int64_t s = 0; s < n_steps; ++s) {
-            v8h ah, al, bh[2], bl[2];
-            {
-                int64_t m = m0 + wm * 32 + l32;
-                int64_t kb = s * 16 + 8 * lh;  // this half-wave's super-block; past the end of K: zeros
-                const bool live = m < M && kb < kb32;
-                if (m >= M) m = M - 1;
-                if (kb >= kb32) kb = kb32 - 8;
-                const int64_t o = m * kb32 + kb;
-                const float4 d0 = *reinterpret_cast<const float4 *>(a.d + o);
-                const float4 d1 = *reinterpret_cast<const float4 *>(a.d + o + 4);
-                const int4 s0 = *reinterpret_cast<const int4 *>(a.isum + o);
-                const int4 s1 = *reinterpret_cast<const int4 *>(a.isum + o + 4);
-                const float av[8] = {d0.x * (float)s0.x, d0.y * (float)s0.y, d0.z * (float)s0.z, d0.w * (float)s0.w,
-                                     d1.x * (float)s1.x, d1.y * (float)s1.y, d1.z * (float)s1.z, d1.w * (float)s1.w};
+        constexpr int SBC = 16;                                   // super-blocks per pass (2 x 16 x 128 x 16 B = 64 KB)
+        static_assert(2 * SBC * BN * 16 <= (int)sizeof(GemmSmem), "the min-term planes must fit the main loop's LDS");
+        uint8_t *plane_hi = smem_raw, *plane_lo = smem_raw + SBC * BN * 16;
+        const int64_t mrow = m0 + wm * 32 + l32 < M ? m0 + wm * 32 + l32 : M - 1;   // rows past M are never stored
+        for (int64_t c0 = 0; c0 < w.nb; c0 += SBC) {
+            const int nsbc = (int)(w.nb - c0 < SBC ? w.nb - c0 : SBC);
+            if (c0 > 0) __syncthreads();   // the previous pass has been read
+            for (int base = 0; base < BN * nsbc; base += 4 * kGemmThreads) {
+                v4i hd[4];
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    _Float16 h, l;
-                    split_h(live ? av[t] * kMinPrescale : 0.f, h, l);
-                    ah[t] = h;
-                    al[t] = l;
+                for (int u = 0; u < 4; ++u) {   // four headers in flight per thread
+                    const int item = min(base + u * kGemmThreads + tid, BN * nsbc - 1);
+                    int64_t n = n0 + (item & (BN - 1));
+                    if (n >= N) n = N - 1;
+                    hd[u] = *reinterpret_cast<const v4i *>(w.q4k + (n * w.nb + c0 + (item >> 7)) * 144);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int item = base + u * kGemmThreads + tid;
+                    if (item >= BN * nsbc) continue;
+                    const ScalesK4 sc = unpack_scales_k4((uint32_t)hd[u][1], (uint32_t)hd[u][2], (uint32_t)hd[u][3]);
+                    const float dmin = h2f((uint32_t)hd[u][0] >> 16);
+                    v8h bh, bl;
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) {
+                        _Float16 h, l;
+                        split_h(-(dmin * (float)min_k4(sc, t)), h, l);
+                        bh[t] = h;
+                        bl[t] = l;
+                    }
+                    *reinterpret_cast<v8h *>(plane_hi + item * 16) = bh;   // item = super-block * 128 + row
+                    *reinterpret_cast<v8h *>(plane_lo + item * 16) = bl;
                 }
             }
+            __syncthreads();
+            const int n_steps = (nsbc + 1) / 2;   // 16 sub-blocks = two super-blocks per product
+            v8h ah, al, ah_n, al_n;
+            auto load_a = [&](v8h &h, v8h &l, int s) {
+                int sbl = 2 * s + lh;
+                if (sbl >= nsbc) sbl = nsbc - 1;   // past the end: any finite operand, the weight side is zero there
+                const v8h *mp = reinterpret_cast<const v8h *>(a.msum + (mrow * w.nb + c0 + sbl) * 16);
+                h = mp[0];
+                l = mp[1];
+            };
+            load_a(ah, al, 0);
+            for (int s = 0; s < n_steps; ++s) {
+                load_a(ah_n, al_n, s + 1 < n_steps ? s + 1 : s);   // in flight during this step
+                const int sbl = 2 * s + lh;
+                const bool live = sbl < nsbc;
 #pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                int64_t sb = s * 2 + lh;
-                const bool live = sb < w.nb;
-                if (!live) sb = w.nb - 1;
-                const uint4 hd = *reinterpret_cast<const uint4 *>(w.q4k + (ncol[j] * w.nb + sb) * 144);
-                const ScalesK4 sc = unpack_scales_k4(hd.y, hd.z, hd.w);
-                const float dmin = live ? h2f(hd.x >> 16) : 0.f;
+                for (int j = 0; j < 2; ++j) {
+                    const int o = ((live ? sbl : 0) * BN + wn * 64 + j * 32 + l32) * 16;
+                    v8h bh = *reinterpret_cast<const v8h *>(plane_hi + o);
+                    v8h bl = *reinterpret_cast<const v8h *>(plane_lo + o);
+                    if (!live) {
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    _Float16 h, l;
-                    split_h(-(dmin * (float)min_k4(sc, t)), h, l);
-                    bh[j][t] = h;
-                    bl[j][t] = l;
+                        for (int t = 0; t < 8; ++t) bh[t] = bl[t] = (_Float16)0.f;
+                    }
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh, acc[j], 0, 0, 0);
                 }
-            }
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh[j], acc[j], 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl[j], acc[j], 0, 0, 0);
-                acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh[j], acc[j], 0, 0, 0);
+                ah = ah_n;
+                al = al_n;
             }
         }
         const float inv = 1.0f / kMinPrescale;
@@ -144,6 +167,7 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const Weigh
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[j][v] *= inv;
+        __syncthreads();   // the planes have been read: the main loop may overwrite them
     }
 
     // ---------------------------------------------------------------- main loop, int8 cores
@@ -503,7 +527,7 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const W
 }  // namespace
 
 hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
-    if (w.type != kTypeQ4_K || w.K % 256 != 0 || M <= 0) return hipErrorInvalidValue;
+    if (w.type != kTypeQ4_K || w.K % 256 != 0 || M <= 0 || !a.msum) return hipErrorInvalidValue;
     const auto kern = &gemm_per32_kernel<kTypeQ4_K>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem));

@@ -98,7 +98,7 @@ ActPlanes act_planes(int kind, int64_t M, int64_t K) {
     if (kind == kActKindQ8_K) aux = (size_t)(M * (K / 16)) * 2;
     if (kind == kActKindQ8X32) aux = (size_t)(M * (K / 32)) * 4;
     p.off_msum = p.off_aux + align_up(aux);
-    p.total = p.off_msum + (kind == kActKindQ8_K ? align_up((size_t)(M * (K / 256)) * 32) : 0);
+    p.total = p.off_msum + (kind == kActKindQ8_K || kind == kActKindQ8X32 ? align_up((size_t)(M * (K / 256)) * 32) : 0);
     return p;
 }
 
@@ -109,7 +109,7 @@ ActView act_view(const ActPlanes &p, uint8_t *base, int64_t K) {
     a.qs = reinterpret_cast<const int8_t *>(base + p.off_qs);
     a.d = reinterpret_cast<const float *>(base + p.off_d);
     a.bsums = p.kind == kActKindQ8_K ? reinterpret_cast<const int16_t *>(base + p.off_aux) : nullptr;
-    a.msum = p.kind == kActKindQ8_K ? reinterpret_cast<const uint16_t *>(base + p.off_msum) : nullptr;
+    a.msum = p.kind == kActKindQ8_K || p.kind == kActKindQ8X32 ? reinterpret_cast<const uint16_t *>(base + p.off_msum) : nullptr;
     a.isum = p.kind == kActKindQ8X32 ? reinterpret_cast<const int32_t *>(base + p.off_aux) : nullptr;
     return a;
 }

@@ -41,7 +41,7 @@ struct ActView {
     const int8_t *qs;      // [rows][K]
     const float *d;        // [rows][K/32] (Q8_0, Q8X32) or [rows][K/256] (Q8_K)
     const int16_t *bsums;  // Q8_K: [rows][K/16]
-    const uint16_t *msum;  // Q8_K: [rows][K/256][16] fp16: d * (sum of 32 codes) * kMinPrescale for the 8
+    const uint16_t *msum;  // Q8_K, Q8X32: [rows][K/256][16] fp16: d * (sum of 32 codes) * kMinPrescale for the 8
                            //       sub-blocks, high parts, then the 8 low parts (v - high); prefill min term
     const int32_t *isum;   // Q8X32: [rows][K/32]
 };

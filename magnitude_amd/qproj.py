@@ -212,6 +212,8 @@ class Context:
             out["msum"] = buf[off_ms:off_ms + m * (k // 256) * 32].view(torch.float16).view(m, k // 256, 2, 8)
         elif kind == ACT_Q8X32:
             out["isum"] = buf[off_aux:off_aux + m * (k // 32) * 4].view(torch.int32).view(m, k // 32)
+            off_ms = off_aux + al(m * (k // 32) * 4)
+            out["msum"] = buf[off_ms:off_ms + m * (k // 256) * 32].view(torch.float16).view(m, k // 256, 2, 8)
         return out
 
     # ---- operators -----------------------------------------------------------------------

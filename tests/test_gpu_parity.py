@@ -177,6 +177,14 @@ def test_quantize_q8x32_bit_exact(ctx, orc):
     assert np.array_equal(got["qs"].cpu().numpy(), raw[:, :, 8:].view(np.int8).reshape(m, k))
     assert np.array_equal(got["d"].cpu().numpy().view(np.uint32), raw[:, :, 0:4].copy().view(np.uint32)[:, :, 0])
     assert np.array_equal(got["isum"].cpu().numpy(), raw[:, :, 4:8].copy().view(np.int32)[:, :, 0])
+    # the prefill kernel's extra plane: d * isum / 16 as an fp16 high part and the fp16 of the rest
+    d32 = raw[:, :, 0:4].copy().view(np.float32)[:, :, 0]
+    v = d32 * raw[:, :, 4:8].copy().view(np.int32)[:, :, 0].astype(np.float32) * np.float32(0.0625)
+    hi = v.astype(np.float16)
+    lo = (v - hi.astype(np.float32)).astype(np.float16)
+    ms = got["msum"].cpu().numpy()
+    assert np.array_equal(ms[:, :, 0].view(np.uint16), hi.reshape(m, k // 256, 8).view(np.uint16))
+    assert np.array_equal(ms[:, :, 1].view(np.uint16), lo.reshape(m, k // 256, 8).view(np.uint16))
 
 
 # ---------------------------------------------------------------- mul_mat, decode and small M
