@@ -16,6 +16,7 @@
 //     header by that lane and held in registers for the 8 sub-blocks of a super-block;
 //   - LDS holds only the two int8 operand tiles and the transposed activation scales, double
 //     buffered over K-steps of 128 so that the global loads of step s+1 overlap step s.
+#include <cstdlib>
 #include "qproj_device.h"
 #include "qproj_internal.h"
 #include "gemm_tiles.h"
@@ -60,9 +61,11 @@ constexpr int kGemmThreads = 512;
 // QT = Q4_K: per-32 int8 activations with fp32 scales and block sums (the prefill format).
 // QT = Q8_0: ggml's Q8_0 activation blocks against Q8_0 weights: the same product without nibbles,
 // without a min term, and with a weight scale per 32 instead of d*sc per sub-block.
+// blockIdx.y selects one of gridDim.y equal stretches of K (whole super-blocks for Q4_K); with more than one
+// the tile goes to part[blockIdx.y][M][N] and sum_parts_kernel adds the stretches up in order.
 template <int QT>
 __global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const WeightView w, const ActView a, int64_t M,
-                                                                   float *__restrict__ y) {
+                                                                   float *__restrict__ y, float *__restrict__ part) {
     constexpr bool kQ4 = QT == kTypeQ4_K;
     extern __shared__ __align__(16) uint8_t smem_raw[];
     GemmSmem &sm = *reinterpret_cast<GemmSmem *>(smem_raw);
@@ -74,6 +77,10 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const Weigh
     const int64_t n0 = (int64_t)tile_n * BN, m0 = (int64_t)tile_m * BM;
     const int64_t kb32 = K / 32;
     const int l32 = lane & 31, lh = lane >> 5;
+    // this workgroup's stretch of K, in units of 256 (Q4_K super-blocks; two K-steps)
+    const int64_t n_units = (K + 255) / 256, per = (n_units + gridDim.y - 1) / gridDim.y;
+    const int64_t u_begin = min((int64_t)blockIdx.y * per, n_units), u_end = min(u_begin + per, n_units);
+    if (gridDim.y > 1) y = part + (size_t)blockIdx.y * M * N;
 
     // the lane's two output columns (clamped for loads; stores are guarded)
     int64_t ncol[2];
@@ -100,9 +107,9 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const Weigh
         static_assert(2 * SBC * BN * 16 <= (int)sizeof(GemmSmem), "the min-term planes must fit the main loop's LDS");
         uint8_t *plane_hi = smem_raw, *plane_lo = smem_raw + SBC * BN * 16;
         const int64_t mrow = m0 + wm * 32 + l32 < M ? m0 + wm * 32 + l32 : M - 1;   // rows past M are never stored
-        for (int64_t c0 = 0; c0 < w.nb; c0 += SBC) {
-            const int nsbc = (int)(w.nb - c0 < SBC ? w.nb - c0 : SBC);
-            if (c0 > 0) __syncthreads();   // the previous pass has been read
+        for (int64_t c0 = u_begin; c0 < u_end; c0 += SBC) {
+            const int nsbc = (int)(u_end - c0 < SBC ? u_end - c0 : SBC);
+            if (c0 > u_begin) __syncthreads();   // the previous pass has been read
             for (int base = 0; base < BN * nsbc; base += 4 * kGemmThreads) {
                 v4i hd[4];
 #pragma unroll
@@ -253,13 +260,15 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const Weigh
         }
     };
 
+    const int64_t ks_begin = u_begin * 2, n_ksteps = min(u_end * 2, K / BK);
     StageRegs regs;
-    load_stage(regs, 0);
-    store_stage(regs, sm.st[0], 0);
+    if (ks_begin < n_ksteps) {
+        load_stage(regs, ks_begin * BK);
+        store_stage(regs, sm.st[ks_begin & 1], ks_begin * BK);
+    }
     __syncthreads();
 
-    const int64_t n_ksteps = K / BK;
-    for (int64_t ks = 0; ks < n_ksteps; ++ks) {
+    for (int64_t ks = ks_begin; ks < n_ksteps; ++ks) {
         const int64_t k0 = ks * BK;
         const GemmStage &st = sm.st[ks & 1];
         if (ks + 1 < n_ksteps) load_stage(regs, k0 + BK);  // in flight during the arithmetic below
@@ -526,27 +535,61 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const W
 
 }  // namespace
 
-hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
-    if (w.type != kTypeQ4_K || w.K % 256 != 0 || M <= 0 || !a.msum) return hipErrorInvalidValue;
-    const auto kern = &gemm_per32_kernel<kTypeQ4_K>;
+namespace {
+// y[i] = part[0][i] + part[1][i] + ... in that order
+__global__ __launch_bounds__(256) void sum_parts_kernel(const float *__restrict__ part, int n_split, size_t n4,
+                                                        float *__restrict__ y) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    float4 s = reinterpret_cast<const float4 *>(part)[i];
+    for (int c = 1; c < n_split; ++c) {
+        const float4 v = reinterpret_cast<const float4 *>(part)[(size_t)c * n4 + i];
+        s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    reinterpret_cast<float4 *>(y)[i] = s;
+}
+
+template <int QT>
+hipError_t launch_per32(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s) {
+    const auto kern = &gemm_per32_kernel<QT>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem));
     if (attr != hipSuccess) return attr;
-    const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + BM - 1) / BM)));
-    hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y);
+    const int n_split = scratch ? per32_splits(w.K, M, w.N) : 1;
+    const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + BM - 1) / BM)), (unsigned)n_split);
+    hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y, scratch);
+    if (n_split > 1) {
+        const size_t n4 = (size_t)M * w.N / 4;
+        hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, scratch, n_split, n4, y);
+    }
     return hipGetLastError();
+}
+}  // namespace
+
+// A grid of fewer than 192 tiles leaves the 256 compute units (two workgroups each) mostly idle and a
+// workgroup's K loop is latency-bound: K is then cut into 2 or 3 stretches done by different workgroups.
+int per32_splits(int64_t K, int64_t M, int64_t N) {
+    static const int forced = getenv("QPROJ_PER32_SPLITS") ? atoi(getenv("QPROJ_PER32_SPLITS")) : 0;
+    const int64_t tiles = ((N + BN - 1) / BN) * ((M + BM - 1) / BM);
+    int n = forced > 0 ? forced : tiles >= 192 ? 1 : tiles >= 96 ? 2 : 3;
+    if ((M * N) % 4 != 0) n = 1;
+    while (n > 1 && K / 256 < 4 * n) --n;   // at least four super-blocks a stretch
+    return n;
+}
+size_t per32_scratch_bytes(int64_t K, int64_t M, int64_t N) {
+    const int n = per32_splits(K, M, N);
+    return n > 1 ? (size_t)n * M * N * 4 : 0;
+}
+
+hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s) {
+    if (w.type != kTypeQ4_K || w.K % 256 != 0 || M <= 0 || !a.msum) return hipErrorInvalidValue;
+    return launch_per32<kTypeQ4_K>(w, a, M, y, scratch, s);
 }
 
 // Q8_0 weights x ggml Q8_0 activation blocks (planes in `a`), K a multiple of 128
-hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
+hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s) {
     if (w.type != kTypeQ8_0 || a.kind != kActKindQ8_0 || w.K % BK != 0 || M <= 0) return hipErrorInvalidValue;
-    const auto kern = &gemm_per32_kernel<kTypeQ8_0>;
-    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem));
-    if (attr != hipSuccess) return attr;
-    const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + BM - 1) / BM)));
-    hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y);
-    return hipGetLastError();
+    return launch_per32<kTypeQ8_0>(w, a, M, y, scratch, s);
 }
 
 // ggml-format activations (Q8_K planes in `a`, including the min-term plane), Q4_K weights, any M

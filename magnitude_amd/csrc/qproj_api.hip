@@ -251,7 +251,14 @@ bool use_mfma_kernel(int type, int64_t M, int64_t K) {
 }
 
 // scratch bytes run_dense_q8act needs for M rows against these tensors
+size_t per32_scratch_max(int n, const qproj_weight *const *w, int64_t M) {   // the targets run one after the other
+    size_t need = 0;
+    for (int i = 0; i < n; ++i) need = std::max(need, per32_scratch_bytes(w[i]->K, M, w[i]->N));
+    return need;
+}
+
 size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
+    if (w[0]->type == kTypeQ8_0 && M >= 64 && w[0]->K % 128 == 0) return per32_scratch_max(n, w, M);   // tiled Q8_0 product
     if (!use_mfma_kernel(w[0]->type, M, w[0]->K)) return 0;
     int64_t sum_n = 0, rgs = 0;
     for (int i = 0; i < n; ++i) {
@@ -290,7 +297,7 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
             const int t = w[0]->type;
             QP_HIP(ctx, t == kTypeQ4_K   ? launch_gemm_q8k(w[i]->view, a, M, y[i], ctx->stream)
                         : t == kTypeQ6_K ? launch_gemm_q6k_q8k(w[i]->view, a, M, y[i], ctx->stream)
-                                         : launch_gemm_q8_0(w[i]->view, a, M, y[i], ctx->stream));
+                                         : launch_gemm_q8_0(w[i]->view, a, M, y[i], scratch, ctx->stream));
         }
         return QPROJ_OK;
     }
@@ -580,14 +587,16 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
             return run_dense_q8act(ctx, n, w, a, M, y_dev, reinterpret_cast<float *>(ctx->ws), x_dev);
         }
         const ActPlanes p = act_planes(act_kind_for(act, w[0]->type), M, K);
-        const size_t extra = act == kActGGML ? dense_scratch_bytes(n, w, M) : 0;
+        const size_t extra = act == kActGGML ? dense_scratch_bytes(n, w, M) : per32_scratch_max(n, w, M);
         int rc = ensure_ws(ctx, p.total + extra);
         if (rc) return rc;
         QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, M, K));
         const ActView a = act_view(p, ctx->ws, K);
         if (act == kActGGML)
             return run_dense_q8act(ctx, n, w, a, M, y_dev, reinterpret_cast<float *>(ctx->ws + p.total));
-        for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], ctx->stream));
+        for (int i = 0; i < n; ++i)
+            QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], extra ? reinterpret_cast<float *>(ctx->ws + p.total) : nullptr,
+                                          ctx->stream));
         return QPROJ_OK;
     }
     if (act == kActF32) {
@@ -632,7 +641,11 @@ int qproj_mul_mat_quantized(qproj_ctx *ctx, int n, const qproj_weight *const *w,
         if (rc) return rc;
         return run_dense_q8act(ctx, n, w, a, M, y_dev, reinterpret_cast<float *>(ctx->ws));
     }
-    for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], ctx->stream));
+    const size_t extra = per32_scratch_max(n, w, M);
+    int rc = ensure_ws(ctx, extra);
+    if (rc) return rc;
+    for (int i = 0; i < n; ++i)
+        QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], extra ? reinterpret_cast<float *>(ctx->ws) : nullptr, ctx->stream));
     return QPROJ_OK;
 }
 

@@ -102,10 +102,13 @@ hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_exper
 hipError_t launch_moe_swiglu_gemv(const GemvArgs &gate_up, int mt, int n_experts_grid, hipStream_t s);
 hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, int64_t n_used, int64_t N,
                               float *y, hipStream_t s);
-hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
+// `scratch`: per32_scratch_bytes(K, M, N) bytes (may be null: then K is never split)
+int per32_splits(int64_t K, int64_t M, int64_t N);
+size_t per32_scratch_bytes(int64_t K, int64_t M, int64_t N);
+hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s);
 // Q4_K weights x ggml Q8_K activations (`a`), large M
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
-hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
+hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s);
 hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s);
 
 }  // namespace qproj
