@@ -533,6 +533,213 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const W
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// The same product for large batches: every wave keeps its 32 weight rows but works on 128 tokens.
+//
+// The kernel above spends four vector instructions per matrix instruction on expanding and scaling
+// weights, because a converted weight fragment feeds only two token tiles.  Here a wave converts the
+// whole super-block of its 32 rows once into 64 registers (both chains, all eight steps) and then
+// walks four token tiles with them, so the conversion is paid once per 128 tokens.  Eight waves =
+// 256 weight rows x 128 tokens per workgroup, one workgroup per compute unit.
+//
+// Nothing passes through staging registers: activations, the min-term tile, the activation scales
+// and the raw weight blocks go from global memory straight into LDS (global_load_lds, 16 bytes a
+// lane, a wave writes one contiguous kilobyte per instruction).  Because such a load cannot pad LDS
+// rows, the activation tile is stored [token][256] with the 16-byte segments of a row XOR-swizzled
+// by the token index: slot s of token r holds segment s ^ (r & 15), which the loading lane simply
+// requests from global memory, and 16 consecutive tokens reading "their" segment g hit 16 different
+// slots.
+template <int NW>
+struct WideSmem {
+    int8_t a[2][128 * 256];          // activations of one super-block [token][16 swizzled segments]
+    uint16_t ms[2][128 * 16];        // min-term operand [token][8 high | 8 low] (fp16 bits)
+    float dx[2][128];                // activation scale of the super-block
+    uint8_t park[NW][5 * 1024];      // per wave: raw blocks of its 32 weight rows (4608 bytes used)
+};
+
+__device__ __forceinline__ void global_to_lds16(const void *g, void *l) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
+                                     (__attribute__((address_space(3))) void *)l, 16, 0, 0);
+}
+__device__ __forceinline__ void global_to_lds4(const void *g, void *l) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
+                                     (__attribute__((address_space(3))) void *)l, 4, 0, 0);
+}
+
+template <int NW>
+__global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const WeightView w, const ActView a, int64_t M,
+                                                                      float *__restrict__ y) {
+    static_assert(NW == 8, "the loading roles below are laid out for eight waves");
+    constexpr int TM = 128, TN = 32 * NW, JT = TM / 32;
+    constexpr int PA = (TM * 16) / (64 * NW);   // 1-KB activation chunks (4 tokens) a wave requests per super-block
+    extern __shared__ __align__(16) uint8_t smem_raw[];
+    WideSmem<NW> &sm = *reinterpret_cast<WideSmem<NW> *>(smem_raw);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t N = w.N, K = w.K, nb = w.nb;
+    int tile_n, tile_m;
+    tile_of_workgroup((int)((N + TN - 1) / TN), (int)((M + TM - 1) / TM), tile_n, tile_m);
+    const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * TM;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    v16f acc[JT];
+#pragma unroll
+    for (int j = 0; j < JT; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+    // ---- global -> LDS requests: wave-uniform bases plus 32-bit lane offsets; rows past the edge of
+    // a matrix repeat its last valid row (computed, never stored)
+    const int64_t wave_row0 = n0 + wave * 32 < N ? n0 + wave * 32 : N - 1;
+    const int wrow_cap = (int)(N - 1 - wave_row0 < 31 ? N - 1 - wave_row0 : 31);
+    const uint8_t *wbase = w.q4k + wave_row0 * nb * 144;
+    uint32_t woff[5];   // piece p = lane + 64*c of the wave's 288 -> row p / 9, 16-byte part p % 9
+#pragma unroll
+    for (int c = 0; c < 5; ++c) {
+        const int p = lane + 64 * c < 287 ? lane + 64 * c : 287;
+        const int r = p / 9 < wrow_cap ? p / 9 : wrow_cap;
+        woff[c] = (uint32_t)(r * (int)nb * 144 + 16 * (p % 9));
+    }
+    const int mrow_cap = (int)(M - 1 - m0 < TM - 1 ? M - 1 - m0 : TM - 1);
+    const int8_t *abase = a.qs + m0 * K;
+    uint32_t aoffg[PA];   // chunk wave + NW*p = tokens 4*chunk .. +3; lane -> token lane/16, slot lane%16
+#pragma unroll
+    for (int p = 0; p < PA; ++p) {
+        const int row = 4 * (wave + NW * p) + (lane >> 4), seg = (lane & 15) ^ (row & 15);
+        aoffg[p] = (uint32_t)((row < mrow_cap ? row : mrow_cap) * (int)K + 16 * seg);
+    }
+    // waves 0..3: min-term tile (2 pieces a token); waves 4, 5: activation scales (one float a token)
+    const uint8_t *msbase = reinterpret_cast<const uint8_t *>(a.msum) + m0 * nb * 32;
+    const int mstok = (wave & 3) * 32 + (lane >> 1), dxtok = tid & 127;
+    const uint32_t msoffg = (uint32_t)((mstok < mrow_cap ? mstok : mrow_cap) * (int)nb * 32 + 16 * (lane & 1));
+    const float *dxbase = a.d + m0 * nb;
+    const uint32_t dxoffg = (uint32_t)((dxtok < mrow_cap ? dxtok : mrow_cap) * (int)nb);
+    uint8_t *park = sm.park[wave];
+    float dxreg;   // the one piece that travels through a register (4-byte items do not fill a 16-byte slot)
+
+    auto request = [&](int64_t sb, int buf) {
+#pragma unroll
+        for (int p = 0; p < PA; ++p) global_to_lds16(abase + sb * 256 + aoffg[p], sm.a[buf] + (wave + NW * p) * 1024);
+        if (wave < 4) global_to_lds16(msbase + sb * 32 + msoffg, reinterpret_cast<uint8_t *>(sm.ms[buf]) + wave * 1024);
+        dxreg = dxbase[sb + dxoffg];
+#pragma unroll
+        for (int c = 0; c < 5; ++c) global_to_lds16(wbase + sb * 144 + woff[c], park + 1024 * c);
+    };
+
+    // the lane's eight activation reads of a token tile: segment t + 8*(l/32) of token l%32 (+32*j) sits in
+    // slot (t + 8*(l/32)) ^ (l%16) = t ^ z with z = 8*(l/32) ^ (l%16), i.e. at byte (256*(l%32) + 16*z) ^ 16*t
+    const int aoffl = l32 * 256 + 16 * ((8 * lh) ^ (l32 & 15));
+
+    const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    auto superblock = [&](const DirectB &b, int buf) {
+        const ScalesK4 sc = unpack_scales_k4((uint32_t)b.hdr[1], (uint32_t)b.hdr[2], (uint32_t)b.hdr[3]);
+        // ---- min term: -dmin*min of the 8 sub-blocks as fp16 high and low parts
+        const float ndmin = -h2f((uint32_t)b.hdr[0] >> 16);
+        v8h mh, ml;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            _Float16 h, l;
+            split_h(ndmin * (float)min_k4(sc, t), h, l);
+            mh[t] = h;
+            ml[t] = lh ? (_Float16)0.f : l;
+        }
+        // ---- both scaled int8 copies of the lane's 128 weights: step t = sub-block 4*(l/32) + t/2, half t%2
+        const uint32_t scw = lh ? sc.sc_hi : sc.sc_lo;
+        const uint32_t lo_w = scw & 0x07070707u, hi_w = (scw >> 3) & 0x07070707u;
+        v4i cl[8], ch[8];
+        auto convert = [&](int t) {
+            const int gg = t >> 2, nib = (t >> 1) & 1, half = t & 1, i = 2 * gg + nib;
+            const uint32_t sl = byte_to_u16x2(lo_w, i), sh = byte_to_u16x2(hi_w, i);
+            const v4i raw = b.q[2 * gg + half];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t x = nib ? ((uint32_t)raw[c] >> 4) & 0x0f0f0f0fu : (uint32_t)raw[c] & 0x0f0f0f0fu;
+                cl[t][c] = (int)pk_mul_u16(x, sl);
+                ch[t][c] = (int)pk_mul_u16(x, sh);
+            }
+        };
+        const float dn = h2f((uint32_t)b.hdr[0] & 0xffffu) * kMinPrescale;   // exact: a power of two
+        const int8_t *ab = sm.a[buf];
+        const uint8_t *msb = reinterpret_cast<const uint8_t *>(sm.ms[buf]);
+        const float *dxs = sm.dx[buf];
+        auto fragment = [&](int j, int t) {
+            return *reinterpret_cast<const v4i *>(ab + j * 32 * 256 + (aoffl ^ (16 * t)));
+        };
+        // The order below is pinned step by step (the scheduling barriers let nothing cross): four
+        // activation fragments are always in flight, a fragment register is refilled as soon as its two
+        // matrix instructions are issued, the activation scales of the tile arrive during its last four
+        // steps, the next tile's first fragments during the flush; in the first tile the conversion of
+        // step t+1 sits between the matrix instructions of step t.
+        v4i ring[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) ring[t] = fragment(0, t);
+#pragma unroll
+        for (int j = 0; j < JT; ++j) {
+            const v8h am = *reinterpret_cast<const v8h *>(msb + (j * 32 + l32) * 32 + 16 * lh);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, mh, acc[j], 0, 0, 0);
+            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, ml, acc[j], 0, 0, 0);
+        }
+        convert(0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < JT; ++j) {
+            v16i ilo, ihi;
+            v4i dq[4];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[t & 3], cl[t], t == 0 ? zi : ilo, 0, 0, 0);
+                ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[t & 3], ch[t], t == 0 ? zi : ihi, 0, 0, 0);
+                if (t < 4) ring[t & 3] = fragment(j, t + 4);
+                else dq[t - 4] = *reinterpret_cast<const v4i *>(dxs + j * 32 + 8 * (t - 4) + 4 * lh);
+                if (j == 0 && t < 7) convert(t + 1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (j + 1 < JT) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) ring[t] = fragment(j + 1, t);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                acc[j][v] = fmaf((float)((ihi[v] << 3) + ilo[v]), __int_as_float(dq[v >> 2][v & 3]) * dn, acc[j][v]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    request(0, 0);
+    sm.dx[0][tid & 127] = dxreg;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int64_t sb = 0; sb < nb; ++sb) {
+        const int buf = (int)(sb & 1);
+        DirectB b;   // out of the strip: header of row l%32, then the lane's 64 nibble bytes
+        b.hdr = *reinterpret_cast<const v4i *>(park + l32 * 144);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) b.q[i] = *reinterpret_cast<const v4i *>(park + l32 * 144 + 16 + 64 * lh + 16 * i);
+        // the strip is about to be overwritten by the next request: its reads must have returned
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        // past the end the last super-block is requested again (into the idle buffer, never read)
+        request(sb + 1 < nb ? sb + 1 : nb - 1, buf ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        superblock(b, buf);
+        sm.dx[buf ^ 1][tid & 127] = dxreg;   // every thread stores (a repeated value past 128): no branch
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+
+    // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
+    const int64_t n = n0 + wave * 32 + l32;
+    const float inv = 1.0f / kMinPrescale;
+#pragma unroll
+    for (int j = 0; j < JT; ++j) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (m < M && n < N) y[m * N + n] = acc[j][v] * inv;
+        }
+    }
+}
+
 }  // namespace
 
 namespace {
@@ -596,6 +803,18 @@ hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, fl
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
     if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || !a.msum || M <= 0) return hipErrorInvalidValue;
     if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 64 token rows of K bytes, 32 weight rows of K*144/256
+    // large batches: 128 tokens x 256 weight rows per workgroup, one workgroup per compute unit
+    static const int wide_env = getenv("QPROJ_Q8K_WIDE") ? atoi(getenv("QPROJ_Q8K_WIDE")) : -1;
+    const int64_t wide_tiles = ((w.N + 255) / 256) * ((M + 127) / 128);
+    if (wide_env >= 0 ? wide_env != 0 : wide_tiles >= 256) {
+        using Smem = WideSmem<8>;
+        const auto kern = &gemm_q4k_q8k_wide_kernel<8>;
+        static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
+        if (attr != hipSuccess) return attr;
+        hipLaunchKernelGGL(kern, dim3((unsigned)wide_tiles), dim3(512), sizeof(Smem), s, w, a, M, y);
+        return hipGetLastError();
+    }
     constexpr int NW = 4;   // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit
     using Smem = DirectSmem<NW>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_direct_kernel<NW>),
