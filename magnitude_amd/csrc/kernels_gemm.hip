@@ -17,6 +17,7 @@
 //   - LDS holds only the two int8 operand tiles and the transposed activation scales, double
 //     buffered over K-steps of 128 so that the global loads of step s+1 overlap step s.
 #include <cstdlib>
+#include <type_traits>
 #include "qproj_device.h"
 #include "qproj_internal.h"
 #include "gemm_tiles.h"
@@ -562,9 +563,13 @@ __device__ __forceinline__ void global_to_lds16(const void *g, void *l) {
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
                                      (__attribute__((address_space(3))) void *)l, 16, 0, 0);
 }
-__device__ __forceinline__ void global_to_lds4(const void *g, void *l) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
-                                     (__attribute__((address_space(3))) void *)l, 4, 0, 0);
+// a wave-uniform pointer pinned to scalar registers: what is added to it afterwards stays a 32-bit lane
+// offset (scalar base + vector offset addressing) instead of becoming a 64-bit pointer per lane
+template <typename T>
+__device__ __forceinline__ const T *scalar_pointer(const T *p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const T *>(((uint64_t)hi << 32) | lo);
 }
 
 template <int NW>
@@ -615,117 +620,170 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
     const float *dxbase = a.d + m0 * nb;
     const uint32_t dxoffg = (uint32_t)((dxtok < mrow_cap ? dxtok : mrow_cap) * (int)nb);
     uint8_t *park = sm.park[wave];
-    float dxreg;   // the one piece that travels through a register (4-byte items do not fill a 16-byte slot)
 
-    auto request = [&](int64_t sb, int buf) {
-#pragma unroll
-        for (int p = 0; p < PA; ++p) global_to_lds16(abase + sb * 256 + aoffg[p], sm.a[buf] + (wave + NW * p) * 1024);
-        if (wave < 4) global_to_lds16(msbase + sb * 32 + msoffg, reinterpret_cast<uint8_t *>(sm.ms[buf]) + wave * 1024);
-        dxreg = dxbase[sb + dxoffg];
-#pragma unroll
-        for (int c = 0; c < 5; ++c) global_to_lds16(wbase + sb * 144 + woff[c], park + 1024 * c);
+    // Addresses are a scalar base that never moves plus a 32-bit lane offset to which the super-block's
+    // displacement is added on the spot: one vector register per request stays live, not a 64-bit pointer.
+    const uint8_t *wbase_s = scalar_pointer(wbase);
+    const int8_t *abase_s = scalar_pointer(abase);
+    const uint8_t *msbase_s = scalar_pointer(msbase);
+    const float *dxbase_s = scalar_pointer(dxbase);
+    auto request_strip = [&](uint32_t sb, int c) {
+        global_to_lds16(wbase_s + (woff[c] + sb * 144u), park + 1024 * c);
+    };
+    auto request_act = [&](uint32_t sb, int buf, int p) {
+        global_to_lds16(abase_s + (aoffg[p] + sb * 256u), sm.a[buf] + (wave + NW * p) * 1024);
+    };
+    auto request_ms = [&](uint32_t sb, int buf) {
+        if (wave < 4) global_to_lds16(msbase_s + (msoffg + sb * 32u), reinterpret_cast<uint8_t *>(sm.ms[buf]) + wave * 1024);
     };
 
     // the lane's eight activation reads of a token tile: segment t + 8*(l/32) of token l%32 (+32*j) sits in
     // slot (t + 8*(l/32)) ^ (l%16) = t ^ z with z = 8*(l/32) ^ (l%16), i.e. at byte (256*(l%32) + 16*z) ^ 16*t
     const int aoffl = l32 * 256 + 16 * ((8 * lh) ^ (l32 & 15));
-
     const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    auto superblock = [&](const DirectB &b, int buf) {
-        const ScalesK4 sc = unpack_scales_k4((uint32_t)b.hdr[1], (uint32_t)b.hdr[2], (uint32_t)b.hdr[3]);
-        // ---- min term: -dmin*min of the 8 sub-blocks as fp16 high and low parts
-        const float ndmin = -h2f((uint32_t)b.hdr[0] >> 16);
-        v8h mh, ml;
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            _Float16 h, l;
-            split_h(ndmin * (float)min_k4(sc, t), h, l);
-            mh[t] = h;
-            ml[t] = lh ? (_Float16)0.f : l;
-        }
-        // ---- both scaled int8 copies of the lane's 128 weights: step t = sub-block 4*(l/32) + t/2, half t%2
+
+    // both scaled int8 copies of the lane's 128 weights (step t = sub-block 4*(l/32) + t/2, half t%2) and the header
+    v4i hdr, cl[8], ch[8];
+    uint32_t lo_w, hi_w;   // base-8 digits of the lane's four sub-block scales
+    auto read_header = [&]() {
+        hdr = *reinterpret_cast<const v4i *>(park + l32 * 144);
+        const ScalesK4 sc = unpack_scales_k4((uint32_t)hdr[1], (uint32_t)hdr[2], (uint32_t)hdr[3]);
         const uint32_t scw = lh ? sc.sc_hi : sc.sc_lo;
-        const uint32_t lo_w = scw & 0x07070707u, hi_w = (scw >> 3) & 0x07070707u;
-        v4i cl[8], ch[8];
-        auto convert = [&](int t) {
-            const int gg = t >> 2, nib = (t >> 1) & 1, half = t & 1, i = 2 * gg + nib;
-            const uint32_t sl = byte_to_u16x2(lo_w, i), sh = byte_to_u16x2(hi_w, i);
-            const v4i raw = b.q[2 * gg + half];
+        lo_w = scw & 0x07070707u;
+        hi_w = (scw >> 3) & 0x07070707u;
+    };
+    auto strip_piece = [&](int t) {   // nibble bytes of step t: 16-byte piece 2*(t/4) + t%2 of the lane's 64
+        return *reinterpret_cast<const v4i *>(park + l32 * 144 + 16 + 64 * lh + 16 * (2 * (t >> 2) + (t & 1)));
+    };
+    auto convert = [&](int t, const v4i &raw) {
+        const int i = t >> 1, nib = i & 1;
+        const uint32_t sl = byte_to_u16x2(lo_w, i), sh = byte_to_u16x2(hi_w, i);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const uint32_t x = nib ? ((uint32_t)raw[c] >> 4) & 0x0f0f0f0fu : (uint32_t)raw[c] & 0x0f0f0f0fu;
-                cl[t][c] = (int)pk_mul_u16(x, sl);
-                ch[t][c] = (int)pk_mul_u16(x, sh);
-            }
-        };
-        const float dn = h2f((uint32_t)b.hdr[0] & 0xffffu) * kMinPrescale;   // exact: a power of two
-        const int8_t *ab = sm.a[buf];
-        const uint8_t *msb = reinterpret_cast<const uint8_t *>(sm.ms[buf]);
-        const float *dxs = sm.dx[buf];
-        auto fragment = [&](int j, int t) {
-            return *reinterpret_cast<const v4i *>(ab + j * 32 * 256 + (aoffl ^ (16 * t)));
-        };
-        // The order below is pinned step by step (the scheduling barriers let nothing cross): four
-        // activation fragments are always in flight, a fragment register is refilled as soon as its two
-        // matrix instructions are issued, the activation scales of the tile arrive during its last four
-        // steps, the next tile's first fragments during the flush; in the first tile the conversion of
-        // step t+1 sits between the matrix instructions of step t.
-        v4i ring[4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) ring[t] = fragment(0, t);
-#pragma unroll
-        for (int j = 0; j < JT; ++j) {
-            const v8h am = *reinterpret_cast<const v8h *>(msb + (j * 32 + l32) * 32 + 16 * lh);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, mh, acc[j], 0, 0, 0);
-            acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, ml, acc[j], 0, 0, 0);
-        }
-        convert(0);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int j = 0; j < JT; ++j) {
-            v16i ilo, ihi;
-            v4i dq[4];
-#pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[t & 3], cl[t], t == 0 ? zi : ilo, 0, 0, 0);
-                ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[t & 3], ch[t], t == 0 ? zi : ihi, 0, 0, 0);
-                if (t < 4) ring[t & 3] = fragment(j, t + 4);
-                else dq[t - 4] = *reinterpret_cast<const v4i *>(dxs + j * 32 + 8 * (t - 4) + 4 * lh);
-                if (j == 0 && t < 7) convert(t + 1);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            if (j + 1 < JT) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) ring[t] = fragment(j + 1, t);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int v = 0; v < 16; ++v)
-                acc[j][v] = fmaf((float)((ihi[v] << 3) + ilo[v]), __int_as_float(dq[v >> 2][v & 3]) * dn, acc[j][v]);
-            __builtin_amdgcn_sched_barrier(0);
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t x = nib ? ((uint32_t)raw[c] >> 4) & 0x0f0f0f0fu : (uint32_t)raw[c] & 0x0f0f0f0fu;
+            cl[t][c] = (int)pk_mul_u16(x, sl);
+            ch[t][c] = (int)pk_mul_u16(x, sh);
         }
     };
 
-    request(0, 0);
-    sm.dx[0][tid & 127] = dxreg;
+    // ---- prologue: requests of super-block 0
+#pragma unroll
+    for (int c = 0; c < 5; ++c) request_strip(0, c);
+#pragma unroll
+    for (int p = 0; p < PA; ++p) request_act(0, 0, p);
+    request_ms(0, 0);
+    sm.dx[0][tid & 127] = dxbase_s[dxoffg];
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    for (int64_t sb = 0; sb < nb; ++sb) {
-        const int buf = (int)(sb & 1);
-        DirectB b;   // out of the strip: header of row l%32, then the lane's 64 nibble bytes
-        b.hdr = *reinterpret_cast<const v4i *>(park + l32 * 144);
+
+    // The two waves that share a SIMD (w and w+4) must not want the same pipe at the same time: the older one
+    // wins every arbitration and the younger one only gets what is left.  So they run the same super-block in
+    // opposite orders.  EARLY waves (0..3) convert the weights of a super-block at its start (vector work first,
+    // the conversion of step t+1 sits between the matrix instructions of step t of the first tile); LATE waves
+    // (4..7) convert the weights of the NEXT super-block at the end of the current one, after their last tile,
+    // so that they start every super-block with matrix work while their partner converts.
+    //
+    // Inside a super-block the order is pinned step by step (the scheduling barriers let nothing cross): four
+    // activation fragments are always in flight, a fragment register is refilled as soon as its two matrix
+    // instructions are issued, the activation scales of a tile arrive during its last four steps, the next
+    // tile's first fragments during the flush.  The requests for the next super-block are issued one per step
+    // in the tiles without conversion work: all waves asking at once right after the barrier only queue up in
+    // the memory pipeline.
+    auto run = [&](auto late_tag) {
+        constexpr bool LATE = decltype(late_tag)::value;
+        if (LATE) {   // weights of super-block 0, with nothing to overlap
+            read_header();
 #pragma unroll
-        for (int i = 0; i < 4; ++i) b.q[i] = *reinterpret_cast<const v4i *>(park + l32 * 144 + 16 + 64 * lh + 16 * i);
-        // the strip is about to be overwritten by the next request: its reads must have returned
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        // past the end the last super-block is requested again (into the idle buffer, never read)
-        request(sb + 1 < nb ? sb + 1 : nb - 1, buf ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
-        superblock(b, buf);
-        sm.dx[buf ^ 1][tid & 127] = dxreg;   // every thread stores (a repeated value past 128): no branch
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-    }
+            for (int t = 0; t < 8; ++t) convert(t, strip_piece(t));
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the strip is about to be overwritten
+        }
+        for (int64_t sb = 0; sb < nb; ++sb) {
+            const int buf = (int)(sb & 1);
+            const uint32_t sb_next = (uint32_t)(sb + 1 < nb ? sb + 1 : nb - 1);   // past the end: requested again, never used
+            v4i raw[4];
+            if (!LATE) {   // out of the strip: header of row l%32, then the lane's 64 nibble bytes
+                read_header();
+#pragma unroll
+                for (int i = 0; i < 4; ++i) raw[i] = *reinterpret_cast<const v4i *>(park + l32 * 144 + 16 + 64 * lh + 16 * i);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the strip is about to be overwritten
+            }
+            const float dxreg = dxbase_s[dxoffg + sb_next];
+            __builtin_amdgcn_sched_barrier(0);
+            const int8_t *ab = sm.a[buf];
+            const uint8_t *msb = reinterpret_cast<const uint8_t *>(sm.ms[buf]);
+            const float *dxs = sm.dx[buf];
+            auto fragment = [&](int j, int t) {
+                return *reinterpret_cast<const v4i *>(ab + j * 32 * 256 + (aoffl ^ (16 * t)));
+            };
+            v4i ring[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) ring[t] = fragment(0, t);
+            // ---- min term: -dmin*min of the 8 sub-blocks as fp16 high and low parts
+            const float dn = h2f((uint32_t)hdr[0] & 0xffffu) * kMinPrescale;   // exact: a power of two
+            {
+                const ScalesK4 sc = unpack_scales_k4((uint32_t)hdr[1], (uint32_t)hdr[2], (uint32_t)hdr[3]);
+                const float ndmin = -h2f((uint32_t)hdr[0] >> 16);
+                v8h mh, ml;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    _Float16 h, l;
+                    split_h(ndmin * (float)min_k4(sc, t), h, l);
+                    mh[t] = h;
+                    ml[t] = lh ? (_Float16)0.f : l;
+                }
+#pragma unroll
+                for (int j = 0; j < JT; ++j) {
+                    const v8h am = *reinterpret_cast<const v8h *>(msb + (j * 32 + l32) * 32 + 16 * lh);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, mh, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(am, ml, acc[j], 0, 0, 0);
+                }
+            }
+            if (!LATE) convert(0, raw[0]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < JT; ++j) {
+                v16i ilo, ihi;
+                v4i dq[4];
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[t & 3], cl[t], t == 0 ? zi : ilo, 0, 0, 0);
+                    ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(ring[t & 3], ch[t], t == 0 ? zi : ihi, 0, 0, 0);
+                    if (t < 4) ring[t & 3] = fragment(j, t + 4);
+                    else dq[t - 4] = *reinterpret_cast<const v4i *>(dxs + j * 32 + 8 * (t - 4) + 4 * lh);
+                    if (!LATE && j == 0 && t < 7) convert(t + 1, raw[2 * ((t + 1) >> 2) + ((t + 1) & 1)]);
+                    // requests for the next super-block, one per step: the strip first (its previous content was
+                    // read at the top of this trip by the early waves, at the end of the last one by the late waves)
+                    if (j == (LATE ? 0 : 1) && t < 5) request_strip(sb_next, t);
+                    if (j == (LATE ? 1 : 2) && (t & 1)) request_act(sb_next, buf ^ 1, t >> 1);
+                    if (j == (LATE ? 1 : 2) && t == 0) request_ms(sb_next, buf ^ 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (j + 1 < JT) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) ring[t] = fragment(j + 1, t);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    acc[j][v] = fmaf((float)((ihi[v] << 3) + ilo[v]), __int_as_float(dq[v >> 2][v & 3]) * dn, acc[j][v]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (LATE) {
+                // the next super-block's raw weights were requested at the top of this trip; of the requests
+                // made since then (four activation chunks; these waves load no min-term piece) none needs
+                // to have landed
+                asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+                read_header();
+#pragma unroll
+                for (int t = 0; t < 8; ++t) convert(t, strip_piece(t));
+            }
+            sm.dx[buf ^ 1][tid & 127] = dxreg;   // every thread stores (a repeated value past 128): no branch
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+    };
+    if (wave < 4) run(std::false_type{});
+    else run(std::true_type{});
 
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
     const int64_t n = n0 + wave * 32 + l32;
