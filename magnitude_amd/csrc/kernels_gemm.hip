@@ -370,7 +370,7 @@ __device__ __forceinline__ uint32_t byte_to_u16x2(uint32_t word, int i) {
 
 template <int NW>
 __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const WeightView w, const ActView a, int64_t M,
-                                                                        float *__restrict__ y) {
+                                                                        float *__restrict__ y, float *__restrict__ part) {
     constexpr int NT = 64 * NW, TN = 32 * NW;
     constexpr int PA = 1024 / NT;   // 16-byte activation pieces a thread moves per super-block
     extern __shared__ __align__(16) uint8_t smem_raw[];
@@ -504,17 +504,20 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const W
         }
     };
 
-    load_next(0);
-    store_next(0);
+    // a grid with gridDim.y > 1 cuts K: this workgroup does the super-blocks [sb_begin, sb_end) and writes a
+    // partial tile that sum_parts_kernel adds to the others in order
+    const int64_t sb_begin = nb * blockIdx.y / gridDim.y, sb_end = nb * (blockIdx.y + 1) / gridDim.y;
+    load_next(sb_begin);
+    store_next((int)(sb_begin & 1));
     __syncthreads();
-    for (int64_t sb = 0; sb < nb; ++sb) {
+    for (int64_t sb = sb_begin; sb < sb_end; ++sb) {
         const int buf = (int)(sb & 1);
         DirectB b;   // out of the strip: header of row l%32, then the lane's 64 nibble bytes
         b.hdr = *reinterpret_cast<const v4i *>(park + l32 * 144);
 #pragma unroll
         for (int i = 0; i < 4; ++i) b.q[i] = *reinterpret_cast<const v4i *>(park + l32 * 144 + 16 + 64 * lh + 16 * i);
         // past the end the last super-block is fetched again: unconditional loads keep the wait counters exact
-        load_next(sb + 1 < nb ? sb + 1 : nb - 1);
+        load_next(sb + 1 < sb_end ? sb + 1 : sb_end - 1);
         __builtin_amdgcn_sched_barrier(0);   // the loads stay ahead of the arithmetic they overlap with
         superblock(b, buf);
         store_next(buf ^ 1);
@@ -524,12 +527,13 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const W
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
     const int64_t n = n0 + wave * 32 + l32;
     const float inv = 1.0f / kMinPrescale;
+    float *out = gridDim.y > 1 ? part + (size_t)blockIdx.y * M * N : y;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < M && n < N) y[m * N + n] = acc[j][v] * inv;
+            if (m < M && n < N) out[m * N + n] = acc[j][v] * inv;
         }
     }
 }
@@ -831,6 +835,29 @@ hipError_t launch_per32(const WeightView &w, const ActView &a, int64_t M, float 
 }
 }  // namespace
 
+hipError_t launch_sum_parts(const float *part, int n_split, size_t n, float *y, hipStream_t s) {
+    const size_t n4 = n / 4;   // callers only split when n is a multiple of 4
+    hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, part, n_split, n4, y);
+    return hipGetLastError();
+}
+
+// K stretches for the kernels that take ggml-format activations (64-token x 128-row tiles, two workgroups per
+// compute unit = 512 places): below 384 tiles K is cut in 2, below 192 in 3, never under twelve super-blocks a
+// stretch (K = 4096 cut in two measured slower than whole: the pass that adds the partial tiles costs more
+// than the fuller grid gains).
+int q8k_tile_splits(int64_t K, int64_t M, int64_t N) {
+    static const int forced = getenv("QPROJ_Q8K_SPLITS") ? atoi(getenv("QPROJ_Q8K_SPLITS")) : 0;
+    const int64_t tiles = ((N + 127) / 128) * ((M + 63) / 64);
+    int n = forced > 0 ? forced : tiles >= 384 ? 1 : tiles >= 192 ? 2 : 3;
+    if ((M * N) % 4 != 0) n = 1;
+    while (n > 1 && K / 256 < 12 * n) --n;
+    return n;
+}
+size_t q8k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N) {
+    const int n = q8k_tile_splits(K, M, N);
+    return n > 1 ? (size_t)n * M * N * 4 : 0;
+}
+
 // A grid of fewer than 192 tiles leaves the 256 compute units (two workgroups each) mostly idle and a
 // workgroup's K loop is latency-bound: K is then cut into 2 or 3 stretches done by different workgroups.
 int per32_splits(int64_t K, int64_t M, int64_t N) {
@@ -858,13 +885,13 @@ hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, fl
 }
 
 // ggml-format activations (Q8_K planes in `a`, including the min-term plane), Q4_K weights, any M
-hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
+hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s) {
     if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || !a.msum || M <= 0) return hipErrorInvalidValue;
     if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 64 token rows of K bytes, 32 weight rows of K*144/256
     // large batches: 128 tokens x 256 weight rows per workgroup, one workgroup per compute unit
     static const int wide_env = getenv("QPROJ_Q8K_WIDE") ? atoi(getenv("QPROJ_Q8K_WIDE")) : -1;
     const int64_t wide_tiles = ((w.N + 255) / 256) * ((M + 127) / 128);
-    if (wide_env >= 0 ? wide_env != 0 : wide_tiles >= 256) {
+    if (wide_env >= 0 ? wide_env != 0 : wide_tiles >= 192) {
         using Smem = WideSmem<8>;
         const auto kern = &gemm_q4k_q8k_wide_kernel<8>;
         static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -878,8 +905,10 @@ hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, flo
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_direct_kernel<NW>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
     if (attr != hipSuccess) return attr;
-    const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64)));
-    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, w, a, M, y);
+    const int n_split = scratch ? q8k_tile_splits(w.K, M, w.N) : 1;
+    const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64)), (unsigned)n_split);
+    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, w, a, M, y, scratch);
+    if (n_split > 1) return launch_sum_parts(scratch, n_split, (size_t)M * w.N, y, s);
     return hipGetLastError();
 }
 

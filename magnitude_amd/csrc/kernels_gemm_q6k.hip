@@ -51,7 +51,7 @@ __device__ __forceinline__ long as_i64(uint32_t lo, uint32_t hi) { return (long)
 
 template <int NW, int JT>
 __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightView w, const ActView a, int64_t M,
-                                                                 float *__restrict__ y) {
+                                                                 float *__restrict__ y, float *__restrict__ part) {
     constexpr int NT = 64 * NW, TN = 32 * NW, TM = 32 * JT;
     constexpr int PA = TM * 16 / NT;   // 16-byte activation pieces a thread moves per super-block
     static_assert(PA >= 1 && TM * 2 <= NT, "tile does not fit the staging scheme");
@@ -235,14 +235,17 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
         }
     };
 
-    load_next(0);
-    store_next(0);
+    // a grid with gridDim.y > 1 cuts K: this workgroup does the super-blocks [sb_begin, sb_end) and writes a
+    // partial tile; the partial tiles are added in order afterwards
+    const int64_t sb_begin = nb * blockIdx.y / gridDim.y, sb_end = nb * (blockIdx.y + 1) / gridDim.y;
+    load_next(sb_begin);
+    store_next((int)(sb_begin & 1));
     __syncthreads();
-    for (int64_t sb = 0; sb < nb; ++sb) {
+    for (int64_t sb = sb_begin; sb < sb_end; ++sb) {
         const int buf = (int)(sb & 1);
         const uint32_t dbits = dcur;
         // past the end the last super-block is fetched again: unconditional loads keep the wait counters exact
-        load_next(sb + 1 < nb ? sb + 1 : nb - 1);
+        load_next(sb + 1 < sb_end ? sb + 1 : sb_end - 1);
         __builtin_amdgcn_sched_barrier(0);   // the loads stay ahead of the arithmetic they overlap with
         superblock(buf, dbits);
         __builtin_amdgcn_sched_barrier(0);   // the strips are read above and overwritten below
@@ -252,12 +255,13 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
 
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
     const int64_t n = n0 + wave * 32 + l32;
+    float *out = gridDim.y > 1 ? part + (size_t)blockIdx.y * M * N : y;
 #pragma unroll
     for (int j = 0; j < JT; ++j) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < M && n < N) y[m * N + n] = acc[j][v];
+            if (m < M && n < N) out[m * N + n] = acc[j][v];
         }
     }
 }
@@ -266,26 +270,29 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
 
 namespace {
 template <int NW, int JT>
-hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
+hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, int n_split, hipStream_t s) {
     using Smem = Q6Smem<NW, JT>;
     const auto kern = &gemm_q6k_q8k_kernel<NW, JT>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
     if (attr != hipSuccess) return attr;
-    const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 32 * JT - 1) / (32 * JT))));
-    hipLaunchKernelGGL(kern, grid, dim3(64 * NW), sizeof(Smem), s, w, a, M, y);
+    const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 32 * JT - 1) / (32 * JT))), (unsigned)n_split);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * NW), sizeof(Smem), s, w, a, M, y, scratch);
+    if (n_split > 1) return launch_sum_parts(scratch, n_split, (size_t)M * w.N, y, s);
     return hipGetLastError();
 }
 }  // namespace
 
 // ggml-format activations (Q8_K planes in `a`), Q6_K weights, any M
-hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, hipStream_t s) {
+hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s) {
     if (w.type != kTypeQ6_K || a.kind != kActKindQ8_K || !a.bsums || M <= 0) return hipErrorInvalidValue;
     if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 64 token rows of K bytes, 32 weight rows of K/2
-    // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit; 32-token tiles when
-    // the grid of 64-token tiles would leave compute units idle
-    if (((w.N + 127) / 128) * ((M + 63) / 64) >= 384) return launch_q6k<4, 2>(w, a, M, y, s);
-    return launch_q6k<4, 1>(w, a, M, y, s);
+    // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit.  A grid of such tiles that
+    // would leave compute units idle is filled by cutting K into stretches (partial tiles added afterwards);
+    // where K is too short for that, 32-token tiles double the number of workgroups instead.
+    const int n_split = scratch ? q8k_tile_splits(w.K, M, w.N) : 1;
+    if (n_split > 1 || ((w.N + 127) / 128) * ((M + 63) / 64) >= 384) return launch_q6k<4, 2>(w, a, M, y, scratch, n_split, s);
+    return launch_q6k<4, 1>(w, a, M, y, nullptr, 1, s);
 }
 
 }  // namespace qproj

@@ -259,13 +259,16 @@ size_t per32_scratch_max(int n, const qproj_weight *const *w, int64_t M) {   // 
 
 size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
     if (w[0]->type == kTypeQ8_0 && M >= 64 && w[0]->K % 128 == 0) return per32_scratch_max(n, w, M);   // tiled Q8_0 product
-    if (!use_mfma_kernel(w[0]->type, M, w[0]->K)) return 0;
+    size_t need = 0;
+    if (M > 16 && w[0]->type != kTypeQ8_0)   // tiled Q4_K / Q6_K products with K cut into stretches
+        for (int i = 0; i < n; ++i) need = std::max(need, q8k_tile_scratch_bytes(w[i]->K, M, w[i]->N));
+    if (!use_mfma_kernel(w[0]->type, M, w[0]->K)) return need;
     int64_t sum_n = 0, rgs = 0;
     for (int i = 0; i < n; ++i) {
         sum_n += w[i]->N;
         rgs += (w[i]->N + 31) / 32;
     }
-    size_t need = mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, std::min<int64_t>(M, 16), sum_n, rgs);
+    need = std::max(need, mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, std::min<int64_t>(M, 16), sum_n, rgs));
     if (M > 16 && M % 16) need = std::max(need, mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, M % 16, sum_n, rgs));
     return need;
 }
@@ -295,8 +298,8 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
     if (tiled(w[0])) {
         for (int i = 0; i < n; ++i) {
             const int t = w[0]->type;
-            QP_HIP(ctx, t == kTypeQ4_K   ? launch_gemm_q8k(w[i]->view, a, M, y[i], ctx->stream)
-                        : t == kTypeQ6_K ? launch_gemm_q6k_q8k(w[i]->view, a, M, y[i], ctx->stream)
+            QP_HIP(ctx, t == kTypeQ4_K   ? launch_gemm_q8k(w[i]->view, a, M, y[i], scratch, ctx->stream)
+                        : t == kTypeQ6_K ? launch_gemm_q6k_q8k(w[i]->view, a, M, y[i], scratch, ctx->stream)
                                          : launch_gemm_q8_0(w[i]->view, a, M, y[i], scratch, ctx->stream));
         }
         return QPROJ_OK;

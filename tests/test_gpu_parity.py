@@ -235,6 +235,24 @@ def test_mul_mat_ggml_mode_prefill_sized_batches(ctx, orc, qtype, m, k, n):
     w.free()
 
 
+@pytest.mark.parametrize("m,k,n", [(1000, 256, 6200), (900, 768, 6200)])
+def test_mul_mat_ggml_mode_q4k_wide_tiles(ctx, orc, m, k, n):
+    """Q4_K with enough 128-token x 256-row tiles (>= 192) to take the wide prefill kernel: one and three
+    super-blocks of K (the late-converting waves prepare a next super-block that does not exist after the
+    last), a ragged last token tile and a last column tile in which six of the eight waves have no rows."""
+    from magnitude_amd import ACT_GGML
+    blocks = make_weight(orc, Q4_K, n, k, seed=1700 + k + n)
+    rng = np.random.default_rng(m + k)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[:, rng.integers(0, k, 8)] *= 30.0
+    w = ctx.upload(Q4_K, k, n, blocks)
+    got = ctx.mul_mat(w, dev(x), ACT_GGML).cpu().numpy()
+    want = orc.mul_mat(Q4_K, blocks, k, x, orc.ACT_GGML)
+    close(got, want, 2e-5)
+    gate(got, want)
+    w.free()
+
+
 @pytest.mark.parametrize("qtype", TYPES)
 @pytest.mark.parametrize("m", [1, 3, 4, 6])
 def test_mul_mat_f32_mode_matches_fp64_dot(ctx, orc, qtype, m):
