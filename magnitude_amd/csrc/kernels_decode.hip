@@ -89,18 +89,6 @@ __device__ __forceinline__ void consume(const Raw<QT> (&raw)[R], float (&acc)[MT
                                         int g, int c, int nch, int nb, int n_rows, int64_t row_begin, int64_t N,
                                         float *y, int M, int lane) {
     constexpr int CH = Geo<QT>::kChunk;
-#ifdef QPROJ_PROBE_NOCOMPUTE
-    if (true) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const uint32_t *w = reinterpret_cast<const uint32_t *>(&raw[r]);
-            uint32_t x = 0;
-#pragma unroll
-            for (int i = 0; i < (int)(sizeof(Raw<QT>) / 4); ++i) x ^= w[i];
-            acc[0][r] += __int_as_float(x & 0x3fffff);
-        }
-    } else
-#endif
     if (lane_block<QT>((int64_t)c * CH, lane) < nb) {
         Frag<QT> f[R];
 #pragma unroll
@@ -178,10 +166,8 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     Raw<QT> buf_a[R], buf_b[R];
     issue<QT, R>(buf_a, rp, 0, 0, last_row, nb, lane);  // in flight while the activations are staged
 
-#ifndef QPROJ_PROBE_NOSTAGE
     stage_activations<QT, MT, FUSE>(smem, args, K, kpad);
     __syncthreads();
-#endif
 
     XTile xt;
     xt.qs = reinterpret_cast<const int8_t *>(smem);

@@ -204,8 +204,13 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
                 const int sb0 = 8 * f + 2 * k;   // sub-blocks sb0 (p = 0) and sb0 + 1 (p = 1) lie side by side in the tile
-                const int s0 = (int)(int8_t)((uint32_t)scv[sb0 >> 2] >> (8 * (sb0 & 3)));
-                const int s1 = (int)(int8_t)((uint32_t)scv[(sb0 + 1) >> 2] >> (8 * ((sb0 + 1) & 3)));
+                int s0 = (int)(int8_t)((uint32_t)scv[sb0 >> 2] >> (8 * (sb0 & 3)));
+                int s1 = (int)(int8_t)((uint32_t)scv[(sb0 + 1) >> 2] >> (8 * ((sb0 + 1) & 3)));
+                // The scales are made opaque registers on purpose: left to itself the compiler reads the byte
+                // straight out of the packed word with a sub-dword operand select, which only exists for the
+                // two-operand multiply, and then needs separate additions (1.5 instructions per product
+                // instead of one multiply-add).
+                asm volatile("" : "+v"(s0), "+v"(s1));
 #pragma unroll
                 for (int j = 0; j < JT; ++j) {
                     const v4i av = *reinterpret_cast<const v4i *>(ap + j * 32 * LA + 8 * sb0);
@@ -214,9 +219,13 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
                     const v16i i1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64((uint32_t)av[2], (uint32_t)av[3]),
                                                                           as_i64(wl[1][k], wh[1][k]), zi, 0, 0, 0);
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) isum[j][v] = __mul24(i0[v], s0) + isum[j][v];
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) isum[j][v] = __mul24(i1[v], s1) + isum[j][v];
+                    for (int v = 0; v < 16; ++v) {
+                        int t = __mul24(i0[v], s0) + isum[j][v];
+                        asm("" : "+v"(t));   // keeps the multiply-adds apart (see above: otherwise mul, mul, add3)
+                        t = __mul24(i1[v], s1) + t;
+                        asm("" : "+v"(t));
+                        isum[j][v] = t;
+                    }
                 }
             }
         }
