@@ -21,6 +21,7 @@
 #include "qproj_device.h"
 #include "qproj_internal.h"
 #include "gemm_tiles.h"
+#include "lds_direct.h"
 
 namespace qproj {
 
@@ -562,19 +563,6 @@ struct WideSmem {
     float dx[2][128];                // activation scale of the super-block
     uint8_t park[NW][5 * 1024];      // per wave: raw blocks of its 32 weight rows (4608 bytes used)
 };
-
-__device__ __forceinline__ void global_to_lds16(const void *g, void *l) {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
-                                     (__attribute__((address_space(3))) void *)l, 16, 0, 0);
-}
-// a wave-uniform pointer pinned to scalar registers: what is added to it afterwards stays a 32-bit lane
-// offset (scalar base + vector offset addressing) instead of becoming a 64-bit pointer per lane
-template <typename T>
-__device__ __forceinline__ const T *scalar_pointer(const T *p) {
-    const uint64_t v = reinterpret_cast<uint64_t>(p);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return reinterpret_cast<const T *>(((uint64_t)hi << 32) | lo);
-}
 
 template <int NW>
 __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const WeightView w, const ActView a, int64_t M,
