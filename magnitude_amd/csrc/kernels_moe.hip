@@ -8,73 +8,31 @@ namespace qproj {
 // indexes the pairs of expert e inside order[]; active[0..active[n_expert]) lists the experts that
 // have pairs, ascending.  Ids outside [0, n_expert) raise *error_flag and
 // their pairs are left out (their outputs are not written).  Pairs of one expert keep ascending
-// pair order so repeated runs produce the same launch geometry: the pair list is cut into S
-// segments, (expert, segment) tasks count their matches, a prefix over segments gives every task
-// its first slot, and a second scan places the pairs.
+// pair order so repeated runs produce the same launch geometry.  Each of the 16 waves takes every
+// 16th expert and sweeps the pair list 64 ids at a time (consecutive lanes on consecutive ids):
+// a ballot of the matches gives the count in the first sweep and, with the number of matching
+// lanes below one's own, the slot in the second.  (A version that read the ids from LDS inside the
+// sweeps was a chain of dependent loads: 19 us for 512 pairs and 128 experts.)
 constexpr int kGroupThreads = 1024;
 constexpr int kGroupLdsIds = 8192;   // pair ids staged in LDS up to this many, read from global beyond
 
-__global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t *__restrict__ ids, int n_pairs,
-                                                                  int n_expert, int S, int32_t *__restrict__ order,
-                                                                  int32_t *__restrict__ offsets,
-                                                                  int32_t *__restrict__ active,
-                                                                  int32_t *__restrict__ error_flag) {
-    extern __shared__ int32_t lds[];
-    int32_t *segcnt = lds;                     // [n_expert * S], then turned into first slots
-    int32_t *first = lds + n_expert * S;       // [n_expert + 1]
-    int32_t *wsum = first + n_expert + 1;      // [32] wave totals of the two scans
-    int32_t *sid = wsum + 32;                  // [min(n_pairs, kGroupLdsIds)]
+// cnt[e] = pairs of expert e on entry; on exit cnt[e] = offsets[e] = its first slot, active[] lists the
+// experts that have pairs.  All threads of the workgroup call it; the caller synchronizes afterwards.
+__device__ __forceinline__ void group_scan(int n_expert, int32_t *cnt, int32_t *wsum, int32_t *__restrict__ offsets,
+                                           int32_t *__restrict__ active) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const bool staged = n_pairs <= kGroupLdsIds;
-    bool bad = false;
-    for (int p = tid; p < n_pairs; p += kGroupThreads) {
-        const int e = ids[p];
-        bad |= e < 0 || e >= n_expert;
-        if (staged) sid[p] = e;
-    }
-    if (bad) atomicOr(error_flag, 1);
-    __syncthreads();
-    const int32_t *src = staged ? sid : ids;
-    const int seg_len = (n_pairs + S - 1) / S;
-    const int n_tasks = n_expert * S;
-    // pass 1: matches of (expert, segment); eight independent reads in flight per step
-    for (int t = tid; t < n_tasks; t += kGroupThreads) {
-        const int e = t / S, sg = t - e * S;
-        const int lo = min(sg * seg_len, n_pairs), hi = min(lo + seg_len, n_pairs);
-        int c = 0;
-        for (int p = lo; p < hi; p += 8) {
-            int v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = src[min(p + u, hi - 1)];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) c += (p + u < hi) & (v[u] == e);
-        }
-        segcnt[t] = c;
-    }
-    __syncthreads();
-    // segment counts -> running starts inside the expert; thread t owns experts [t * per, t * per + per)
+    // exclusive scans over the workgroup (shuffles inside a wave, wave totals through LDS) of the pair
+    // counts (-> offsets) and of the non-empty flags (-> compact list of the experts that have work);
+    // thread t owns experts [t * per, t * per + per)
     const int per = (n_expert + kGroupThreads - 1) / kGroupThreads;
-    int tot[8], local = 0;
+    int tot[8], local = 0, local_f = 0;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const int e = tid * per + i;
-        tot[i] = 0;
-        if (i < per && e < n_expert) {
-            int run = 0;
-            for (int sg = 0; sg < S; ++sg) {
-                const int c = segcnt[e * S + sg];
-                segcnt[e * S + sg] = run;
-                run += c;
-            }
-            tot[i] = run;
-        }
+        tot[i] = i < per && e < n_expert ? cnt[e] : 0;
         local += tot[i];
+        local_f += tot[i] > 0;
     }
-    // exclusive scans over the workgroup (shuffles inside a wave, wave totals through LDS) of the pair
-    // counts (-> offsets) and of the non-empty flags (-> compact list of the experts that have work)
-    int local_f = 0;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) local_f += tot[i] > 0;
     int incl = local, incl_f = local_f;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -98,7 +56,7 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
     for (int i = 0; i < 8; ++i) {
         const int e = tid * per + i;
         if (i < per && e < n_expert) {
-            first[e] = before;
+            cnt[e] = before;   // from here on: the expert's first slot
             offsets[e] = before;
             before += tot[i];
             if (tot[i] > 0) active[before_f++] = e;
@@ -108,30 +66,144 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
         offsets[n_expert] = before;
         active[n_expert] = before_f;   // how many experts have pairs
     }
-    __syncthreads();
-    // pass 2: placement, ascending pair order inside every expert
-    for (int t = tid; t < n_tasks; t += kGroupThreads) {
-        const int e = t / S, sg = t - e * S;
-        const int lo = min(sg * seg_len, n_pairs), hi = min(lo + seg_len, n_pairs);
-        int w = first[e] + segcnt[t];
-        for (int p = lo; p < hi; p += 8) {
-            int v[8];
+}
+
+template <bool STAGED>
+__device__ __forceinline__ void group_sweeps(const int32_t *__restrict__ ids, const int32_t *sid, int n_pairs, int n_expert,
+                                             int32_t *cnt, int32_t *wsum, int32_t *__restrict__ order,
+                                             int32_t *__restrict__ offsets, int32_t *__restrict__ active) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int kWaves = kGroupThreads / 64;
+    auto id_at = [&](int p) { return p < n_pairs ? (STAGED ? sid[p] : ids[p]) : -1; };
+    // A lane keeps the ids of its positions in registers, kHeld at a time (1024 pairs per wave and block),
+    // and runs through its experts on them: the sweeps are ballots on registers, not a chain of loads.
+    constexpr int kHeld = 16;
+    // sweep 1: pairs per expert (cnt starts at zero)
+    for (int base = 0; base < n_pairs; base += 64 * kHeld) {
+        int v[kHeld];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) v[u] = src[min(p + u, hi - 1)];
+        for (int u = 0; u < kHeld; ++u) v[u] = id_at(base + 64 * u + lane);
+        for (int e = wave; e < n_expert; e += kWaves) {
+            int c = 0;
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (p + u < hi && v[u] == e) order[w++] = p + u;
+            for (int u = 0; u < kHeld; ++u) c += __popcll(__ballot(v[u] == e));
+            if (lane == 0) cnt[e] += c;   // every expert belongs to one wave
         }
+    }
+    __syncthreads();
+    group_scan(n_expert, cnt, wsum, offsets, active);
+    __syncthreads();
+    // sweep 2: placement, ascending pair order inside every expert (cnt[e] = the expert's next free slot)
+    for (int base = 0; base < n_pairs; base += 64 * kHeld) {
+        int v[kHeld];
+#pragma unroll
+        for (int u = 0; u < kHeld; ++u) v[u] = id_at(base + 64 * u + lane);
+        for (int e = wave; e < n_expert; e += kWaves) {
+            int w = cnt[e];
+#pragma unroll
+            for (int u = 0; u < kHeld; ++u) {
+                const bool mine = v[u] == e;
+                const unsigned long long m = __ballot(mine);
+                if (mine)
+                    order[w + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0))] =
+                        base + 64 * u + lane;
+                w += __popcll(m);
+            }
+            if (lane == 0) cnt[e] = w;
+        }
+    }
+}
+
+// The sweeps above cost n_expert x n_pairs / 1024 steps.  Up to 8192 pairs (and while the table below fits
+// LDS) the work is made proportional to n_pairs instead: a wave takes 64 consecutive pairs, and 64 rounds of
+// "broadcast lane j's id, ballot who has the same" give every lane its rank among the equal ids of the block
+// and the size of its group; the first lane of a group files that size under blk[block][expert].  A prefix
+// over the blocks per expert, the scan over the experts, and every pair knows its slot:
+// first[expert] + blk[block][expert] + rank.
+constexpr int kBlocksPerWave = 8;   // 16 waves x 8 blocks x 64 = 8192 pairs
+
+__global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t *__restrict__ ids, int n_pairs,
+                                                                  int n_expert, int32_t *__restrict__ order,
+                                                                  int32_t *__restrict__ offsets,
+                                                                  int32_t *__restrict__ active,
+                                                                  int32_t *__restrict__ error_flag, int by_block) {
+    extern __shared__ int32_t lds[];
+    int32_t *cnt = lds;                 // [n_expert] pairs of the expert, then its first slot
+    int32_t *wsum = cnt + n_expert;     // [32] wave totals of the two scans
+    int32_t *tab = wsum + 32;           // by_block: blk[n_blocks][n_expert]; else the staged ids
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (!by_block) {
+        const bool staged = n_pairs <= kGroupLdsIds;
+        bool bad = false;
+        for (int p = tid; p < n_pairs; p += kGroupThreads) {
+            const int e = ids[p];
+            bad |= e < 0 || e >= n_expert;
+            if (staged) tab[p] = e;
+        }
+        for (int e = tid; e < n_expert; e += kGroupThreads) cnt[e] = 0;
+        if (bad) atomicOr(error_flag, 1);
+        __syncthreads();
+        if (staged) group_sweeps<true>(ids, tab, n_pairs, n_expert, cnt, wsum, order, offsets, active);
+        else group_sweeps<false>(ids, tab, n_pairs, n_expert, cnt, wsum, order, offsets, active);
+        return;
+    }
+    const int n_blocks = (n_pairs + 63) / 64;
+    int vid[kBlocksPerWave], rank[kBlocksPerWave];
+    bool bad = false;
+#pragma unroll
+    for (int i = 0; i < kBlocksPerWave; ++i) {   // the loads first: they travel while the table is cleared
+        const int p = 64 * (wave + 16 * i) + lane;
+        vid[i] = p < n_pairs ? ids[p] : -1;
+        bad |= p < n_pairs && (vid[i] < 0 || vid[i] >= n_expert);
+        if (vid[i] >= n_expert) vid[i] = -1;
+    }
+    for (int t = tid; t < n_blocks * n_expert; t += kGroupThreads) tab[t] = 0;
+    if (bad) atomicOr(error_flag, 1);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kBlocksPerWave; ++i) {
+        const int blk = wave + 16 * i;
+        if (blk < n_blocks) {   // wave-uniform
+            const int v = vid[i];
+            int r = 0, size = 0;
+            for (int j = 0; j < 64; ++j) {
+                const int ej = __builtin_amdgcn_readlane(v, j);
+                const unsigned long long m = __ballot(v == ej);
+                const int below = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
+                r = lane == j ? below : r;
+                size = lane == j ? __popcll(m) : size;
+            }
+            rank[i] = r;
+            if (r == 0 && v >= 0) tab[blk * n_expert + v] = size;
+        }
+    }
+    __syncthreads();
+    // per expert: group sizes of the blocks -> first slot of the block's group inside the expert; total
+    for (int e = tid; e < n_expert; e += kGroupThreads) {
+        int run = 0;
+        for (int b = 0; b < n_blocks; ++b) {
+            const int c = tab[b * n_expert + e];
+            tab[b * n_expert + e] = run;
+            run += c;
+        }
+        cnt[e] = run;
+    }
+    __syncthreads();
+    group_scan(n_expert, cnt, wsum, offsets, active);
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < kBlocksPerWave; ++i) {
+        const int blk = wave + 16 * i, v = vid[i];
+        if (blk < n_blocks && v >= 0) order[cnt[v] + tab[blk * n_expert + v] + rank[i]] = 64 * blk + lane;
     }
 }
 
 hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_expert, int32_t *order,
                             int32_t *offsets, int32_t *active, int32_t *error_flag, hipStream_t s) {
     if (n_expert > 8192 || n_pairs > 0x7fffffff) return hipErrorInvalidValue;
-    int S = (int)(kGroupThreads / n_expert);
-    if (S < 1) S = 1;
-    if (S > n_pairs) S = (int)(n_pairs > 0 ? n_pairs : 1);
-    const size_t lds = ((size_t)n_expert * S + n_expert + 1 + 32 + (n_pairs <= kGroupLdsIds ? n_pairs : 0)) * sizeof(int32_t);
+    const size_t table = (size_t)((n_pairs + 63) / 64) * (size_t)n_expert;
+    const bool by_block = n_pairs <= 64 * 16 * kBlocksPerWave && table <= 24 * 1024;   // at most 96 KB of LDS
+    const size_t lds = ((size_t)n_expert + 32 + (by_block ? table : n_pairs <= kGroupLdsIds ? (size_t)n_pairs : 0)) * sizeof(int32_t);
     static size_t allowed = 48 * 1024;
     if (lds > allowed) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(moe_group_kernel),
@@ -139,8 +211,8 @@ hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_exper
         if (e != hipSuccess) return e;
         allowed = lds;
     }
-    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(kGroupThreads), lds, s, ids, (int)n_pairs, (int)n_expert, S,
-                       order, offsets, active, error_flag);
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(kGroupThreads), lds, s, ids, (int)n_pairs, (int)n_expert,
+                       order, offsets, active, error_flag, by_block ? 1 : 0);
     return hipGetLastError();
 }
 

@@ -372,6 +372,26 @@ def test_mul_mat_id_matches_oracle(ctx, orc, moe, B):
     close(got, orc.mul_mat_id(Q4_K, moe["up"], k, n, E, xt, ids), 2e-5)
 
 
+@pytest.mark.parametrize("E,B", [(16, 600), (16, 1100), (512, 500)])
+def test_mul_mat_id_grouping_of_many_pairs(ctx, orc, E, B):
+    """The three ways the grouping pass sorts pairs by expert, on small expert matrices so that the oracle
+    stays quick: 4800 pairs (ranks inside blocks of 64 pairs, several blocks per wave), 8800 pairs (more
+    than the per-block path holds: sweeps over the ids in global memory) and 4000 pairs over 512 experts
+    (block table too large for LDS: sweeps over ids staged in LDS).  Experts get hundreds of rows each, so
+    the grouped kernel also runs its several-passes-per-expert loop."""
+    from magnitude_amd import ACT_GGML
+    k, n, top = 256, 32, 8
+    blocks = orc.quantize(Q4_K, (np.random.default_rng(E + B).standard_normal((E * n, k)) * 0.02).astype(np.float32)).reshape(E, n, -1)
+    rng = np.random.default_rng(7 * E + B)
+    ids, _ = routing(rng, B, top, E)
+    w = ctx.upload(Q4_K, k, n, blocks, n_expert=E)
+    x = rng.standard_normal((B, 1, k)).astype(np.float32)
+    got = ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML).cpu().numpy()
+    want = orc.mul_mat_id(Q4_K, blocks, k, n, E, x, ids)
+    close(got, want, 2e-5)
+    w.free()
+
+
 def test_mul_mat_id_reports_bad_expert_ids(ctx, orc, moe):
     from magnitude_amd import ACT_GGML, QprojError
     E, k, n = moe["E"], moe["d_model"], moe["d_ff"]
