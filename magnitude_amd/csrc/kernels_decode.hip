@@ -18,6 +18,8 @@ constexpr int kDecodeThreads = 1024;
 constexpr int kDecodeWaves = kDecodeThreads / 64;
 
 // activations into LDS: FUSE quantizes fp32 rows here; otherwise planes quantized earlier are copied
+constexpr int kPrefetchedChunks = 4;   // 256-wide pieces of activation row 0 a wave fetches ahead of its first weights (K up to 16384)
+
 template <int QT, int MT, bool FUSE>
 __device__ __forceinline__ void stage_activations(uint8_t *smem, const GemvArgs &args, int64_t K, int kpad,
                                                   const float4 *first = nullptr) {
@@ -34,7 +36,8 @@ __device__ __forceinline__ void stage_activations(uint8_t *smem, const GemvArgs 
             for (int ch = wave; ch < n_chunks; ch += kDecodeWaves) {
                 const int e0 = ch * 256 + 4 * lane;
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (first && m == 0 && ch == wave) v = *first;   // row 0's first chunk was fetched by the caller
+                if (first && m == 0 && ch < wave + kDecodeWaves * kPrefetchedChunks)
+                    v = first[(ch - wave) / kDecodeWaves];   // row 0's first chunks were fetched by the caller
                 else if (have && e0 < K) v = *reinterpret_cast<const float4 *>(x + e0);
                 if (QT == kTypeQ8_0) {
                     int s;
@@ -168,15 +171,19 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     // The wave's piece of the activation row is requested BEFORE the first weights: loads return in order, and
     // behind a step of weights coming from HBM the quantizing prologue would wait two microseconds for sixteen
     // bytes that sit in L2 (phase clocks: staging 3000-4400 cycles of a workgroup's 25000).
-    float4 x_first = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 x_first[kPrefetchedChunks];
     if (FUSE) {
-        const int e0 = wave * 256 + 4 * lane;
-        if (e0 < K) x_first = *reinterpret_cast<const float4 *>(args.x + e0);
+#pragma unroll
+        for (int i = 0; i < kPrefetchedChunks; ++i) {
+            const int e0 = (wave + kDecodeWaves * i) * 256 + 4 * lane;
+            x_first[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (e0 < K) x_first[i] = *reinterpret_cast<const float4 *>(args.x + e0);
+        }
     }
     Raw<QT> buf_a[R], buf_b[R];
     issue<QT, R>(buf_a, rp, 0, 0, last_row, nb, lane);  // in flight while the activations are staged
 
-    stage_activations<QT, MT, FUSE>(smem, args, K, kpad, FUSE ? &x_first : nullptr);
+    stage_activations<QT, MT, FUSE>(smem, args, K, kpad, FUSE ? x_first : nullptr);
     __syncthreads();
 
     XTile xt;
