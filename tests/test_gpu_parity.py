@@ -437,6 +437,76 @@ def test_moe_ffn_matches_oracle(ctx, orc, moe, B):
         close(gsep, gid, 2e-5)   # decode kernel vs grouped matrix-core kernel: same integer dots, other fp32 order
 
 
+# ---------------------------------------------------------------- replayed from a HIP graph
+
+def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):
+    """Serving loops replay the projections from HIP graphs.  Once the context's workspace has its size the
+    compute entry points only launch kernels, so a captured sequence must reproduce the eager results bit
+    for bit on every replay - with other eager work and synchronizations of the same context in between,
+    and with new activation values written into the same buffers.  Covered: the decode kernel (M = 1),
+    quantizer + small-batch kernel with K cut into chunks and the chunk sum (M = 8, Q6_K, K = 14336), the
+    tiled kernels with partial tiles added afterwards (M = 200, K = 14336), the MoE FFN with its grouping pass."""
+    from magnitude_amd import Context, ACT_GGML, ACT_Q8X32
+    stream = torch.cuda.Stream()
+    c = Context(0, stream=stream.cuda_stream)
+    try:
+        k, n = 4096, 256
+        w4 = c.upload(Q4_K, k, n, make_weight(orc, Q4_K, n, k, seed=1500 + k + n))
+        k6, n6 = 14336, 128
+        w6 = c.upload(Q6_K, k6, n6, make_weight(orc, Q6_K, n6, k6, seed=1500 + k6 + n6))
+        w4l = c.upload(Q4_K, k6, n6, make_weight(orc, Q4_K, n6, k6, seed=1500 + k6 + n6))
+        E, d_model, d_ff, top, B = moe["E"], moe["d_model"], moe["d_ff"], 8, 8
+        g = c.upload(Q4_K, d_model, d_ff, moe["gate"], n_expert=E)
+        u = c.upload(Q4_K, d_model, d_ff, moe["up"], n_expert=E)
+        d = c.upload(Q4_K, d_ff, d_model, moe["down"], n_expert=E)
+        rng = np.random.default_rng(77)
+        ids, wts = routing(rng, B, top, E)
+        ids_d, wts_d = dev(ids), dev(wts)
+        xs = {"dec": torch.empty((1, k), device="cuda"), "small": torch.empty((8, k6), device="cuda"),
+              "tiled": torch.empty((200, k6), device="cuda"), "moe": torch.empty((B, d_model), device="cuda")}
+        ys = {"dec": torch.empty((1, n), device="cuda"), "small": torch.empty((8, n6), device="cuda"),
+              "tiled6": torch.empty((200, n6), device="cuda"), "tiled4": torch.empty((200, n6), device="cuda"),
+              "per32": torch.empty((200, n6), device="cuda"), "moe": torch.empty((B, d_model), device="cuda")}
+
+        def fill(seed):
+            gen = torch.Generator(device="cuda").manual_seed(seed)
+            for t in xs.values():
+                t.copy_(torch.randn(t.shape, device="cuda", generator=gen))
+            torch.cuda.synchronize()
+
+        def calls():
+            c.mul_mat(w4, xs["dec"], ACT_GGML, out=ys["dec"], sync=False)
+            c.mul_mat(w6, xs["small"], ACT_GGML, out=ys["small"], sync=False)
+            c.mul_mat(w6, xs["tiled"], ACT_GGML, out=ys["tiled6"], sync=False)
+            c.mul_mat(w4l, xs["tiled"], ACT_GGML, out=ys["tiled4"], sync=False)
+            c.mul_mat(w4l, xs["tiled"], ACT_Q8X32, out=ys["per32"], sync=False)
+            c.moe_ffn(g, u, d, xs["moe"], ids_d, wts_d, ACT_GGML, out=ys["moe"], sync=False)
+
+        def eager(seed):
+            fill(seed)
+            calls()
+            c.sync()
+            return {name: t.clone() for name, t in ys.items()}
+
+        eager(1)                                   # sizes the workspace: nothing allocates during capture
+        graph = torch.cuda.CUDAGraph()
+        fill(2)
+        with torch.cuda.graph(graph, stream=stream):
+            calls()
+        for seed in (3, 4, 5):
+            want = eager(seed)                     # eager work of the same context between the replays
+            for t in ys.values():
+                t.zero_()
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for name, t in ys.items():
+                assert torch.equal(t, want[name]), f"replay with inputs {seed}: {name} differs from the eager call"
+            assert float(ys["moe"].abs().sum()) > 0
+    finally:
+        c.close()
+
+
 # ---------------------------------------------------------------- full benchmark sizes
 
 @pytest.mark.parametrize("qtype,k,n", [(Q4_K, 4096, 14336), (Q6_K, 14336, 4096), (Q8_0, 4096, 4096)])
