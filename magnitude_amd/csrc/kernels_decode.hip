@@ -18,7 +18,9 @@ constexpr int kDecodeThreads = 1024;
 constexpr int kDecodeWaves = kDecodeThreads / 64;
 
 // activations into LDS: FUSE quantizes fp32 rows here; otherwise planes quantized earlier are copied
-constexpr int kPrefetchedChunks = 4;   // 256-wide pieces of activation row 0 a wave fetches ahead of its first weights (K up to 16384)
+// 256-wide pieces of the activation rows a wave fetches ahead of its first weights: four registers' worth,
+// shared out over the rows (one row: K up to 16384 is covered, two rows: 8192, four rows: 4096)
+constexpr int kPrefetchedPieces = 4;
 
 template <int QT, int MT, bool FUSE>
 __device__ __forceinline__ void stage_activations(uint8_t *smem, const GemvArgs &args, int64_t K, int kpad,
@@ -36,8 +38,9 @@ __device__ __forceinline__ void stage_activations(uint8_t *smem, const GemvArgs 
             for (int ch = wave; ch < n_chunks; ch += kDecodeWaves) {
                 const int e0 = ch * 256 + 4 * lane;
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (first && m == 0 && ch < wave + kDecodeWaves * kPrefetchedChunks)
-                    v = first[(ch - wave) / kDecodeWaves];   // row 0's first chunks were fetched by the caller
+                constexpr int kPer = kPrefetchedPieces / MT;   // pieces per row the caller fetched
+                if (first && ch < wave + kDecodeWaves * kPer)
+                    v = first[m * kPer + (ch - wave) / kDecodeWaves];
                 else if (have && e0 < K) v = *reinterpret_cast<const float4 *>(x + e0);
                 if (QT == kTypeQ8_0) {
                     int s;
@@ -171,14 +174,17 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     // The wave's piece of the activation row is requested BEFORE the first weights: loads return in order, and
     // behind a step of weights coming from HBM the quantizing prologue would wait two microseconds for sixteen
     // bytes that sit in L2 (phase clocks: staging 3000-4400 cycles of a workgroup's 25000).
-    float4 x_first[kPrefetchedChunks];
+    float4 x_first[kPrefetchedPieces];
     if (FUSE) {
+        constexpr int kPer = kPrefetchedPieces / MT;
 #pragma unroll
-        for (int i = 0; i < kPrefetchedChunks; ++i) {
-            const int e0 = (wave + kDecodeWaves * i) * 256 + 4 * lane;
-            x_first[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (e0 < K) x_first[i] = *reinterpret_cast<const float4 *>(args.x + e0);
-        }
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) {
+                const int e0 = (wave + kDecodeWaves * i) * 256 + 4 * lane;
+                x_first[m * kPer + i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (m < args.M && e0 < K) x_first[m * kPer + i] = *reinterpret_cast<const float4 *>(args.x + (int64_t)m * K + e0);
+            }
     }
     Raw<QT> buf_a[R], buf_b[R];
     issue<QT, R>(buf_a, rp, 0, 0, last_row, nb, lane);  // in flight while the activations are staged
