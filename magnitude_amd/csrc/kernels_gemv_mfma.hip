@@ -59,6 +59,7 @@ struct MfmaArgs {
     int n_expert;
     int x_div;             // activation row of pair p is p / x_div
     int wgs_per_expert;
+    int rg_loop;           // row groups a wave works through one after the other (the staged rows are reused)
     // pair mode (ids non-null): workgroup set s serves pair s alone with expert ids[s]; no order / offsets / active
     const int32_t *ids;
     int n_pairs;
@@ -551,16 +552,18 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
 
     // wave -> (row group, K part)
     const int rgl = wave / g.kw, kp = wave - rgl * g.kw;
-    const int row0 = (rs * g.rw + rgl) * 32;
     const int part_sb = (nsb + g.kw - 1) / g.kw;
     const int s0 = min(kp * part_sb, nsb), s1 = min(s0 + part_sb, nsb);  // range inside the staged chunk
-    const bool rows_ok = row0 < N;
-    const int steps = rows_ok ? s1 - s0 : 0;
-    const int items = NT * steps;                       // (tensor, super-block) pairs this wave streams
-    const int last_sb = c0 + (steps > 0 ? s1 - 1 : 0);  // loads past the range repeat its last super-block
-
+    int row0 = 0, steps = 0, items = 0, last_sb = c0;
+    bool rows_ok = false;
     Stager<QT> sa, sb_;
-    {
+    // the wave's rg-th row group: rows, how much of K, where its blocks start
+    auto set_rowgroup = [&](int rg) {
+        row0 = ((rs * g.rg_loop + rg) * g.rw + rgl) * 32;
+        rows_ok = row0 < N;
+        steps = rows_ok ? s1 - s0 : 0;
+        items = NT * steps;                       // (tensor, super-block) pairs this wave streams
+        last_sb = c0 + (steps > 0 ? s1 - 1 : 0);  // loads past the range repeat its last super-block
         const int64_t row = (int64_t)expert * N + (rows_ok ? row0 : 0);
         sa.rebase(0, w, row);
         sa.rebase(1, SWIGLU ? g.t[1].w : w, row);
@@ -568,7 +571,7 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
         sb_.rebase(0, w, row);
         sb_.rebase(1, SWIGLU ? g.t[1].w : w, row);
         sb_.init(w, rows_ok ? min(31, N - 1 - row0) : 0, lane);
-    }
+    };
     // item i -> tensor i / steps, super-block c0 + s0 + i % steps (clamped: harmless repeats past the end)
     auto issue = [&](Stager<QT> &st, int i) {
         const int t = SWIGLU && steps > 0 && i >= steps ? 1 : 0;
@@ -578,23 +581,29 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
     int *map = reinterpret_cast<int *>(smem + L.off_map);
 
     // dense launches stage all (<= MT) rows at once; an expert with more than MT pairs takes several passes
-    for (int m0 = 0; m0 < (GROUPED ? n_rows : 1); m0 += MT) {
+    for (int m0 = 0; m0 < (GROUPED ? n_rows : 1); m0 += MT)
+    for (int rg = 0; rg < g.rg_loop; ++rg) {   // the rows staged for this pass serve all of the wave's row groups
         const int m_cnt = min(MT, n_rows - m0);
+        set_rowgroup(rg);
         issue(sa, 0);
         issue(sb_, 1);
-        if constexpr (GROUPED) {
-            if (m0 > 0) __syncthreads();   // the previous pass is done with the staged rows and the regions
-            if ((int)threadIdx.x < MT)
-                map[threadIdx.x] = (int)threadIdx.x >= m_cnt ? 0
-                                   : g.ids      ? pair0 + m0 + (int)threadIdx.x
-                                                : g.order[pair0 + m0 + (int)threadIdx.x];
+        if (rg == 0) {
+            if constexpr (GROUPED) {
+                if (m0 > 0) __syncthreads();   // the previous pass is done with the staged rows and the regions
+                if ((int)threadIdx.x < MT)
+                    map[threadIdx.x] = (int)threadIdx.x >= m_cnt ? 0
+                                       : g.ids      ? pair0 + m0 + (int)threadIdx.x
+                                                    : g.order[pair0 + m0 + (int)threadIdx.x];
+                __syncthreads();
+            }
+            if (g.x)
+                stage_quantize<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
+            else
+                stage_activations<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
             __syncthreads();
+        } else if (g.kw > 1) {
+            __syncthreads();   // the partial tiles the previous row group left in the regions have been summed
         }
-        if (g.x)
-            stage_quantize<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
-        else
-            stage_activations<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
-        __syncthreads();
 
         float out[NT][NV];
 #pragma unroll
@@ -767,6 +776,7 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s)
     g.chunk_sb = p.chunk_sb;
     g.kw = p.kw;
     g.rw = W / p.kw;
+    g.rg_loop = 1;
     int wg = 0;
     size_t part_off = 0;
     for (int i = 0; i < args.n_targets; ++i) {
@@ -815,7 +825,21 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
         g.t[i].w = args.t[i].w;
         g.t[i].y = args.t[i].y;
     }
-    g.wgs_per_expert = (int)((rg_e + g.rw - 1) / g.rw);
+    // Short K makes a row group a few steps of work against a prologue (row map, staged rows, barriers) of
+    // several microseconds.  A wave can take two row groups in a row and pay the prologue once; measured on
+    // the 128-expert FFN's down projection (K = 768): worth it for a grid of one to three workgroups per
+    // compute unit (416 workgroups: the FFN at B = 8 goes from 61.6 to 55.3 us), neutral above (992
+    // workgroups, B = 64), harmful below (64 workgroups, B = 1: 24 -> 31 us), and four in a row always lose.
+    static const int forced_loop = getenv("QPROJ_MOE_RG_LOOP") ? atoi(getenv("QPROJ_MOE_RG_LOOP")) : 0;
+    {
+        const int64_t wgs1 = (args.ids ? n_pairs : std::min<int64_t>(w.E, n_pairs)) * ((rg_e + g.rw - 1) / g.rw);
+        const int64_t cus = 256;
+        int loop = forced_loop > 0 ? forced_loop : (wgs1 > cus && wgs1 <= 3 * cus) ? 2 : 1;
+        loop = (int)std::min<int64_t>(loop, std::max<int64_t>(1, rg_e / g.rw));
+        while (loop > 1 && rg_e % ((int64_t)g.rw * loop) != 0) --loop;   // no half-empty last workgroup
+        g.rg_loop = std::min(loop, 8);
+    }
+    g.wgs_per_expert = (int)((rg_e + (int64_t)g.rw * g.rg_loop - 1) / ((int64_t)g.rw * g.rg_loop));
     g.n_expert = (int)w.E;
     g.ids = args.ids;
     g.n_pairs = args.n_pairs;
