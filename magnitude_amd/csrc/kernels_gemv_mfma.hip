@@ -559,7 +559,7 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
     Stager<QT> sa, sb_;
     // the wave's rg-th row group: rows, how much of K, where its blocks start
     auto set_rowgroup = [&](int rg) {
-        row0 = ((rs * g.rg_loop + rg) * g.rw + rgl) * 32;
+        row0 = ((rs * (GROUPED ? g.rg_loop : 1) + rg) * g.rw + rgl) * 32;
         rows_ok = row0 < N;
         steps = rows_ok ? s1 - s0 : 0;
         items = NT * steps;                       // (tensor, super-block) pairs this wave streams
@@ -582,7 +582,7 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
 
     // dense launches stage all (<= MT) rows at once; an expert with more than MT pairs takes several passes
     for (int m0 = 0; m0 < (GROUPED ? n_rows : 1); m0 += MT)
-    for (int rg = 0; rg < g.rg_loop; ++rg) {   // the rows staged for this pass serve all of the wave's row groups
+    for (int rg = 0; rg < (GROUPED ? g.rg_loop : 1); ++rg) {   // the rows staged for this pass serve all of the wave's row groups
         const int m_cnt = min(MT, n_rows - m0);
         set_rowgroup(rg);
         issue(sa, 0);
