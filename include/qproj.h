@@ -108,6 +108,20 @@ size_t qproj_act_bytes(int kind, int wtype, int64_t M, int64_t K);
 int qproj_quantize_activations(qproj_ctx *ctx, int kind, int wtype, const float *x_dev, int64_t M,
                                int64_t K, void *out_dev);
 
+/* The two graph nodes llama.cpp puts in front of every attention and feed-forward block (build_norm with
+ * LLM_NORM_RMS: GGML_OP_RMS_NORM, then GGML_OP_MUL by the norm weights), reached like everything else here
+ * through context.decode (/root/reference/inference/crates/icn-engine/src/lib.rs:2264):
+ *   y[m][k] = (x[m][k] * (1 / sqrtf(mean_k(x[m]^2) + eps))) * gamma[k],   mean taken in double.
+ * gamma_dev may be null (the norm alone).  K a multiple of 32. */
+int qproj_rms_norm(qproj_ctx *ctx, const float *x_dev, const float *gamma_dev, float eps, int64_t M, int64_t K,
+                   float *y_dev);
+
+/* qproj_rms_norm followed by qproj_quantize_activations in one launch: the normalised rows go straight from
+ * registers into the activation planes (same bytes as the two calls one after the other) and feed
+ * qproj_mul_mat_quantized.  The per-32 format needs K % 256 == 0 here. */
+int qproj_rms_norm_quantize(qproj_ctx *ctx, int kind, int wtype, const float *x_dev, const float *gamma_dev,
+                            float eps, int64_t M, int64_t K, void *out_dev);
+
 /* GGML_OP_MUL_MAT: y_dev[M][N] = x_dev[M][K] . W^T.  Picks the decode (M=1), small-batch
  * (M<=16) or prefill kernel from M.  W must have n_expert == 1. */
 int qproj_mul_mat(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int64_t M, float *y_dev,

@@ -13,21 +13,7 @@ __global__ __launch_bounds__(256) void quant_q8k_kernel(const float *__restrict_
     const int lane = threadIdx.x & 63;
     if (sb >= n_super) return;  // whole wave leaves together
     const float4 v = reinterpret_cast<const float4 *>(x + sb * 256)[lane];
-    int bsum;
-    float dd;
-    const uint32_t packed = wave_quantize_q8k(v, lane, bsum, dd);
-    reinterpret_cast<uint32_t *>(qs + sb * 256)[lane] = packed;
-    if ((lane & 3) == 0) bsums[sb * 16 + (lane >> 2)] = (int16_t)bsum;
-    if (lane == 0) d[sb] = dd;
-    // d * (sum over a 32-wide sub-block), split into two fp16 parts, in the order the prefill
-    // kernel feeds them to the fp16 matrix instruction
-    const int pair = bsum + __shfl_xor(bsum, 4);
-    if ((lane & 7) == 0) {
-        const float v = dd * (float)pair * kMinPrescale;
-        const _Float16 hi = (_Float16)v, lo = (_Float16)(v - (float)hi);
-        msum[sb * 16 + (lane >> 3)] = __builtin_bit_cast(uint16_t, hi);
-        msum[sb * 16 + 8 + (lane >> 3)] = __builtin_bit_cast(uint16_t, lo);
-    }
+    wave_store_q8k(v, lane, sb, qs, d, bsums, msum);
 }
 
 // FP16_SCALE: ggml Q8_0 blocks (scale rounded through fp16).  Otherwise the prefill format:
@@ -44,24 +30,7 @@ __global__ __launch_bounds__(256) void quant_q8_32_kernel(const float *__restric
     const bool live = e0 < n_elems;  // rows are multiples of 32, so a block is all in or all out
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (live) v = *reinterpret_cast<const float4 *>(x + e0);
-    int s;
-    float dd;
-    const uint32_t packed = wave_quantize_q8_32(v, s, dd);
-    if (!live) return;
-    *reinterpret_cast<uint32_t *>(qs + e0) = packed;
-    if ((lane & 7) == 0) {
-        const int64_t b = e0 >> 5;
-        d[b] = FP16_SCALE ? h2f(f2h(dd)) : dd;
-        if (!FP16_SCALE) {
-            isum[b] = s;
-            // d * (sum of the block's codes), split into two fp16 parts, in the order the prefill kernel
-            // feeds them to the fp16 matrix instruction: per 256 elements 8 high parts, then 8 low parts
-            const float v = dd * (float)s * kMinPrescale;
-            const _Float16 hi = (_Float16)v, lo = (_Float16)(v - (float)hi);
-            msum[ch * 16 + (lane >> 3)] = __builtin_bit_cast(uint16_t, hi);
-            msum[ch * 16 + 8 + (lane >> 3)] = __builtin_bit_cast(uint16_t, lo);
-        }
-    }
+    wave_store_q8_32<FP16_SCALE>(v, lane, e0, ch, live, qs, d, isum, msum);
 }
 
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,

@@ -549,6 +549,35 @@ int qproj_quantize_activations(qproj_ctx *ctx, int kind, int wtype, const float 
     return QPROJ_OK;
 }
 
+int qproj_rms_norm(qproj_ctx *ctx, const float *x_dev, const float *gamma_dev, float eps, int64_t M, int64_t K,
+                   float *y_dev) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (!x_dev || !y_dev) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_rms_norm: null argument");
+    if (M < 0 || K <= 0 || K % 32 != 0) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_rms_norm: K must be a positive multiple of 32");
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    QP_HIP(ctx, launch_rms_norm(-1, x_dev, gamma_dev, eps, M, K, y_dev, nullptr, nullptr, nullptr, nullptr, nullptr, ctx->stream));
+    return QPROJ_OK;
+}
+
+int qproj_rms_norm_quantize(qproj_ctx *ctx, int kind, int wtype, const float *x_dev, const float *gamma_dev, float eps,
+                            int64_t M, int64_t K, void *out_dev) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (!x_dev || !out_dev) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_rms_norm_quantize: null argument");
+    if (qproj_act_bytes(kind, wtype, M, K) == 0)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_rms_norm_quantize: bad kind or shape");
+    const int k = act_kind_for(kind, wtype);
+    if (k == kActKindQ8X32 && K % 256 != 0)
+        return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_rms_norm_quantize: the per-32 format needs K % 256 == 0 here");
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    const ActPlanes p = act_planes(k, M, K);
+    uint8_t *base = static_cast<uint8_t *>(out_dev);
+    QP_HIP(ctx, launch_rms_norm(k, x_dev, gamma_dev, eps, M, K, nullptr, reinterpret_cast<int8_t *>(base + p.off_qs),
+                                reinterpret_cast<float *>(base + p.off_d), reinterpret_cast<int16_t *>(base + p.off_aux),
+                                reinterpret_cast<uint16_t *>(base + p.off_msum),
+                                reinterpret_cast<int32_t *>(base + p.off_aux), ctx->stream));
+    return QPROJ_OK;
+}
+
 int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
                         float *const *y_dev, int act) {
     if (!ctx) return QPROJ_ERR_INVALID_ARG;

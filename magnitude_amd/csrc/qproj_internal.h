@@ -82,6 +82,9 @@ hipError_t launch_dequantize(const WeightView &w, float *out, hipStream_t s);
 hipError_t launch_repack_to_planes(int type, const uint8_t *gguf, uint8_t *planes_base, const WeightView &w,
                                    int64_t n_blocks, hipStream_t s);
 hipError_t launch_repack_to_gguf(int type, const WeightView &w, uint8_t *gguf, int64_t n_blocks, hipStream_t s);
+// RMS_NORM + MUL by the norm weights (gamma may be null); kind < 0: fp32 rows to y, otherwise the planes of `kind`
+hipError_t launch_rms_norm(int kind, const float *x, const float *gamma, float eps, int64_t M, int64_t K, float *y,
+                           int8_t *qs, float *d, int16_t *bsums, uint16_t *msum, int32_t *isum, hipStream_t s);
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
                                int16_t *bsums, uint16_t *msum, int32_t *isum, hipStream_t s);
 hipError_t launch_gemv_q8act(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);

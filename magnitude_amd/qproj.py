@@ -47,6 +47,8 @@ SYMBOLS = {
     "qproj_dequantize": (_i32, [_vp, _vp, _vp]),
     "qproj_act_bytes": (_sz, [_i32, _i32, _i64, _i64]),
     "qproj_quantize_activations": (_i32, [_vp, _i32, _i32, _vp, _i64, _i64, _vp]),
+    "qproj_rms_norm": (_i32, [_vp, _vp, _vp, C.c_float, _i64, _i64, _vp]),
+    "qproj_rms_norm_quantize": (_i32, [_vp, _i32, _i32, _vp, _vp, C.c_float, _i64, _i64, _vp]),
     "qproj_mul_mat": (_i32, [_vp, _vp, _vp, _i64, _vp, _i32]),
     "qproj_mul_mat_multi": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i64, C.POINTER(_vp), _i32]),
     "qproj_mul_mat_quantized": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i32, _i64, C.POINTER(_vp)]),
@@ -248,6 +250,38 @@ class Context:
         if sync:
             self.sync()
         return ys
+
+    def rms_norm(self, x: torch.Tensor, gamma: Optional[torch.Tensor], eps: float,
+                 out: Optional[torch.Tensor] = None, sync: bool = True) -> torch.Tensor:
+        """GGML_OP_RMS_NORM followed by GGML_OP_MUL with the norm weights (gamma None: the norm alone)."""
+        x = x.contiguous()
+        m, k = x.shape
+        y = out if out is not None else torch.empty_like(x)
+        if sync:
+            torch.cuda.current_stream().synchronize()
+        self._check(self.lib.qproj_rms_norm(self.handle, _ptr(x), 0 if gamma is None else _ptr(gamma.contiguous()),
+                                            C.c_float(eps), m, k, _ptr(y)))
+        if sync:
+            self.sync()
+        return y
+
+    def rms_norm_quantize_raw(self, x: torch.Tensor, gamma: Optional[torch.Tensor], eps: float, kind: int, wtype: int,
+                              out: Optional[torch.Tensor] = None, sync: bool = True) -> torch.Tensor:
+        """Norm, weight multiply and activation quantizer in one launch; the buffer feeds mul_mat_quantized."""
+        x = x.contiguous()
+        m, k = x.shape
+        nbytes = int(self.lib.qproj_act_bytes(kind, wtype, m, k))
+        if nbytes == 0:
+            raise ValueError("bad activation shape or kind")
+        buf = out if out is not None else torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        if sync:
+            torch.cuda.current_stream().synchronize()
+        self._check(self.lib.qproj_rms_norm_quantize(self.handle, kind, wtype, _ptr(x),
+                                                     0 if gamma is None else _ptr(gamma.contiguous()),
+                                                     C.c_float(eps), m, k, _ptr(buf)))
+        if sync:
+            self.sync()
+        return buf
 
     def quantize_activations_raw(self, x: torch.Tensor, kind: int, wtype: int,
                                  out: Optional[torch.Tensor] = None, sync: bool = True) -> torch.Tensor:

@@ -75,6 +75,8 @@ def lib() -> C.CDLL:
         L.orc_moe_ffn.argtypes = [i32, i32, vp, vp, vp, i64, i64, i64, f32p, vp, f32p, i64, i64,
                                   f32p, i32, i32]
         L.orc_time_mul_mat.restype = C.c_double
+        L.orc_rms_norm.argtypes = [vp, vp, C.c_float, i64, i64, vp]
+        L.orc_rms_norm.restype = None
         L.orc_time_mul_mat.argtypes = [i32, vp, i64, i64, f32p, i64, f32p, i32, i32, i32]
         L.orc_max_threads.restype = i32
         _lib = L
@@ -209,6 +211,16 @@ def time_mul_mat(qtype: int, w: np.ndarray, k: int, x: np.ndarray, act: int, nth
     m = x.shape[0]
     y = np.empty((m, n), dtype=np.float32)
     return float(lib().orc_time_mul_mat(qtype, _p(w), k, n, _p(x), m, _p(y), act, nthreads, reps))
+
+
+def rms_norm(x: np.ndarray, gamma, eps: float) -> np.ndarray:
+    """RMS_NORM then MUL by the norm weights, row by row (gamma None: the norm alone)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    m, k = x.shape
+    y = np.empty_like(x)
+    g = None if gamma is None else np.ascontiguousarray(gamma, dtype=np.float32)
+    lib().orc_rms_norm(_p(x), 0 if g is None else _p(g), C.c_float(eps), m, k, _p(y))
+    return y
 
 
 def max_threads() -> int:

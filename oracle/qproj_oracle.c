@@ -861,3 +861,22 @@ double orc_time_mul_mat(int type, const void *w, int64_t K, int64_t N, const flo
     clock_gettime(CLOCK_MONOTONIC, &t1);
     return (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
 }
+
+/* ggml-cpu ops.cpp ggml_compute_forward_rms_norm_f32: the squares are formed in float and summed in
+ * ggml_float (double), the mean goes back to float before eps is added, the row is scaled in place
+ * (ggml_vec_scale_f32), and the multiplication by the norm weights is a separate GGML_OP_MUL node,
+ * i.e. a second rounding. */
+void orc_rms_norm(const float *x, const float *gamma, float eps, int64_t M, int64_t K, float *y) {
+    for (int64_t m = 0; m < M; ++m) {
+        const float *xr = x + m * K;
+        float *yr = y + m * K;
+        double sum = 0.0;
+        for (int64_t k = 0; k < K; ++k) sum += (double)(xr[k] * xr[k]);
+        const float mean = (float)(sum / (double)K);
+        const float scale = 1.0f / sqrtf(mean + eps);
+        for (int64_t k = 0; k < K; ++k) {
+            const float v = xr[k] * scale;
+            yr[k] = gamma ? v * gamma[k] : v;
+        }
+    }
+}

@@ -38,6 +38,13 @@
  *   fp32 association in vec_dot . follows ggml's generic C code; ggml's own
  *                                 SIMD paths associate differently, so GPU
  *                                 comparisons use a tolerance, integers exact.
+ *   rms_norm (+ weight multiply) . PARITY UNPINNED against ggml (the double-precision
+ *                                 sum of float squares and the two roundings of
+ *                                 x*scale*weight are recalled from ggml-cpu's
+ *                                 ggml_compute_forward_rms_norm_f32 and ggml_mul;
+ *                                 no reference-held vector exists); pinned by what
+ *                                 the mathematics fixes: closed forms on constant
+ *                                 and one-hot rows, scale invariance, fp64 brute force.
  */
 #ifndef QPROJ_ORACLE_H
 #define QPROJ_ORACLE_H
@@ -126,6 +133,11 @@ int orc_moe_ffn(int type_gate_up, int type_down, const void *gate, const void *u
 double orc_time_mul_mat(int type, const void *w, int64_t K, int64_t N, const float *x, int64_t M,
                         float *y, int act, int nthreads, int reps);
 int orc_max_threads(void);
+
+/* GGML_OP_RMS_NORM followed by GGML_OP_MUL with the norm weights (llama.cpp build_norm, LLM_NORM_RMS):
+ * per row  sum = sum_k (double)(x[k]*x[k]);  scale = 1/sqrtf((float)(sum/K) + eps);
+ *          y[k] = (x[k]*scale) * gamma[k]      (gamma may be NULL: plain RMS_NORM) */
+void orc_rms_norm(const float *x, const float *gamma, float eps, int64_t M, int64_t K, float *y);
 
 #ifdef __cplusplus
 }

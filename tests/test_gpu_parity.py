@@ -437,6 +437,74 @@ def test_moe_ffn_matches_oracle(ctx, orc, moe, B):
         close(gsep, gid, 2e-5)   # decode kernel vs grouped matrix-core kernel: same integer dots, other fp32 order
 
 
+# ---------------------------------------------------------------- RMS norm in front of the projections
+
+@pytest.mark.parametrize("m,k", [(1, 4096), (5, 14336), (3, 20480), (7, 288), (64, 4096)])
+def test_rms_norm_matches_oracle(ctx, orc, m, k):
+    """RMS_NORM + MUL by the norm weights: the sum of squares is taken in double on both sides and only
+    its order differs (a different last bit of the double can move the float scale by one ulp once in a
+    few hundred thousand rows), every other step is the same float operation: equal to the last bit here."""
+    rng = np.random.default_rng(m * 31 + k)
+    x = (rng.standard_normal((m, k)) * rng.uniform(0.05, 20.0, (m, 1))).astype(np.float32)
+    g = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    got = ctx.rms_norm(dev(x), dev(g), 1e-5).cpu().numpy()
+    np.testing.assert_array_max_ulp(got, orc.rms_norm(x, g, 1e-5), maxulp=1)
+    got = ctx.rms_norm(dev(x), None, 1e-6).cpu().numpy()
+    np.testing.assert_array_max_ulp(got, orc.rms_norm(x, None, 1e-6), maxulp=1)
+
+
+@pytest.mark.parametrize("m,k", [(1, 4096), (5, 14336), (3, 20480), (130, 4096)])
+@pytest.mark.parametrize("qtype", [Q4_K, Q8_0])
+def test_rms_norm_quantize_writes_the_bytes_of_the_two_calls(ctx, orc, qtype, m, k):
+    """The fused launch must leave exactly the activation planes that qproj_rms_norm followed by
+    qproj_quantize_activations leaves (all planes, compared as raw bytes), for ggml's format of the
+    weight type and for the per-32 prefill format; a projection fed from them equals the unfused one."""
+    from magnitude_amd import ACT_GGML, ACT_Q8X32
+    rng = np.random.default_rng(m * 17 + k + qtype)
+    x = dev((rng.standard_normal((m, k)) * rng.uniform(0.05, 20.0, (m, 1))).astype(np.float32))
+    g = dev((1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32))
+    normed = ctx.rms_norm(x, g, 1e-5)
+    for kind in ([ACT_GGML, ACT_Q8X32] if qtype == Q4_K else [ACT_GGML]):
+        two = ctx.quantize_activations_raw(normed, kind, qtype)
+        one = ctx.rms_norm_quantize_raw(x, g, 1e-5, kind, qtype)
+        assert one.shape == two.shape
+        n_qs = m * k
+        assert torch.equal(one[:n_qs], two[:n_qs]), "codes differ"
+        assert torch.equal(one, two) or _planes_equal(ctx, one, two, kind, qtype, m, k), f"planes differ (kind {kind})"
+    n = 96
+    blocks = make_weight(orc, qtype, n, k, seed=1900 + k + n)
+    w = ctx.upload(qtype, k, n, blocks)
+    fused = ctx.rms_norm_quantize_raw(x, g, 1e-5, ACT_GGML, qtype)
+    y1 = ctx.mul_mat_quantized([w], fused, ACT_GGML, m, [torch.empty((m, n), device="cuda")])[0]
+    y2 = ctx.mul_mat_quantized([w], ctx.quantize_activations_raw(normed, ACT_GGML, qtype), ACT_GGML, m,
+                               [torch.empty((m, n), device="cuda")])[0]
+    assert torch.equal(y1, y2)
+    want = orc.mul_mat(qtype, blocks, k, orc.rms_norm(x.cpu().numpy(), g.cpu().numpy(), 1e-5), orc.ACT_GGML)
+    close(y1.cpu().numpy(), want, 2e-5)
+    w.free()
+
+
+def _planes_equal(ctx, a, b, kind, qtype, m, k):
+    """Compares the planes of two activation buffers and ignores the alignment padding between them."""
+    from magnitude_amd import ACT_GGML
+    al = lambda v: (v + 255) // 256 * 256
+    per256 = kind == ACT_GGML and qtype != Q8_0
+    dblk = 256 if per256 else 32
+    spans = [(0, m * k)]
+    off_d = al(m * k)
+    spans.append((off_d, off_d + m * (k // dblk) * 4))
+    off_aux = off_d + al(m * (k // dblk) * 4)
+    if per256:
+        spans.append((off_aux, off_aux + m * (k // 16) * 2))
+        off_ms = off_aux + al(m * (k // 16) * 2)
+        spans.append((off_ms, off_ms + m * (k // 256) * 32))
+    elif kind != ACT_GGML:
+        spans.append((off_aux, off_aux + m * (k // 32) * 4))
+        off_ms = off_aux + al(m * (k // 32) * 4)
+        spans.append((off_ms, off_ms + m * (k // 256) * 32))
+    return all(torch.equal(a[lo:hi], b[lo:hi]) for lo, hi in spans)
+
+
 # ---------------------------------------------------------------- replayed from a HIP graph
 
 def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):

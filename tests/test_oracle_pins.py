@@ -460,3 +460,46 @@ def test_moe_ffn_equals_explicit_numpy(orc):
     perm = np.array([2, 0, 1])
     y2 = orc.moe_ffn(Q4_K, Q4_K, gate, up, down, d_model, d_ff, E, x, ids[:, perm].copy(), wts[:, perm].copy(), orc.ACT_F64)
     assert np.allclose(y, y2, rtol=1e-5, atol=1e-7)
+
+
+# ---------------------------------------------------------------- rms_norm (+ weight multiply)
+
+def test_rms_norm_closed_forms(orc):
+    """Rows whose norm is known exactly: a mistake in where eps goes (outside the root, added to the sum
+    instead of the mean), a mean over K-1, or a missing weight multiply fails one of them."""
+    k = 64
+    # constant row 1, eps = 3: mean = 1, 1/sqrt(1 + 3) = 0.5 exactly
+    y = orc.rms_norm(np.ones((1, k), np.float32), None, 3.0)
+    assert np.array_equal(y, np.full((1, k), 0.5, np.float32))
+    # one-hot row a*e_j, eps = 0: mean = a^2/K, y_j = sqrt(K) * sign(a) (K = 64: exactly 8), zeros elsewhere
+    x = np.zeros((2, k), np.float32)
+    x[0, 5], x[1, 63] = 3.0, -0.25
+    y = orc.rms_norm(x, None, 0.0)
+    want = np.zeros_like(x)
+    want[0, 5], want[1, 63] = 8.0, -8.0
+    assert np.array_equal(y, want)
+    # the weights multiply the normalised value element by element; rows are independent
+    g = np.arange(1, k + 1, dtype=np.float32)
+    y = orc.rms_norm(np.ones((3, k), np.float32), g, 3.0)
+    assert np.array_equal(y, np.tile(0.5 * g, (3, 1)))
+    # eps is added to the mean, not to the sum: constant row 2 over K = 64 with eps = 12 -> 2/sqrt(4 + 12) = 0.5
+    y = orc.rms_norm(np.full((1, k), 2.0, np.float32), None, 12.0)
+    assert np.array_equal(y, np.full((1, k), 0.5, np.float32))
+
+
+def test_rms_norm_against_fp64_and_scale_invariance(orc):
+    rng = np.random.default_rng(21)
+    for k in (32, 288, 4096, 14336):
+        x = (rng.standard_normal((4, k)) * rng.uniform(0.01, 30.0, (4, 1))).astype(np.float32)
+        g = rng.standard_normal(k).astype(np.float32)
+        eps = 1e-5
+        y = orc.rms_norm(x, g, eps)
+        x64 = x.astype(np.float64)
+        ref = x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + eps) * g
+        # float roundings of the mean, the root, the reciprocal and the two products: a few ulp of the fp64 value
+        assert np.all(np.abs(y - ref) <= 4.0 * np.spacing(np.abs(ref).astype(np.float32)) + 1e-30)
+        # a power-of-two rescaling of the row changes nothing when eps = 0 (every step scales exactly)
+        y0 = orc.rms_norm(x, g, 0.0)
+        assert np.array_equal(orc.rms_norm(x * np.float32(8.0), g, 0.0), y0)
+        assert np.array_equal(orc.rms_norm(x, None, 0.0) * g, y0)
+
