@@ -114,7 +114,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--layers", type=int, default=32)
-    ap.add_argument("--legs", default="step,roofline,verify,q8_0,prefill,moe,llama_bench,cpu")
+    ap.add_argument("--legs", default="step,roofline,verify,q8_0,norm,prefill,moe,llama_bench,cpu")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--split-quantize", action="store_true",
                     help="run the activation quantizer as a separate launch instead of inside the projection kernel")
@@ -327,6 +327,38 @@ def main():
         log(f"[bench] q8_0 4096x4096 M=1: {ms * 1e3:.2f} us  {out['q8_0']['GBps']:.0f} GB/s")
         for w in ws:
             w.free()
+
+    # ------------------------------------------------------------------ norm leg (fused neighbours of the path)
+    if "norm" in legs:
+        # RMS norm + norm weights in front of the gate/up projections of the 32 layers: three separate calls
+        # (norm, then the projection call with its own quantizer) against the single entry point
+        gamma = torch.ones(D_MODEL, device=dev) + 0.1 * torch.randn(D_MODEL, device=dev)
+        res = {}
+        for m in (1, 512):
+            xn = torch.randn((m, D_MODEL), device=dev)
+            xnormed = torch.empty_like(xn)
+            yg = [torch.empty((m, D_FF), device=dev) for _ in range(2)]
+
+            def separate():
+                for lw in layers:
+                    ctx.rms_norm(xn, gamma, 1e-5, out=xnormed, sync=False)
+                    ctx.mul_mat_multi([lw["gate"], lw["up"]], xnormed, ACT_GGML, outs=yg, sync=False)
+
+            def fused():
+                for lw in layers:
+                    ctx.rms_norm_mul_mat([lw["gate"], lw["up"]], xn, gamma, 1e-5, ACT_GGML, outs=yg, sync=False)
+
+            row = {}
+            for name, f in (("separate", separate), ("fused", fused)):
+                f()
+                ctx.sync()
+                run = (None if args.no_graph else capture(torch, stream, f)) or f
+                run()
+                torch.cuda.synchronize()
+                row[name + "_us"] = timer.time_ms(run, max(5, args.steps)) / len(layers) * 1e3
+            res[f"M={m}"] = row
+            log(f"[bench] norm + gate/up, M={m}: separate calls {row['separate_us']:.1f} us, one call {row['fused_us']:.1f} us per layer")
+        out["norm"] = res
 
     # ------------------------------------------------------------------ prefill leg (config 4)
     if "prefill" in legs:

@@ -122,6 +122,13 @@ int qproj_rms_norm(qproj_ctx *ctx, const float *x_dev, const float *gamma_dev, f
 int qproj_rms_norm_quantize(qproj_ctx *ctx, int kind, int wtype, const float *x_dev, const float *gamma_dev,
                             float eps, int64_t M, int64_t K, void *out_dev);
 
+/* qproj_rms_norm (gamma_dev may be null) followed by qproj_mul_mat_multi on the normalised rows, the sequence
+ * norm -> q/k/v and norm -> gate/up of every transformer block.  One launch where the decode kernel serves
+ * (its prologue normalises and quantizes the row: M <= 2 with K <= 16384 / M), otherwise the fused
+ * norm + quantizer launch followed by the projection.  Same results as the separate calls. */
+int qproj_rms_norm_mul_mat(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev,
+                           const float *gamma_dev, float eps, int64_t M, float *const *y_dev, int act);
+
 /* GGML_OP_MUL_MAT: y_dev[M][N] = x_dev[M][K] . W^T.  Picks the decode (M=1), small-batch
  * (M<=16) or prefill kernel from M.  W must have n_expert == 1. */
 int qproj_mul_mat(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int64_t M, float *y_dev,

@@ -143,4 +143,22 @@ __device__ __forceinline__ void wave_store_q8_32(const float4 &v, int lane, int6
     }
 }
 
+
+// Sum of squares of a row spread over a workgroup of 16 waves in ggml's precision (float products summed in
+// double).  The order is fixed - lane's own pieces, butterfly over the wave, waves 0..15 - so that every
+// kernel that normalises a row gets the same bits.  `partial` is 16 doubles of LDS; contains a barrier.
+__device__ __forceinline__ double sum4_sq(const float4 &v) {
+    return (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
+}
+__device__ __forceinline__ double workgroup_sum16(double s, double *partial) {
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d);
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = s;
+    __syncthreads();
+    double total = 0.0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) total += partial[w];
+    return total;
+}
+
 }  // namespace qproj

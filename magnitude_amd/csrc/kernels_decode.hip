@@ -186,8 +186,42 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
                 if (m < args.M && e0 < K) x_first[m * kPer + i] = *reinterpret_cast<const float4 *>(args.x + (int64_t)m * K + e0);
             }
     }
+    // RMS norm fused in front of the quantizer (the launcher only asks for it when the prefetched pieces are the
+    // whole row): weights of the norm fetched with the row, sum of squares over the workgroup in the order of
+    // the standalone kernel, then the pieces are replaced by (x * scale) * gamma.
+    float4 g_first[kPrefetchedPieces / MT];
+    if (FUSE && args.norm) {
+#pragma unroll
+        for (int i = 0; i < kPrefetchedPieces / MT; ++i) {
+            const int e0 = (wave + kDecodeWaves * i) * 256 + 4 * lane;
+            g_first[i] = make_float4(1.f, 1.f, 1.f, 1.f);
+            if (args.norm_gamma && e0 < K) g_first[i] = *reinterpret_cast<const float4 *>(args.norm_gamma + e0);
+        }
+    }
     Raw<QT> buf_a[R], buf_b[R];
     issue<QT, R>(buf_a, rp, 0, 0, last_row, nb, lane);  // in flight while the activations are staged
+    if (FUSE && args.norm) {
+        __shared__ double norm_partial[kDecodeWaves];
+        constexpr int kPer = kPrefetchedPieces / MT;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            double sq = 0.0;
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) sq += sum4_sq(x_first[m * kPer + i]);
+            if (m > 0) __syncthreads();   // the partial sums of the previous row have been read
+            const double total = workgroup_sum16(sq, norm_partial);
+            const float mean = (float)(total / (double)K);
+            const float scale = 1.0f / sqrtf(mean + args.norm_eps);
+#pragma unroll
+            for (int i = 0; i < kPer; ++i) {
+                float4 &v = x_first[m * kPer + i];
+                v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
+                if (args.norm_gamma) {
+                    v.x *= g_first[i].x; v.y *= g_first[i].y; v.z *= g_first[i].z; v.w *= g_first[i].w;
+                }
+            }
+        }
+    }
 
     stage_activations<QT, MT, FUSE>(smem, args, K, kpad, FUSE ? x_first : nullptr);
     __syncthreads();
@@ -349,6 +383,10 @@ hipError_t launch_decode_mt(const GemvArgs &args, int mt, hipStream_t s) {
 }
 
 }  // namespace
+
+bool decode_kernel_norm_fits(int mt, int64_t K) {
+    return mt >= 1 && mt <= kPrefetchedPieces && K <= (int64_t)256 * kDecodeWaves * (kPrefetchedPieces / mt);
+}
 
 // the largest K whose activation rows fit the LDS image (mt rows)
 bool decode_kernel_fits(int type, int mt, int64_t K) {

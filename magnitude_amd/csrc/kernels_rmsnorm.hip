@@ -21,12 +21,6 @@ namespace {
 constexpr int kNormWaves = 16, kNormThreads = 64 * kNormWaves;
 constexpr int kHeld = 4;   // 256-float pieces a wave keeps in registers: rows up to 16384 floats are read once
 
-__device__ __forceinline__ double wave_sum(double v) {
-#pragma unroll
-    for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d);
-    return v;
-}
-
 // MODE 0: store fp32.  MODE 1: Q8_K planes.  MODE 2: ggml Q8_0 blocks.  MODE 3: per-32 prefill format.
 template <int MODE>
 __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
@@ -46,22 +40,16 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const float *__r
         const int64_t e0 = (int64_t)(wave + kNormWaves * i) * 256 + 4 * lane;
         held[i] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (e0 < K) held[i] = *reinterpret_cast<const float4 *>(xr + e0);
-        s += (double)(held[i].x * held[i].x) + (double)(held[i].y * held[i].y) + (double)(held[i].z * held[i].z) +
-             (double)(held[i].w * held[i].w);
+        s += sum4_sq(held[i]);
     }
     for (int p = wave + kNormWaves * kHeld; p < n_pieces; p += kNormWaves) {   // rows longer than 16384
         const int64_t e0 = (int64_t)p * 256 + 4 * lane;
         if (e0 < K) {
             const float4 v = *reinterpret_cast<const float4 *>(xr + e0);
-            s += (double)(v.x * v.x) + (double)(v.y * v.y) + (double)(v.z * v.z) + (double)(v.w * v.w);
+            s += sum4_sq(v);
         }
     }
-    s = wave_sum(s);
-    if (lane == 0) partial[wave] = s;
-    __syncthreads();
-    double total = 0.0;
-#pragma unroll
-    for (int w = 0; w < kNormWaves; ++w) total += partial[w];
+    const double total = workgroup_sum16(s, partial);
     const float mean = (float)(total / (double)K);
     const float scale = 1.0f / sqrtf(mean + eps);
 

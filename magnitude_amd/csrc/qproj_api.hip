@@ -578,8 +578,15 @@ int qproj_rms_norm_quantize(qproj_ctx *ctx, int kind, int wtype, const float *x_
     return QPROJ_OK;
 }
 
-int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
-                        float *const *y_dev, int act) {
+namespace {
+struct NormSpec {   // RMS norm (+ weights) applied to the rows before they are used
+    const float *gamma;
+    float eps;
+};
+}  // namespace
+
+static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
+                              float *const *y_dev, int act, const NormSpec *norm) {
     if (!ctx) return QPROJ_ERR_INVALID_ARG;
     if (n <= 0 || n > kMaxTargets || !w || !y_dev || !x_dev)
         return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: null argument or more than 4 tensors");
@@ -593,8 +600,9 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
     if (M == 0) return QPROJ_OK;
     QP_HIP(ctx, hipSetDevice(ctx->device));
     const int64_t K = w[0]->K;
-    if (act == kActGGML && !use_mfma_kernel(w[0]->type, M, K) && use_decode_kernel(w[0]->type, M, K)) {
-        // decode regime: the kernel quantizes the activation rows itself, no scratch needed
+    if (act == kActGGML && !use_mfma_kernel(w[0]->type, M, K) && use_decode_kernel(w[0]->type, M, K) &&
+        (!norm || decode_kernel_norm_fits(pow2_ceil(M), K))) {
+        // decode regime: the kernel (normalises and) quantizes the activation rows itself, no scratch needed
         GemvArgs g{};
         g.n_targets = n;
         for (int i = 0; i < n; ++i) {
@@ -602,6 +610,9 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
             g.t[i].y = y_dev[i];
         }
         g.x = x_dev;
+        g.norm = norm != nullptr;
+        g.norm_gamma = norm ? norm->gamma : nullptr;
+        g.norm_eps = norm ? norm->eps : 0.f;
         g.M = (int)M;
         g.x_div = 1;
         QP_HIP(ctx, launch_gemv_decode(g, pow2_ceil(M), true, ctx->stream));
@@ -610,7 +621,7 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
     if (act == kActGGML || act == kActQ8X32) {
         if (act == kActQ8X32 && w[0]->type != kTypeQ4_K)
             return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat: the per-32 int8 path is built for Q4_K weights");
-        if (act == kActGGML && dense_fuses_quantizer(w[0], M)) {
+        if (act == kActGGML && !norm && dense_fuses_quantizer(w[0], M)) {
             int rc = ensure_ws(ctx, dense_scratch_bytes(n, w, M));
             if (rc) return rc;
             ActView a{};
@@ -622,7 +633,17 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
         const size_t extra = act == kActGGML ? dense_scratch_bytes(n, w, M) : per32_scratch_max(n, w, M);
         int rc = ensure_ws(ctx, p.total + extra);
         if (rc) return rc;
-        QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, M, K));
+        if (norm) {   // norm, weights and quantizer in one launch
+            if (p.kind == kActKindQ8X32 && K % 256 != 0)
+                return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_rms_norm_mul_mat: the per-32 format needs K % 256 == 0");
+            QP_HIP(ctx, launch_rms_norm(p.kind, x_dev, norm->gamma, norm->eps, M, K, nullptr,
+                                        reinterpret_cast<int8_t *>(ctx->ws + p.off_qs), reinterpret_cast<float *>(ctx->ws + p.off_d),
+                                        reinterpret_cast<int16_t *>(ctx->ws + p.off_aux),
+                                        reinterpret_cast<uint16_t *>(ctx->ws + p.off_msum),
+                                        reinterpret_cast<int32_t *>(ctx->ws + p.off_aux), ctx->stream));
+        } else {
+            QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, M, K));
+        }
         const ActView a = act_view(p, ctx->ws, K);
         if (act == kActGGML)
             return run_dense_q8act(ctx, n, w, a, M, y_dev, reinterpret_cast<float *>(ctx->ws + p.total));
@@ -632,6 +653,13 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
         return QPROJ_OK;
     }
     if (act == kActF32) {
+        if (norm) {   // normalised rows to the workspace, then the fp32 kernel reads them
+            int rc = ensure_ws(ctx, (size_t)M * K * 4);
+            if (rc) return rc;
+            QP_HIP(ctx, launch_rms_norm(-1, x_dev, norm->gamma, norm->eps, M, K, reinterpret_cast<float *>(ctx->ws), nullptr,
+                                        nullptr, nullptr, nullptr, nullptr, ctx->stream));
+            x_dev = reinterpret_cast<const float *>(ctx->ws);
+        }
         for (int64_t m0 = 0; m0 < M; m0 += 4) {
             const int64_t mc = std::min<int64_t>(4, M - m0);
             GemvArgs g{};
@@ -648,6 +676,17 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
         return QPROJ_OK;
     }
     return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: unknown activation mode");
+}
+
+int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
+                        float *const *y_dev, int act) {
+    return mul_mat_multi_impl(ctx, n, w, x_dev, M, y_dev, act, nullptr);
+}
+
+int qproj_rms_norm_mul_mat(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, const float *gamma_dev,
+                           float eps, int64_t M, float *const *y_dev, int act) {
+    const NormSpec norm{gamma_dev, eps};
+    return mul_mat_multi_impl(ctx, n, w, x_dev, M, y_dev, act, &norm);
 }
 
 int qproj_mul_mat_quantized(qproj_ctx *ctx, int n, const qproj_weight *const *w, const void *act_dev, int kind,

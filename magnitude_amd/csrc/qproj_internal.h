@@ -64,6 +64,9 @@ struct GemvArgs {
     GemvTarget t[kMaxTargets];
     ActView a;
     const float *x;        // f32 activations (F32 mode) [rows][K]
+    const float *norm_gamma;   // decode kernel with its quantizer fused: RMS-normalise the rows first and
+    float norm_eps;            // multiply by these weights (null: rows are used as they are)
+    bool norm;
     int M;                 // activation rows in this launch (dense mode), <= MT
     // expert-grouped mode (MUL_MAT_ID); null order = dense
     const int32_t *order;   // pair indices sorted by expert
@@ -90,6 +93,7 @@ hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, i
 hipError_t launch_gemv_q8act(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
 // persistent decode kernel (mt <= 4 rows); fuse_quantize: args.x holds fp32 rows, else args.a
 bool decode_kernel_fits(int type, int mt, int64_t K);
+bool decode_kernel_norm_fits(int mt, int64_t K);   // the fused RMS norm needs the whole row in the prologue's registers
 hipError_t launch_gemv_decode(const GemvArgs &args, int mt, bool fuse_quantize, hipStream_t s);
 // int8 matrix-core kernel for 1..16 activation rows (K % 256 == 0); `scratch` holds the per-K-chunk
 // results when K > 4096 (mfma_gemv_scratch_bytes, 0 if none is needed)

@@ -48,6 +48,7 @@ SYMBOLS = {
     "qproj_act_bytes": (_sz, [_i32, _i32, _i64, _i64]),
     "qproj_quantize_activations": (_i32, [_vp, _i32, _i32, _vp, _i64, _i64, _vp]),
     "qproj_rms_norm": (_i32, [_vp, _vp, _vp, C.c_float, _i64, _i64, _vp]),
+    "qproj_rms_norm_mul_mat": (_i32, [_vp, _i32, _vp, _vp, _vp, C.c_float, _i64, _vp, _i32]),
     "qproj_rms_norm_quantize": (_i32, [_vp, _i32, _i32, _vp, _vp, C.c_float, _i64, _i64, _vp]),
     "qproj_mul_mat": (_i32, [_vp, _vp, _vp, _i64, _vp, _i32]),
     "qproj_mul_mat_multi": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i64, C.POINTER(_vp), _i32]),
@@ -282,6 +283,25 @@ class Context:
         if sync:
             self.sync()
         return buf
+
+    def rms_norm_mul_mat(self, ws: Sequence[Weight], x: torch.Tensor, gamma: Optional[torch.Tensor], eps: float,
+                         act: int = ACT_GGML, outs: Optional[Sequence[torch.Tensor]] = None, sync: bool = True):
+        """RMS norm (+ norm weights) and the MUL_MATs that share the normalised rows (q/k/v, gate/up)."""
+        x2 = x.reshape(-1, ws[0].K).contiguous()
+        m = x2.shape[0]
+        ys = list(outs) if outs is not None else [
+            torch.empty((m, w.N), dtype=torch.float32, device=x.device) for w in ws]
+        n = len(ws)
+        wa = (_vp * n)(*[w.handle for w in ws])
+        ya = (_vp * n)(*[_ptr(y) for y in ys])
+        if sync:
+            torch.cuda.current_stream().synchronize()
+        self._check(self.lib.qproj_rms_norm_mul_mat(self.handle, n, wa, _ptr(x2),
+                                                    0 if gamma is None else _ptr(gamma.contiguous()),
+                                                    C.c_float(eps), m, ya, act))
+        if sync:
+            self.sync()
+        return ys
 
     def quantize_activations_raw(self, x: torch.Tensor, kind: int, wtype: int,
                                  out: Optional[torch.Tensor] = None, sync: bool = True) -> torch.Tensor:

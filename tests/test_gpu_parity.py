@@ -484,6 +484,37 @@ def test_rms_norm_quantize_writes_the_bytes_of_the_two_calls(ctx, orc, qtype, m,
     w.free()
 
 
+@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 200])
+def test_rms_norm_mul_mat_equals_the_separate_calls(ctx, orc, qtype, m):
+    """norm -> projections in one call: the decode kernel normalises in its prologue (M = 1, 2 while the row
+    fits the prefetched pieces: K = 4096 and 14336 at M = 1, 4096 at M = 2), everything else runs the fused
+    norm + quantizer launch and then the projection.  Bit for bit the result of qproj_rms_norm followed by
+    qproj_mul_mat_multi, for ggml's activation format, the per-32 format and fp32 activations."""
+    from magnitude_amd import ACT_GGML, ACT_Q8X32, ACT_F32
+    for k, n in ((4096, 160), (14336, 96)):
+        blocks = make_weight(orc, qtype, n, k, seed=2100 + k + n + qtype)
+        w1 = ctx.upload(qtype, k, n, blocks)
+        w2 = ctx.upload(qtype, k, n, make_weight(orc, qtype, n, k, seed=2200 + k + n + qtype))
+        rng = np.random.default_rng(m + k + qtype)
+        x = dev((rng.standard_normal((m, k)) * rng.uniform(0.1, 10.0, (m, 1))).astype(np.float32))
+        g = dev((1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32))
+        normed = ctx.rms_norm(x, g, 1e-5)
+        acts = [ACT_GGML] + ([ACT_Q8X32] if qtype == Q4_K and m >= 48 else []) + ([ACT_F32] if m <= 4 else [])
+        for act in acts:
+            want = ctx.mul_mat_multi([w1, w2], normed, act)
+            got = ctx.rms_norm_mul_mat([w1, w2], x, g, 1e-5, act)
+            for a, b in zip(got, want):
+                assert torch.equal(a, b), f"act {act} K {k}"
+        if m == 1:   # and against the CPU restatement of the whole chain
+            ref = orc.mul_mat(qtype, blocks, k, orc.rms_norm(x.cpu().numpy(), g.cpu().numpy(), 1e-5), orc.ACT_GGML)
+            close(ctx.rms_norm_mul_mat([w1], x, g, 1e-5, ACT_GGML)[0].cpu().numpy(), ref, 2e-5)
+            got = ctx.rms_norm_mul_mat([w1], x, None, 1e-6, ACT_GGML)[0]
+            assert torch.equal(got, ctx.mul_mat(w1, ctx.rms_norm(x, None, 1e-6), ACT_GGML))
+        w1.free()
+        w2.free()
+
+
 def _planes_equal(ctx, a, b, kind, qtype, m, k):
     """Compares the planes of two activation buffers and ignores the alignment padding between them."""
     from magnitude_amd import ACT_GGML
