@@ -158,7 +158,7 @@ def main():
     # ------------------------------------------------------------------ weights
     L = args.layers
     layers = []
-    need_layers = bool(legs & {"step", "roofline", "verify", "cpu", "llama_bench"})
+    need_layers = bool(legs & {"step", "roofline", "verify", "cpu", "llama_bench", "norm"})
     if need_layers:
         t0 = time.time()
         for l in range(L):
