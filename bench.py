@@ -348,8 +348,22 @@ def main():
                 for lw in layers:
                     ctx.rms_norm_mul_mat([lw["gate"], lw["up"]], xn, gamma, 1e-5, ACT_GGML, outs=yg, sync=False)
 
+            hbuf = torch.empty((m, D_FF), device=dev)
+
+            def separate_ffn():   # ... and the swiglu that joins gate and up, as one more elementwise launch
+                for lw in layers:
+                    ctx.rms_norm(xn, gamma, 1e-5, out=xnormed, sync=False)
+                    ctx.mul_mat_multi([lw["gate"], lw["up"]], xnormed, ACT_GGML, outs=yg, sync=False)
+                    torch.mul(torch.nn.functional.silu(yg[0]), yg[1], out=hbuf)
+
+            def fused_ffn():
+                for lw in layers:
+                    ctx.ffn_gate_up(lw["gate"], lw["up"], xn, ACT_GGML, gamma=gamma, eps=1e-5, out=hbuf, sync=False)
+
             row = {}
-            for name, f in (("separate", separate), ("fused", fused)):
+            for name, f in (("separate", separate), ("fused", fused), ("separate_swiglu", separate_ffn), ("fused_swiglu", fused_ffn)):
+                if name == "separate_swiglu" and not args.no_graph:
+                    continue   # torch's elementwise launches are on torch's stream: only timed in eager mode
                 f()
                 ctx.sync()
                 run = (None if args.no_graph else capture(torch, stream, f)) or f
@@ -357,7 +371,8 @@ def main():
                 torch.cuda.synchronize()
                 row[name + "_us"] = timer.time_ms(run, max(5, args.steps)) / len(layers) * 1e3
             res[f"M={m}"] = row
-            log(f"[bench] norm + gate/up, M={m}: separate calls {row['separate_us']:.1f} us, one call {row['fused_us']:.1f} us per layer")
+            log(f"[bench] norm + gate/up, M={m}: separate calls {row['separate_us']:.1f} us, one call {row['fused_us']:.1f} us per layer; "
+                f"with swiglu in the same call {row['fused_swiglu_us']:.1f} us")
         out["norm"] = res
 
     # ------------------------------------------------------------------ prefill leg (config 4)

@@ -129,6 +129,17 @@ int qproj_rms_norm_quantize(qproj_ctx *ctx, int kind, int wtype, const float *x_
 int qproj_rms_norm_mul_mat(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev,
                            const float *gamma_dev, float eps, int64_t M, float *const *y_dev, int act);
 
+/* The front half of llama.cpp's dense feed-forward (build_ffn with LLM_FFN_SILU, LLM_FFN_PAR: the two MUL_MATs
+ * and the swiglu that joins them):  h_dev[M][N] = silu(gate . x) * (up . x),  silu(v) = v / (1 + expf(-v)).
+ * gate and up are dense tensors of one shape and type.  One launch for M <= 2 (the decode kernel walks row r
+ * of both tensors in the same wave), otherwise qproj_mul_mat_multi into scratch and an elementwise pass.
+ * The second form puts qproj_rms_norm (gamma_dev may be null) in front: norm -> gate/up -> swiglu. */
+int qproj_ffn_gate_up(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, const float *x_dev,
+                      int64_t M, float *h_dev, int act);
+int qproj_rms_norm_ffn_gate_up(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up,
+                               const float *x_dev, const float *gamma_dev, float eps, int64_t M, float *h_dev,
+                               int act);
+
 /* GGML_OP_MUL_MAT: y_dev[M][N] = x_dev[M][K] . W^T.  Picks the decode (M=1), small-batch
  * (M<=16) or prefill kernel from M.  W must have n_expert == 1. */
 int qproj_mul_mat(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int64_t M, float *y_dev,

@@ -90,9 +90,22 @@ __device__ __forceinline__ void issue(Raw<QT> (&raw)[R], const RowPtr<QT> &rp, i
     }
 }
 
+// gate / up pairing: step g is row g of both tensors
+template <int QT>
+__device__ __forceinline__ void issue_pair(Raw<QT> (&raw)[2], const RowPtr<QT> &rp_gate, const RowPtr<QT> &rp_up, int g, int c,
+                                           int last_row, int nb, int lane) {
+    constexpr int BPC = Geo<QT>::kChunk / Geo<QT>::kBlk;
+    int blk = c * BPC + lane / Geo<QT>::kLanesPerBlk;
+    if (blk >= nb) blk = nb - 1;
+    const int rel = g > last_row ? last_row : g;
+    raw[0].load(rp_gate, (uint32_t)blk, lane, (uint32_t)rel);
+    raw[1].load(rp_up, (uint32_t)blk, lane, (uint32_t)rel);
+}
+
 // XREG: the lane's activation slices live in `xr` (one chunk covers K); otherwise they are read
-// from the LDS image for chunk c.
-template <int QT, int MT, int R, bool XREG>
+// from the LDS image for chunk c.  PAIR (R = 2): the two rows of a step are row g of the gate and of the up
+// tensor, and what is stored is silu(gate) * up.
+template <int QT, int MT, int R, bool XREG, bool PAIR = false>
 __device__ __forceinline__ void consume(const Raw<QT> (&raw)[R], float (&acc)[MT][R], const Dot<QT> (&xr)[MT], const XTile &xt,
                                         int g, int c, int nch, int nb, int n_rows, int64_t row_begin, int64_t N,
                                         float *y, int M, int lane) {
@@ -123,7 +136,13 @@ __device__ __forceinline__ void consume(const Raw<QT> (&raw)[R], float (&acc)[MT
             for (int i = 0; i < 4; ++i) q[i] = (v0 + i < V) ? acc[(v0 + i) / R][(v0 + i) % R] : 0.f;
             const float t = wave_sum4(q, lane);
             const int i = lane - 12;  // lanes 12..15 hold the four sums
-            if (i >= 0 && i < 4 && v0 + i < V) {
+            if constexpr (PAIR) {
+                const float up = __shfl_down(t, 1);   // sums 2m (gate) and 2m+1 (up) sit in neighbouring lanes
+                if (i >= 0 && i < 4 && v0 + i < V && ((v0 + i) & 1) == 0) {
+                    const int m = (v0 + i) / 2;
+                    if (m < M && g < n_rows) y[(int64_t)m * N + row_begin + g] = (t / (1.0f + expf(-t))) * up;
+                }
+            } else if (i >= 0 && i < 4 && v0 + i < V) {
                 const int m = (v0 + i) / R, r = (v0 + i) % R;
                 if (m < M && g * R + r < n_rows) y[(int64_t)m * N + row_begin + g * R + r] = t;
             }
@@ -135,8 +154,9 @@ __device__ __forceinline__ void consume(const Raw<QT> (&raw)[R], float (&acc)[MT
     }
 }
 
-template <int QT, int MT, int R, bool XREG, bool FUSE>
+template <int QT, int MT, int R, bool XREG, bool FUSE, bool PAIR = false>
 __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvArgs args, int kpad) {
+    static_assert(!PAIR || R == 2, "the gate/up pairing walks two rows a step");
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int CH = Geo<QT>::kChunk;
     constexpr int BLK = Geo<QT>::kBlk;
@@ -153,7 +173,7 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     int wave_first = 0, rpw = args.t[0].rows_per_wave;
 #pragma unroll
     for (int i = 1; i < kMaxTargets; ++i) {
-        if (i < args.n_targets && gw >= args.t[i].first_block) {
+        if (!PAIR && i < args.n_targets && gw >= args.t[i].first_block) {
             w = args.t[i].w;
             y = args.t[i].y;
             wave_first = args.t[i].first_block;
@@ -165,11 +185,16 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     int n_rows = 0;  // rows this wave owns
     if (row_begin < N) n_rows = (int)((N - row_begin) < rpw ? (N - row_begin) : rpw);
     n_rows = uniform(n_rows);
-    const int n_groups = (n_rows + R - 1) / R;
+    const int n_groups = PAIR ? n_rows : (n_rows + R - 1) / R;
     const int n_iter = n_groups * nch;
     const int last_row = n_rows > 0 ? n_rows - 1 : 0;
-    RowPtr<QT> rp;
+    RowPtr<QT> rp, rp_up;
     rp.set(w, row_begin < N ? row_begin : 0);
+    rp_up.set(PAIR ? args.t[1].w : w, row_begin < N ? row_begin : 0);
+    auto issue_rows = [&](Raw<QT> (&raw)[R], int g, int c) {
+        if constexpr (PAIR) issue_pair<QT>(raw, rp, rp_up, g, c, last_row, nb, lane);
+        else issue<QT, R>(raw, rp, g, c, last_row, nb, lane);
+    };
 
     // The wave's piece of the activation row is requested BEFORE the first weights: loads return in order, and
     // behind a step of weights coming from HBM the quantizing prologue would wait two microseconds for sixteen
@@ -199,7 +224,7 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
         }
     }
     Raw<QT> buf_a[R], buf_b[R];
-    issue<QT, R>(buf_a, rp, 0, 0, last_row, nb, lane);  // in flight while the activations are staged
+    issue_rows(buf_a, 0, 0);  // in flight while the activations are staged
     if (FUSE && args.norm) {
         __shared__ double norm_partial[kDecodeWaves];
         constexpr int kPer = kPrefetchedPieces / MT;
@@ -253,31 +278,31 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
         // peeled form measured slower, 19.8 against 17-18.7 us, and the plain loop below is kept.)
         int g = 0;
         for (; g + 2 < n_groups; g += 2) {
-            issue<QT, R>(buf_b, rp, g + 1, 0, last_row, nb, lane);
+            issue_rows(buf_b, g + 1, 0);
             __builtin_amdgcn_sched_barrier(0);
-            consume<QT, MT, R, XREG>(buf_a, acc, xr, xt, g, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
-            issue<QT, R>(buf_a, rp, g + 2, 0, last_row, nb, lane);
+            consume<QT, MT, R, XREG, PAIR>(buf_a, acc, xr, xt, g, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
+            issue_rows(buf_a, g + 2, 0);
             __builtin_amdgcn_sched_barrier(0);
-            consume<QT, MT, R, XREG>(buf_b, acc, xr, xt, g + 1, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
+            consume<QT, MT, R, XREG, PAIR>(buf_b, acc, xr, xt, g + 1, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
         }
         if (g + 1 < n_groups) {
-            issue<QT, R>(buf_b, rp, g + 1, 0, last_row, nb, lane);
+            issue_rows(buf_b, g + 1, 0);
             __builtin_amdgcn_sched_barrier(0);
-            consume<QT, MT, R, XREG>(buf_a, acc, xr, xt, g, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
-            consume<QT, MT, R, XREG>(buf_b, acc, xr, xt, g + 1, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
+            consume<QT, MT, R, XREG, PAIR>(buf_a, acc, xr, xt, g, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
+            consume<QT, MT, R, XREG, PAIR>(buf_b, acc, xr, xt, g + 1, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
         } else if (g < n_groups) {
-            consume<QT, MT, R, XREG>(buf_a, acc, xr, xt, g, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
+            consume<QT, MT, R, XREG, PAIR>(buf_a, acc, xr, xt, g, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
         }
         return;
     }
     if (XREG) {  // one chunk per row: the step index is the row group
         for (int g = 0; g < n_groups; g += 2) {
-            issue<QT, R>(buf_b, rp, g + 1 < n_groups ? g + 1 : n_groups - 1, 0, last_row, nb, lane);
+            issue_rows(buf_b, g + 1 < n_groups ? g + 1 : n_groups - 1, 0);
             __builtin_amdgcn_sched_barrier(0);
-            consume<QT, MT, R, XREG>(buf_a, acc, xr, xt, g, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
-            issue<QT, R>(buf_a, rp, g + 2 < n_groups ? g + 2 : n_groups - 1, 0, last_row, nb, lane);
+            consume<QT, MT, R, XREG, PAIR>(buf_a, acc, xr, xt, g, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
+            issue_rows(buf_a, g + 2 < n_groups ? g + 2 : n_groups - 1, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (g + 1 < n_groups) consume<QT, MT, R, XREG>(buf_b, acc, xr, xt, g + 1, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
+            if (g + 1 < n_groups) consume<QT, MT, R, XREG, PAIR>(buf_b, acc, xr, xt, g + 1, 0, 1, nb, n_rows, row_begin, N, y, args.M, lane);
         }
         return;
     }
@@ -291,15 +316,15 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     };
     for (int it = 0; it < n_iter; it += 2) {
         if (issued + 1 < n_iter) { advance(ig, ic); ++issued; }
-        issue<QT, R>(buf_b, rp, uniform(ig), uniform(ic), last_row, nb, lane);
+        issue_rows(buf_b, uniform(ig), uniform(ic));
         __builtin_amdgcn_sched_barrier(0);  // keep the loads ahead of the arithmetic that follows
-        consume<QT, MT, R, XREG>(buf_a, acc, xr, xt, uniform(cg), uniform(cc), nch, nb, n_rows, row_begin, N, y, args.M, lane);
+        consume<QT, MT, R, XREG, PAIR>(buf_a, acc, xr, xt, uniform(cg), uniform(cc), nch, nb, n_rows, row_begin, N, y, args.M, lane);
         advance(cg, cc);
         if (issued + 1 < n_iter) { advance(ig, ic); ++issued; }
-        issue<QT, R>(buf_a, rp, uniform(ig), uniform(ic), last_row, nb, lane);
+        issue_rows(buf_a, uniform(ig), uniform(ic));
         __builtin_amdgcn_sched_barrier(0);
         if (it + 1 < n_iter) {
-            consume<QT, MT, R, XREG>(buf_b, acc, xr, xt, uniform(cg), uniform(cc), nch, nb, n_rows, row_begin, N, y, args.M, lane);
+            consume<QT, MT, R, XREG, PAIR>(buf_b, acc, xr, xt, uniform(cg), uniform(cc), nch, nb, n_rows, row_begin, N, y, args.M, lane);
             advance(cg, cc);
         }
     }
@@ -319,11 +344,15 @@ int env_int(const char *name, int dflt) {
     return e && *e ? atoi(e) : dflt;
 }
 
-template <int QT, int MT, int R, bool XREG, bool FUSE>
+template <int QT, int MT, int R, bool XREG, bool FUSE, bool PAIR = false>
 hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
     constexpr int CH = Geo<QT>::kChunk;
     constexpr int BLK = Geo<QT>::kBlk;
     GemvArgs a = args;
+    if (PAIR) {   // gate and up are walked together: the waves are dealt over the rows of one of them
+        if (a.n_targets != 2 || a.t[0].w.N != a.t[1].w.N || a.t[0].w.K != a.t[1].w.K) return hipErrorInvalidValue;
+        a.n_targets = 1;
+    }
     int64_t rows_total = 0;
     for (int i = 0; i < a.n_targets; ++i) rows_total += a.t[i].w.N;
     if (rows_total == 0) return hipSuccess;
@@ -350,7 +379,8 @@ hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
     const int64_t K = a.t[0].w.K;
     const int kpad = (int)((K + CH - 1) / CH * CH);
     const size_t smem = (size_t)MT * kpad + (size_t)MT * (kpad / BLK) * 4 + (QT != kTypeQ8_0 ? (size_t)MT * (kpad / 16) * 2 : 0);
-    auto kern = &gemv_decode_kernel<QT, MT, R, XREG, FUSE>;
+    if (PAIR) a.n_targets = 2;
+    auto kern = &gemv_decode_kernel<QT, MT, R, XREG, FUSE, PAIR>;
     if (smem > 48 * 1024) {
         static size_t allowed = 0;
         if (smem > allowed) {
@@ -367,6 +397,11 @@ hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
 template <int QT, bool FUSE>
 hipError_t launch_decode_mt(const GemvArgs &args, int mt, hipStream_t s) {
     const bool one_chunk = QT != kTypeQ8_0 && args.t[0].w.K <= Geo<QT>::kChunk;
+    if (args.swiglu_pair) {
+        if (mt == 1) return one_chunk ? launch_decode<QT, 1, 2, true, FUSE, true>(args, s) : launch_decode<QT, 1, 2, false, FUSE, true>(args, s);
+        if (mt == 2) return one_chunk ? launch_decode<QT, 2, 2, true, FUSE, true>(args, s) : launch_decode<QT, 2, 2, false, FUSE, true>(args, s);
+        return hipErrorInvalidValue;
+    }
     switch (mt) {
     case 1: {
         // two rows per step only when every wave has at least two rows to walk

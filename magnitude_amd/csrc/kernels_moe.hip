@@ -229,6 +229,22 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
     y[i] = s;
 }
 
+// h = silu(g) * u with ggml's expression for silu, x / (1 + expf(-x))
+__global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ g, const float *__restrict__ u, size_t n,
+                                                     float *__restrict__ h) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) {
+        const float x = g[i];
+        h[i] = (x / (1.0f + expf(-x))) * u[i];
+    }
+}
+
+hipError_t launch_swiglu(const float *g, const float *u, size_t n, float *h, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, g, u, n, h);
+    return hipGetLastError();
+}
+
 hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, int64_t n_used, int64_t N,
                               float *y, hipStream_t s) {
     const int64_t n = B * N;

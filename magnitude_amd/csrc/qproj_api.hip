@@ -20,6 +20,8 @@ struct qproj_ctx {
     std::string err;
     uint8_t *ws = nullptr;      // scratch: quantized activations, MoE lists and intermediates
     size_t ws_bytes = 0;
+    uint8_t *ws2 = nullptr;     // second scratch: gate and up outputs of the unfused FFN front end
+    size_t ws2_bytes = 0;
     int32_t *flag_dev = nullptr;  // raised by kernels that meet bad device-side input
 };
 
@@ -73,6 +75,20 @@ int ensure_ws(qproj_ctx *ctx, size_t bytes) {
     const size_t want = align_up(bytes + bytes / 4);
     QP_HIP(ctx, hipMalloc((void **)&ctx->ws, want));
     ctx->ws_bytes = want;
+    return QPROJ_OK;
+}
+
+int ensure_ws2(qproj_ctx *ctx, size_t bytes) {
+    if (bytes <= ctx->ws2_bytes) return QPROJ_OK;
+    if (ctx->ws2) {
+        QP_HIP(ctx, hipStreamSynchronize(ctx->stream));
+        QP_HIP(ctx, hipFree(ctx->ws2));
+        ctx->ws2 = nullptr;
+        ctx->ws2_bytes = 0;
+    }
+    const size_t want = align_up(bytes + bytes / 4);
+    QP_HIP(ctx, hipMalloc((void **)&ctx->ws2, want));
+    ctx->ws2_bytes = want;
     return QPROJ_OK;
 }
 
@@ -440,6 +456,7 @@ int qproj_ctx_destroy(qproj_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
+    if (ctx->ws2) (void)hipFree(ctx->ws2);
     if (ctx->flag_dev) (void)hipFree(ctx->flag_dev);
     if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
     delete ctx;
@@ -687,6 +704,57 @@ int qproj_rms_norm_mul_mat(qproj_ctx *ctx, int n, const qproj_weight *const *w, 
                            float eps, int64_t M, float *const *y_dev, int act) {
     const NormSpec norm{gamma_dev, eps};
     return mul_mat_multi_impl(ctx, n, w, x_dev, M, y_dev, act, &norm);
+}
+
+// silu(gate . x) * (up . x), optionally behind an RMS norm: one launch where the decode kernel serves
+static int ffn_gate_up_impl(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, const float *x_dev,
+                            int64_t M, float *h_dev, int act, const NormSpec *norm) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (!gate || !up || !x_dev || !h_dev) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_ffn_gate_up: null argument");
+    if (gate->E != 1 || up->E != 1 || gate->K != up->K || gate->N != up->N || gate->type != up->type)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_ffn_gate_up: gate and up must be dense tensors of one shape and type");
+    if (M < 0) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_ffn_gate_up: negative M");
+    if (M == 0) return QPROJ_OK;
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    const int64_t K = gate->K, N = gate->N;
+    if (act == kActGGML && M <= 2 && !use_mfma_kernel(gate->type, M, K) && use_decode_kernel(gate->type, M, K) &&
+        (!norm || decode_kernel_norm_fits(pow2_ceil(M), K))) {
+        GemvArgs g{};
+        g.n_targets = 2;
+        g.t[0].w = gate->view;
+        g.t[1].w = up->view;
+        g.t[0].y = h_dev;
+        g.t[1].y = h_dev;
+        g.swiglu_pair = true;
+        g.x = x_dev;
+        g.norm = norm != nullptr;
+        g.norm_gamma = norm ? norm->gamma : nullptr;
+        g.norm_eps = norm ? norm->eps : 0.f;
+        g.M = (int)M;
+        g.x_div = 1;
+        QP_HIP(ctx, launch_gemv_decode(g, pow2_ceil(M), true, ctx->stream));
+        return QPROJ_OK;
+    }
+    // larger batches: the two projections into scratch, then the elementwise product
+    int rc = ensure_ws2(ctx, (size_t)2 * M * N * 4);
+    if (rc) return rc;
+    float *gu[2] = {reinterpret_cast<float *>(ctx->ws2), reinterpret_cast<float *>(ctx->ws2) + (size_t)M * N};
+    const qproj_weight *ws[2] = {gate, up};
+    rc = mul_mat_multi_impl(ctx, 2, ws, x_dev, M, gu, act, norm);
+    if (rc) return rc;
+    QP_HIP(ctx, launch_swiglu(gu[0], gu[1], (size_t)M * N, h_dev, ctx->stream));
+    return QPROJ_OK;
+}
+
+int qproj_ffn_gate_up(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, const float *x_dev, int64_t M,
+                      float *h_dev, int act) {
+    return ffn_gate_up_impl(ctx, gate, up, x_dev, M, h_dev, act, nullptr);
+}
+
+int qproj_rms_norm_ffn_gate_up(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, const float *x_dev,
+                               const float *gamma_dev, float eps, int64_t M, float *h_dev, int act) {
+    const NormSpec norm{gamma_dev, eps};
+    return ffn_gate_up_impl(ctx, gate, up, x_dev, M, h_dev, act, &norm);
 }
 
 int qproj_mul_mat_quantized(qproj_ctx *ctx, int n, const qproj_weight *const *w, const void *act_dev, int kind,

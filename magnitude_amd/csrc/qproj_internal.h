@@ -67,6 +67,8 @@ struct GemvArgs {
     const float *norm_gamma;   // decode kernel with its quantizer fused: RMS-normalise the rows first and
     float norm_eps;            // multiply by these weights (null: rows are used as they are)
     bool norm;
+    bool swiglu_pair;          // decode kernel: targets 0 and 1 are gate and up of one FFN (same K and N); a wave
+                               // walks row r of both and stores silu(gate_r . x) * (up_r . x) to t[0].y
     int M;                 // activation rows in this launch (dense mode), <= MT
     // expert-grouped mode (MUL_MAT_ID); null order = dense
     const int32_t *order;   // pair indices sorted by expert
@@ -104,6 +106,8 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s)
 bool mfma_grouped_fits(int type, int64_t K);
 hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool swiglu, hipStream_t s);
 hipError_t launch_gemv_f32(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
+// h[i] = silu(g[i]) * u[i], the expression of ggml's swiglu on floats
+hipError_t launch_swiglu(const float *g, const float *u, size_t n, float *h, hipStream_t s);
 hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_expert, int32_t *order,
                             int32_t *offsets, int32_t *active, int32_t *error_flag, hipStream_t s);
 hipError_t launch_moe_swiglu_gemv(const GemvArgs &gate_up, int mt, int n_experts_grid, hipStream_t s);

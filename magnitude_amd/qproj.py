@@ -48,6 +48,8 @@ SYMBOLS = {
     "qproj_act_bytes": (_sz, [_i32, _i32, _i64, _i64]),
     "qproj_quantize_activations": (_i32, [_vp, _i32, _i32, _vp, _i64, _i64, _vp]),
     "qproj_rms_norm": (_i32, [_vp, _vp, _vp, C.c_float, _i64, _i64, _vp]),
+    "qproj_ffn_gate_up": (_i32, [_vp, _vp, _vp, _vp, _i64, _vp, _i32]),
+    "qproj_rms_norm_ffn_gate_up": (_i32, [_vp, _vp, _vp, _vp, _vp, C.c_float, _i64, _vp, _i32]),
     "qproj_rms_norm_mul_mat": (_i32, [_vp, _i32, _vp, _vp, _vp, C.c_float, _i64, _vp, _i32]),
     "qproj_rms_norm_quantize": (_i32, [_vp, _i32, _i32, _vp, _vp, C.c_float, _i64, _i64, _vp]),
     "qproj_mul_mat": (_i32, [_vp, _vp, _vp, _i64, _vp, _i32]),
@@ -302,6 +304,25 @@ class Context:
         if sync:
             self.sync()
         return ys
+
+    def ffn_gate_up(self, gate: Weight, up: Weight, x: torch.Tensor, act: int = ACT_GGML,
+                    gamma: Optional[torch.Tensor] = None, eps: Optional[float] = None,
+                    out: Optional[torch.Tensor] = None, sync: bool = True) -> torch.Tensor:
+        """h = silu(gate . x) * (up . x); with eps given, behind an RMS norm (gamma: the norm weights or None)."""
+        x2 = x.reshape(-1, gate.K).contiguous()
+        m = x2.shape[0]
+        h = out if out is not None else torch.empty((m, gate.N), dtype=torch.float32, device=x.device)
+        if sync:
+            torch.cuda.current_stream().synchronize()
+        if eps is None:
+            self._check(self.lib.qproj_ffn_gate_up(self.handle, gate.handle, up.handle, _ptr(x2), m, _ptr(h), act))
+        else:
+            self._check(self.lib.qproj_rms_norm_ffn_gate_up(self.handle, gate.handle, up.handle, _ptr(x2),
+                                                            0 if gamma is None else _ptr(gamma.contiguous()),
+                                                            C.c_float(eps), m, _ptr(h), act))
+        if sync:
+            self.sync()
+        return h
 
     def quantize_activations_raw(self, x: torch.Tensor, kind: int, wtype: int,
                                  out: Optional[torch.Tensor] = None, sync: bool = True) -> torch.Tensor:

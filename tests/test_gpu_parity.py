@@ -515,6 +515,35 @@ def test_rms_norm_mul_mat_equals_the_separate_calls(ctx, orc, qtype, m):
         w2.free()
 
 
+@pytest.mark.parametrize("qtype", TYPES)
+@pytest.mark.parametrize("m", [1, 2, 5, 130])
+def test_ffn_gate_up_swiglu(ctx, orc, qtype, m):
+    """h = silu(gate . x) * (up . x): for M <= 2 the decode kernel walks row r of both tensors in one wave and
+    applies the product when it stores; larger batches take the two projections and an elementwise pass.
+    Checked against the separate projections (same dot products: only the last bit of expf may differ from
+    torch's) and against the CPU restatement; the form behind an RMS norm against the unfused chain."""
+    from magnitude_amd import ACT_GGML
+    for k, n in ((4096, 224), (14336, 72)):
+        gate_b = make_weight(orc, qtype, n, k, seed=2300 + k + n + qtype)
+        up_b = make_weight(orc, qtype, n, k, seed=2400 + k + n + qtype)
+        wg, wu = ctx.upload(qtype, k, n, gate_b), ctx.upload(qtype, k, n, up_b)
+        rng = np.random.default_rng(m + k + 5 * qtype)
+        x = dev((rng.standard_normal((m, k)) * 2.0).astype(np.float32))
+        gam = dev((1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32))
+        for norm in (False, True):
+            xin = ctx.rms_norm(x, gam, 1e-5) if norm else x
+            g, u = ctx.mul_mat_multi([wg, wu], xin, ACT_GGML)
+            want = (g / (1.0 + torch.exp(-g))) * u
+            got = ctx.ffn_gate_up(wg, wu, x, ACT_GGML, gamma=gam if norm else None, eps=1e-5 if norm else None)
+            assert torch.allclose(got, want, rtol=2e-6, atol=1e-9), f"norm={norm} K={k}"
+        xh = x.cpu().numpy()
+        go, uo = orc.mul_mat(qtype, gate_b, k, xh, orc.ACT_GGML), orc.mul_mat(qtype, up_b, k, xh, orc.ACT_GGML)
+        ref = (go / (1.0 + np.exp(-go.astype(np.float64)))).astype(np.float32) * uo
+        close(ctx.ffn_gate_up(wg, wu, x, ACT_GGML).cpu().numpy(), ref, 5e-5)
+        wg.free()
+        wu.free()
+
+
 def _planes_equal(ctx, a, b, kind, qtype, m, k):
     """Compares the planes of two activation buffers and ignores the alignment padding between them."""
     from magnitude_amd import ACT_GGML
