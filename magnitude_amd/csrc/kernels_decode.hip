@@ -170,20 +170,29 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     // this wave's target and run of rows (selected once; everything below is wave-uniform)
     WeightView w = args.t[0].w;
     float *y = args.t[0].y;
-    int wave_first = 0, rpw = args.t[0].rows_per_wave;
+    int wave_first = 0, rpp = args.t[0].rows_per_pair;
 #pragma unroll
     for (int i = 1; i < kMaxTargets; ++i) {
         if (!PAIR && i < args.n_targets && gw >= args.t[i].first_block) {
             w = args.t[i].w;
             y = args.t[i].y;
             wave_first = args.t[i].first_block;
-            rpw = args.t[i].rows_per_wave;
+            rpp = args.t[i].rows_per_pair;
         }
     }
     const int64_t N = w.N;
-    const int64_t row_begin = (int64_t)(gw - wave_first) * rpw;
+    // Rows are dealt to pairs of neighbouring waves: rpp consecutive rows a pair, the even wave taking the larger
+    // part.  A target with 1.5 rows per wave then keeps every wave busy (2 + 1) where whole rows per wave would
+    // leave a third of the workgroups without work, and with two rows a step the even wave's part is rounded up
+    // to an even count so that no step fetches its last row twice (7 + 7 becomes 8 + 6).
+    const int wl = gw - wave_first;
+    int part_even = (rpp + 1) >> 1;
+    if (!PAIR && R == 2) part_even = (part_even + 1) & ~1;
+    if (part_even > rpp) part_even = rpp;
+    const int64_t row_begin = (int64_t)(wl >> 1) * rpp + ((wl & 1) ? part_even : 0);
+    const int own = (wl & 1) ? rpp - part_even : part_even;
     int n_rows = 0;  // rows this wave owns
-    if (row_begin < N) n_rows = (int)((N - row_begin) < rpw ? (N - row_begin) : rpw);
+    if (row_begin < N) n_rows = (int)((N - row_begin) < own ? (N - row_begin) : own);
     n_rows = uniform(n_rows);
     const int n_groups = PAIR ? n_rows : (n_rows + R - 1) / R;
     const int n_iter = n_groups * nch;
@@ -371,9 +380,9 @@ hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
         if (i == a.n_targets - 1 || given + share > n_waves - left_after) share = n_waves - left_after - given;
         if (share < 1) return hipErrorInvalidValue;
         a.t[i].first_block = given;
-        int rpw = (int)((a.t[i].w.N + share - 1) / share);
-        a.t[i].rows_per_wave = rpw;
-        if ((int64_t)rpw * (int64_t)a.t[i].w.nb * 256 >= ((int64_t)1 << 31)) return hipErrorInvalidValue;  // 32-bit row offsets
+        const int rpp = (int)((2 * a.t[i].w.N + share - 1) / share);  // rows per pair of waves
+        a.t[i].rows_per_pair = rpp;
+        if ((int64_t)rpp * (int64_t)a.t[i].w.nb * 256 >= ((int64_t)1 << 31)) return hipErrorInvalidValue;  // 32-bit row offsets
         given += share;
     }
     const int64_t K = a.t[0].w.K;
@@ -404,7 +413,8 @@ hipError_t launch_decode_mt(const GemvArgs &args, int mt, hipStream_t s) {
     }
     switch (mt) {
     case 1: {
-        // two rows per step only when every wave has at least two rows to walk
+        // two rows per step only when every wave has at least two rows to walk (with 1.5 rows per wave, split
+        // 2 + 1 over a pair of waves, two-row steps measured slower: q/k/v 7.4 against 6.4 us)
         int64_t rows_total = 0;
         for (int i = 0; i < args.n_targets; ++i) rows_total += args.t[i].w.N;
         const bool pairs = rows_total >= (int64_t)2 * cu_count() * kDecodeWaves;

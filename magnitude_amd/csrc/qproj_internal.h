@@ -55,7 +55,7 @@ struct GemvTarget {
     WeightView w;
     float *y;              // [rows][N]
     int first_block;       // first blockIdx.x (tiled kernels) or first wave (decode kernel) of the target
-    int rows_per_wave;     // decode kernel: consecutive rows each wave of the target walks
+    int rows_per_pair;     // decode kernel: consecutive rows each pair of neighbouring waves of the target walks
 };
 constexpr int kMaxTargets = 4;
 
