@@ -170,6 +170,33 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate_exps, const qproj_wei
                   const qproj_weight *down_exps, const float *x_dev, const int32_t *ids_dev,
                   const float *weights_dev, int64_t n_used, int64_t B, float *y_dev, int act);
 
+/* Backend eligibility probe: what the reference's server asks of a GPU runtime before it offers the
+ * backend pack that needs it (/root/reference/inference/crates/icn-server/src/cuda_driver.rs:343-401
+ * inspect(): initialise, driver version, device count, one architecture string and one hardware label per
+ * device; /root/reference/inference/crates/icn-server/src/backend_eligibility.rs:17-31 maps the outcome to
+ * the contract's usable / absent / failed states,
+ * /root/reference/inference/crates/icn-contracts/src/bootstrap_protocol.rs:22-39).
+ *   usable : at least one gfx950 device; architectures / hardware_labels list every device that reported
+ *            an architecture, in ordinal order, each entry NUL-terminated;
+ *   absent : the runtime reports no device, or none of the devices is a gfx950 (this library carries
+ *            gfx950 code objects only);
+ *   failed : the runtime is there and a probe call failed.
+ * diagnostic is a single line of at most 240 characters, as the reference bounds its own.
+ * Never fails across the boundary: the return value is QPROJ_OK unless out is null. */
+enum qproj_eligibility_state { QPROJ_ELIGIBILITY_USABLE = 0, QPROJ_ELIGIBILITY_ABSENT = 1, QPROJ_ELIGIBILITY_FAILED = 2 };
+#define QPROJ_PROBE_MAX_DEVICES 16
+typedef struct qproj_eligibility {
+    int state;                                           /* enum qproj_eligibility_state          */
+    int driver_api;                                      /* hipDriverGetVersion                   */
+    int runtime_api;                                     /* hipRuntimeGetVersion                  */
+    int n_devices;                                       /* entries filled below                  */
+    char architectures[QPROJ_PROBE_MAX_DEVICES][32];     /* "gfx950"                              */
+    char hardware_labels[QPROJ_PROBE_MAX_DEVICES][256];  /* device name, trimmed                  */
+    char runtime_library[1024];                          /* path the HIP runtime was loaded from  */
+    char diagnostic[244];                                /* absent / failed: why                  */
+} qproj_eligibility;
+int qproj_probe_eligibility(qproj_eligibility *out);
+
 /* library build tag: "qproj-<version>-gfx950" */
 const char *qproj_version(void);
 

@@ -1,6 +1,7 @@
 // C ABI of the qproj library: contexts, weight upload, operator dispatch.
 #include "../../include/qproj.h"
 
+#include <dlfcn.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -394,6 +395,58 @@ int grouped_mt(int64_t n_pairs, int64_t E) {
 extern "C" {
 
 const char *qproj_version(void) { return "qproj-0.1-gfx950"; }
+
+int qproj_probe_eligibility(qproj_eligibility *out) {
+    if (!out) return QPROJ_ERR_INVALID_ARG;
+    memset(out, 0, sizeof(*out));
+    auto say = [&](int state, const char *what, hipError_t e) {
+        out->state = state;
+        char line[512];
+        if (e != hipSuccess) snprintf(line, sizeof(line), "%s: %s", what, hipGetErrorString(e));
+        else snprintf(line, sizeof(line), "%s", what);
+        size_t n = 0;
+        for (const char *c = line; *c && n < 240; ++c) out->diagnostic[n++] = (*c == '\r' || *c == '\n') ? ' ' : *c;
+        out->diagnostic[n] = 0;
+        (void)hipGetLastError();
+        return QPROJ_OK;
+    };
+    Dl_info info;
+    if (dladdr(reinterpret_cast<const void *>(&hipInit), &info) != 0 && info.dli_fname)
+        snprintf(out->runtime_library, sizeof(out->runtime_library), "%s", info.dli_fname);
+    hipError_t e = hipInit(0);
+    if (e == hipErrorNoDevice) return say(QPROJ_ELIGIBILITY_ABSENT, "no HIP device is available", hipSuccess);
+    if (e != hipSuccess) return say(QPROJ_ELIGIBILITY_FAILED, "HIP initialisation failed", e);
+    const hipError_t ev = hipDriverGetVersion(&out->driver_api);
+    (void)hipRuntimeGetVersion(&out->runtime_api);
+    int count = 0;
+    const hipError_t ec = hipGetDeviceCount(&count);
+    if (ec == hipErrorNoDevice || (ec == hipSuccess && count <= 0))
+        return say(QPROJ_ELIGIBILITY_ABSENT, "no HIP device is available", hipSuccess);
+    if (ev != hipSuccess || ec != hipSuccess || out->driver_api <= 0)
+        return say(QPROJ_ELIGIBILITY_FAILED, "HIP probe failed (driver version / device count)", ev != hipSuccess ? ev : ec);
+    bool native = false;
+    for (int i = 0; i < count && out->n_devices < QPROJ_PROBE_MAX_DEVICES; ++i) {
+        hipDeviceProp_t p;
+        if (hipGetDeviceProperties(&p, i) != hipSuccess || p.gcnArchName[0] == 0) continue;
+        char *arch = out->architectures[out->n_devices];
+        size_t n = 0;   // "gfx950:sramecc+:xnack-" -> "gfx950"
+        while (p.gcnArchName[n] && p.gcnArchName[n] != ':' && n < 31) { arch[n] = p.gcnArchName[n]; ++n; }
+        arch[n] = 0;
+        native = native || strcmp(arch, "gfx950") == 0;
+        const char *b = p.name;
+        while (*b == ' ') ++b;
+        size_t len = strlen(b);
+        while (len > 0 && b[len - 1] == ' ') --len;
+        if (len > 255) len = 255;
+        memcpy(out->hardware_labels[out->n_devices], b, len);
+        out->n_devices++;
+    }
+    (void)hipGetLastError();
+    if (out->n_devices == 0) return say(QPROJ_ELIGIBILITY_FAILED, "HIP devices did not report an architecture", hipSuccess);
+    if (!native) return say(QPROJ_ELIGIBILITY_ABSENT, "no gfx950 device is available", hipSuccess);
+    out->state = QPROJ_ELIGIBILITY_USABLE;
+    return QPROJ_OK;
+}
 
 int qproj_device_count(int *count) {
     if (!count) return QPROJ_ERR_INVALID_ARG;

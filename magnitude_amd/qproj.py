@@ -58,7 +58,18 @@ SYMBOLS = {
     "qproj_mul_mat_id": (_i32, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _i32]),
     "qproj_moe_ffn": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i32]),
     "qproj_version": (C.c_char_p, []),
+    "qproj_probe_eligibility": (_i32, [_vp]),
 }
+
+PROBE_MAX_DEVICES = 16
+
+
+class Eligibility(C.Structure):
+    """struct qproj_eligibility of include/qproj.h"""
+    _fields_ = [("state", C.c_int), ("driver_api", C.c_int), ("runtime_api", C.c_int), ("n_devices", C.c_int),
+                ("architectures", (C.c_char * 32) * PROBE_MAX_DEVICES),
+                ("hardware_labels", (C.c_char * 256) * PROBE_MAX_DEVICES),
+                ("runtime_library", C.c_char * 1024), ("diagnostic", C.c_char * 244)]
 
 
 class QprojError(RuntimeError):
@@ -88,6 +99,26 @@ def load_library(path: Optional[str] = None) -> C.CDLL:
     if path is None:
         _lib = lib
     return lib
+
+
+def probe_eligibility() -> dict:
+    """The backend eligibility entry a HIP backend would add to the server's report, in the contract's
+    serialised shape (/root/reference/inference/crates/icn-contracts/src/bootstrap_protocol.rs:14-39: tag
+    "state" in lowercase, camelCase fields): {"state": "usable", "driverApi", "architectures",
+    "driverLibrary"} or {"state": "absent" | "failed", "diagnostic"}.  "hardwareLabels" and "runtimeApi"
+    ride along for usable devices (the reference keeps its hardware labels beside the report,
+    /root/reference/inference/crates/icn-server/src/cuda_driver.rs:78)."""
+    e = Eligibility()
+    st = load_library().qproj_probe_eligibility(C.byref(e))
+    if st:
+        raise QprojError(st, "qproj_probe_eligibility")
+    if e.state == 0:
+        n = e.n_devices
+        return {"state": "usable", "driverApi": e.driver_api, "runtimeApi": e.runtime_api,
+                "architectures": [e.architectures[i].value.decode() for i in range(n)],
+                "hardwareLabels": [e.hardware_labels[i].value.decode(errors="replace") for i in range(n)],
+                "driverLibrary": e.runtime_library.decode(errors="replace")}
+    return {"state": "absent" if e.state == 1 else "failed", "diagnostic": e.diagnostic.decode(errors="replace")}
 
 
 def row_bytes(qtype: int, k: int) -> int:

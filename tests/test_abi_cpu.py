@@ -60,6 +60,29 @@ def test_null_and_no_device_errors_do_not_crash(lib):
         assert not h.value
 
 
+def test_eligibility_probe_answers_in_the_contract_shape(lib):
+    """Mirrors cuda_driver.rs inspect() / backend_eligibility.rs cuda(): usable lists one architecture per
+    device, absent and failed carry a bounded single-line diagnostic; never crashes without a GPU."""
+    from magnitude_amd import qproj
+    assert lib.qproj_probe_eligibility(None) == 1
+    assert C.sizeof(qproj.Eligibility) == 16 + 16 * 32 + 16 * 256 + 1024 + 244
+    r = qproj.probe_eligibility()
+    assert r["state"] in ("usable", "absent", "failed")
+    n = C.c_int(0)
+    rc = lib.qproj_device_count(C.byref(n))
+    if r["state"] == "usable":
+        assert rc == 0 and n.value >= 1
+        assert set(r) == {"state", "driverApi", "runtimeApi", "architectures", "hardwareLabels", "driverLibrary"}
+        assert r["driverApi"] > 0 and "gfx950" in r["architectures"]
+        assert len(r["architectures"]) == len(r["hardwareLabels"]) >= n.value
+        assert r["driverLibrary"]
+    else:
+        assert rc == 5      # whatever keeps the probe from "usable" also keeps contexts from being created
+        assert set(r) == {"state", "diagnostic"}
+        d = r["diagnostic"]
+        assert 0 < len(d) <= 240 and "\n" not in d and "\r" not in d
+
+
 def test_product_code_never_touches_the_oracle():
     """The shipped package and the benchmark's GPU leg must not import or link the CPU oracle."""
     pkg = os.path.join(ROOT, "magnitude_amd")

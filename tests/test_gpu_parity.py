@@ -107,6 +107,19 @@ def test_dequantize_bit_exact_quantizer_output(ctx, orc, qtype):
     assert np.array_equal(got.view(np.uint32), orc.dequantize(qtype, blocks, 2048).view(np.uint32))
 
 
+def test_eligibility_probe_reports_the_gfx950_device(ctx):
+    """On a box with the GPU the probe is "usable", names the architecture the library is built for and
+    agrees with torch about the device."""
+    from magnitude_amd import qproj
+    r = qproj.probe_eligibility()
+    assert r["state"] == "usable", r
+    assert r["driverApi"] > 0 and r["runtimeApi"] > 0
+    assert r["architectures"][0] == "gfx950"
+    assert len(r["architectures"]) == len(r["hardwareLabels"]) == torch.cuda.device_count()
+    assert r["hardwareLabels"][0].strip() == r["hardwareLabels"][0] != ""
+    assert "amdhip64" in r["driverLibrary"]
+
+
 def test_upload_rejects_bad_arguments(ctx, orc):
     from magnitude_amd import QprojError
     blocks = make_weight(orc, Q4_K, 4, 256, seed=1)
