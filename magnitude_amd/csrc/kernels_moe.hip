@@ -1,4 +1,5 @@
 // Expert grouping for MUL_MAT_ID and the weighted combine of the MoE feed-forward.
+#include "actquant_device.h"
 #include "qproj_device.h"
 #include "qproj_internal.h"
 
@@ -126,7 +127,20 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
                                                                   int n_expert, int32_t *__restrict__ order,
                                                                   int32_t *__restrict__ offsets,
                                                                   int32_t *__restrict__ active,
-                                                                  int32_t *__restrict__ error_flag, int by_block) {
+                                                                  int32_t *__restrict__ error_flag, int by_block,
+                                                                  const RowQuantJob job) {
+    // Workgroups past the first have nothing to do with the grouping: they quantize the activation rows the
+    // grouped projection is going to read (one 256-wide chunk a wave, ggml's quantize_row_q8_K as in the
+    // standalone quantizer), so that the two passes, which depend only on the call's inputs, share a launch.
+    if (blockIdx.x > 0) {
+        const int64_t sb = (int64_t)(blockIdx.x - 1) * (kGroupThreads / 64) + (threadIdx.x >> 6);
+        if (sb < job.n_super) {   // whole wave decides together
+            const int lane = threadIdx.x & 63;
+            const float4 v = reinterpret_cast<const float4 *>(job.x + sb * 256)[lane];
+            wave_store_q8k(v, lane, sb, job.qs, job.d, job.bsums, job.msum);
+        }
+        return;
+    }
     extern __shared__ int32_t lds[];
     int32_t *cnt = lds;                 // [n_expert] pairs of the expert, then its first slot
     int32_t *wsum = cnt + n_expert;     // [32] wave totals of the two scans
@@ -199,7 +213,8 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
 }
 
 hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_expert, int32_t *order,
-                            int32_t *offsets, int32_t *active, int32_t *error_flag, hipStream_t s) {
+                            int32_t *offsets, int32_t *active, int32_t *error_flag, const RowQuantJob *quantize,
+                            hipStream_t s) {
     if (n_expert > 8192 || n_pairs > 0x7fffffff) return hipErrorInvalidValue;
     const size_t table = (size_t)((n_pairs + 63) / 64) * (size_t)n_expert;
     const bool by_block = n_pairs <= 64 * 16 * kBlocksPerWave && table <= 24 * 1024;   // at most 96 KB of LDS
@@ -211,8 +226,12 @@ hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_exper
         if (e != hipSuccess) return e;
         allowed = lds;
     }
-    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(kGroupThreads), lds, s, ids, (int)n_pairs, (int)n_expert,
-                       order, offsets, active, error_flag, by_block ? 1 : 0);
+    RowQuantJob job{};
+    if (quantize) job = *quantize;
+    const int64_t extra = (job.n_super + kGroupThreads / 64 - 1) / (kGroupThreads / 64);
+    if (extra >= 0x7fffffff) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(moe_group_kernel, dim3((unsigned)(1 + extra)), dim3(kGroupThreads), lds, s, ids, (int)n_pairs,
+                       (int)n_expert, order, offsets, active, error_flag, by_block ? 1 : 0, job);
     return hipGetLastError();
 }
 

@@ -131,6 +131,18 @@ ActView act_view(const ActPlanes &p, uint8_t *base, int64_t K) {
     return a;
 }
 
+// the same work as run_quantize (Q8_K planes only), described for the grouping launch to carry
+RowQuantJob quantize_job(const ActPlanes &p, uint8_t *base, const float *x, int64_t M, int64_t K) {
+    RowQuantJob j{};
+    j.x = x;
+    j.n_super = M * K / 256;
+    j.qs = reinterpret_cast<int8_t *>(base + p.off_qs);
+    j.d = reinterpret_cast<float *>(base + p.off_d);
+    j.bsums = reinterpret_cast<int16_t *>(base + p.off_aux);
+    j.msum = reinterpret_cast<uint16_t *>(base + p.off_msum);
+    return j;
+}
+
 hipError_t run_quantize(qproj_ctx *ctx, const ActPlanes &p, uint8_t *base, const float *x, int64_t M, int64_t K) {
     return launch_quantize_act(p.kind, x, M, K, reinterpret_cast<int8_t *>(base + p.off_qs),
                                reinterpret_cast<float *>(base + p.off_d),
@@ -866,13 +878,17 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     if (rc) return rc;
     // few pairs an expert: the grouped kernel quantizes the rows it needs in its prologue
     const bool fuse = grouped_fuses_quantizer(w->type, K, n_pairs, w->E);
-    if (!fuse) QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, rows, K));
     int32_t *order = reinterpret_cast<int32_t *>(ctx->ws + off_order);
     int32_t *offsets = reinterpret_cast<int32_t *>(ctx->ws + off_offsets);
     int32_t *active = reinterpret_cast<int32_t *>(ctx->ws + off_active);
     const bool pair_mode = grouped_pair_mode(w->type, K, n_pairs, w->E);
+    // the quantizer and the grouping pass read only the call's inputs: one launch carries both
+    const bool joined = !fuse && !pair_mode && p.kind == kActKindQ8_K;
+    const RowQuantJob job = quantize_job(p, ctx->ws, x_dev, rows, K);
+    if (!fuse && !joined) QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, rows, K));
     if (!pair_mode)
-        QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, w->E, order, offsets, active, ctx->flag_dev, ctx->stream));
+        QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, w->E, order, offsets, active, ctx->flag_dev,
+                                     joined ? &job : nullptr, ctx->stream));
     GemvArgs g{};
     g.n_targets = 1;
     g.t[0].w = w->view;
@@ -938,11 +954,15 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
 
     const bool fuse_x = grouped_fuses_quantizer(gate->type, d_model, n_pairs, E);
     const bool fuse_h = grouped_fuses_quantizer(down->type, d_ff, n_pairs, E);
-    if (!fuse_x) QP_HIP(ctx, run_quantize(ctx, px, ws, x_dev, B, d_model));
     const bool pair_mode = grouped_pair_mode(gate->type, d_model, n_pairs, E) &&
                            grouped_pair_mode(down->type, d_ff, n_pairs, E);
+    // the quantizer of x and the grouping pass read only the call's inputs: one launch carries both
+    const bool joined = !fuse_x && !pair_mode && px.kind == kActKindQ8_K;
+    const RowQuantJob job = quantize_job(px, ws, x_dev, B, d_model);
+    if (!fuse_x && !joined) QP_HIP(ctx, run_quantize(ctx, px, ws, x_dev, B, d_model));
     if (!pair_mode)
-        QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, E, order, offsets, active, ctx->flag_dev, ctx->stream));
+        QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, E, order, offsets, active, ctx->flag_dev,
+                                     joined ? &job : nullptr, ctx->stream));
     GemvArgs g{};
     if (pair_mode) {
         g.ids = ids_dev;

@@ -108,8 +108,18 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
 hipError_t launch_gemv_f32(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
 // h[i] = silu(g[i]) * u[i], the expression of ggml's swiglu on floats
 hipError_t launch_swiglu(const float *g, const float *u, size_t n, float *h, hipStream_t s);
+// Q8_K quantization of n_super 256-wide chunks of x, carried by the spare workgroups of the grouping launch
+struct RowQuantJob {
+    const float *x;
+    int64_t n_super;
+    int8_t *qs;
+    float *d;
+    int16_t *bsums;
+    uint16_t *msum;
+};
 hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_expert, int32_t *order,
-                            int32_t *offsets, int32_t *active, int32_t *error_flag, hipStream_t s);
+                            int32_t *offsets, int32_t *active, int32_t *error_flag, const RowQuantJob *quantize,
+                            hipStream_t s);
 hipError_t launch_moe_swiglu_gemv(const GemvArgs &gate_up, int mt, int n_experts_grid, hipStream_t s);
 hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, int64_t n_used, int64_t N,
                               float *y, hipStream_t s);
