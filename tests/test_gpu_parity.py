@@ -450,6 +450,31 @@ def test_moe_ffn_matches_oracle(ctx, orc, moe, B):
         close(gsep, gid, 2e-5)   # decode kernel vs grouped matrix-core kernel: same integer dots, other fp32 order
 
 
+@pytest.mark.parametrize("E", [72, 128])
+def test_moe_ffn_many_experts(ctx, orc, moe, E):
+    """The FFN at the expert counts of the 128-expert configuration, where the grouped launches take their
+    many-workgroup shapes (8 staged rows a pass at E = 128, 16 at E = 72) and the quantizer of x rides in the
+    grouping launch."""
+    from magnitude_amd import ACT_GGML
+    d_model, d_ff, top, B = moe["d_model"], moe["d_ff"], 8, 64
+    rng = np.random.default_rng(300 + E)
+    pick = rng.integers(0, moe["E"], size=E)          # the fixture's 16 experts, repeated
+    gate_b, up_b, down_b = (np.ascontiguousarray(moe[k][pick]) for k in ("gate", "up", "down"))
+    ids, wts = routing(rng, B, top, E)
+    ids[5] = ids[4]                                    # two tokens with the same experts: more than one pair an expert for sure
+    x = rng.standard_normal((B, d_model)).astype(np.float32)
+    g = ctx.upload(Q4_K, d_model, d_ff, gate_b, n_expert=E)
+    u = ctx.upload(Q4_K, d_model, d_ff, up_b, n_expert=E)
+    d = ctx.upload(Q4_K, d_ff, d_model, down_b, n_expert=E)
+    got = ctx.moe_ffn(g, u, d, dev(x), dev(ids), dev(wts), ACT_GGML).cpu().numpy()
+    want = orc.moe_ffn(Q4_K, Q4_K, gate_b, up_b, down_b, d_model, d_ff, E, x, ids, wts, orc.ACT_GGML)
+    # one int8 code of the re-quantized intermediate moving by a step (last bit of expf) shows up as ~7e-4 of the
+    # output scale in one element of 131072 here; everything else sits below 1e-6
+    close(got, want, 1e-3)
+    gate(got, want)
+    assert np.median(np.abs(got - want)) <= 1e-6 * np.abs(want).max()
+
+
 # ---------------------------------------------------------------- RMS norm in front of the projections
 
 @pytest.mark.parametrize("m,k", [(1, 4096), (5, 14336), (3, 20480), (7, 288), (64, 4096)])
