@@ -207,17 +207,29 @@ def main():
     if "step" in legs:
         step()
         ctx.sync()
-        run = None if args.no_graph else capture(torch, stream, step)
-        out["config"]["hip_graph"] = run is not None
-        run = run or step
-        for _ in range(args.warmup):
-            run()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            run()
-        torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / args.steps
+        def timed(run):
+            for _ in range(args.warmup):
+                run()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                run()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / args.steps
+
+        # The 128 launches of a step are issued either one by one or as a replay of a HIP graph; both are timed
+        # (warmup + the same number of steps each) and the step is quoted on the faster route.  Issued one by
+        # one the host stays ahead of the device here (a launch costs it about 6 us, the average kernel 9 us),
+        # and the replay has measured 3 % slower than that on this runtime.
+        modes = {"eager": timed(step)}
+        replay = None if args.no_graph else capture(torch, stream, step)
+        if replay is not None:
+            modes["hip_graph"] = timed(replay)
+        best = min(modes, key=modes.get)
+        dt = modes[best]
+        out["config"]["launch_route"] = best
+        out["config"]["hip_graph"] = best == "hip_graph"
+        out["ms_per_step_by_route"] = {k: v * 1e3 for k, v in modes.items()}
         bytes_step = L * LAYER_BYTES
         out["ms_per_step"] = dt * 1e3
         out["value"] = bytes_step / dt / 1e9
@@ -225,7 +237,8 @@ def main():
         out["tokens_per_s_projection_only"] = 1.0 / dt
         out["bytes_per_step"] = bytes_step
         log(f"[bench] step: {dt * 1e3:.3f} ms  {out['value']:.0f} GB/s ({out['pct_hbm_peak']:.1f}% of 8 TB/s)  "
-            f"{1.0 / dt:.0f} tok/s (projections only)")
+            f"{1.0 / dt:.0f} tok/s (projections only)  [" +
+            ", ".join(f"{k} {v * 1e3:.3f} ms" for k, v in modes.items()) + "]")
 
     # ------------------------------------------------------------------ roofline leg: dominant kernel
     ev_rows, ev_meas, ev_cal = [], [], []
