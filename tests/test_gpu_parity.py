@@ -704,6 +704,31 @@ def test_full_size_against_device_fp64_of_proven_parts(ctx, qtype, k, n):
     assert torch.equal(ctx.mul_mat(w, 2 * x, ACT_GGML), 2 * ctx.mul_mat(w, x, ACT_GGML))
 
 
+@pytest.mark.parametrize("ns", [(28677,), (4096, 1024, 1024), (14336, 14336), (9001, 5003), (12289, 1)])
+@pytest.mark.parametrize("m", [1, 2])
+def test_decode_row_dealing_at_full_grids(ctx, ns, m):
+    """Row counts that give the decode kernel's waves several rows each, dealt to pairs of waves in uneven
+    parts (8 + 6, 8 + 7, 2 + 1, a last pair cut short by the end of the tensor), one to three tensors a launch:
+    every row of every tensor against the fp64 product of the dequantized weights and the dequantized
+    quantized activations (both proven bit-exact above), and against the launch of each tensor alone."""
+    from magnitude_amd import ACT_GGML, synth
+    k = 4096
+    ws = [ctx.upload_from_device(Q4_K, k, n, synth.random_weight(Q4_K, n, k, seed=600 + i, device="cuda"))
+          for i, n in enumerate(ns)]
+    g = torch.Generator(device="cuda").manual_seed(sum(ns) + m)
+    x = torch.randn((m, k), generator=g, device="cuda", dtype=torch.float32)
+    a = ctx.quantize_activations(x, ACT_GGML, Q4_K)
+    xq = (a["qs"].double().view(m, k // 256, 256) * a["d"].double()[:, :, None]).view(m, k)
+    ys = ctx.mul_mat_multi(ws, x, ACT_GGML)
+    for w, y in zip(ws, ys):
+        ref = xq @ ctx.dequantize(w).double().T
+        err = ((y.double() - ref).abs() / ref.abs().clamp(min=1.0)).max().item()
+        assert err <= 2e-5, (w.N, err)
+        assert torch.equal(y, ctx.mul_mat(w, x, ACT_GGML))
+    for w in ws:
+        w.free()
+
+
 def test_full_size_prefill_gemm_against_device_fp64(ctx):
     from magnitude_amd import ACT_Q8X32, synth
     k, n, m = 4096, 4096, 512
