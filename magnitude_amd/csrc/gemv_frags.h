@@ -29,6 +29,14 @@ template <> struct Geo<kTypeQ6_K> {
 template <> struct Geo<kTypeQ8_0> {
     static constexpr int kChunk = 1024, kBlk = 32, kLanesPerBlk = 2;
 };
+// Q8_0 for the decode kernel: a step covers 4096 weights as four 1024-wide parts, lane l holding half a block
+// (16 weights) of each -- blocks l/2, 32 + l/2, 64 + l/2, 96 + l/2 of the chunk -- so that a row of K = 4096
+// is one step of five loads a lane instead of four dependent steps.  Same planes, same arithmetic per block.
+constexpr int kTypeQ8_0Wide = 1008;
+template <> struct Geo<kTypeQ8_0Wide> {
+    static constexpr int kChunk = 4096, kBlk = 32, kLanesPerBlk = 2;
+};
+template <int QT> constexpr bool is_q8_0 = QT == kTypeQ8_0 || QT == kTypeQ8_0Wide;
 
 // block (super-block) index inside the row that `lane` works on in the chunk starting at k0
 template <int QT>
@@ -82,6 +90,7 @@ template <> struct RowPtr<kTypeQ8_0> {
     }
     __device__ __forceinline__ const void *dummy() const { return qs; }
 };
+template <> struct RowPtr<kTypeQ8_0Wide> : RowPtr<kTypeQ8_0> {};
 
 // ------------------------------------------------------------------------------------------
 template <int QT> struct Raw;
@@ -192,6 +201,43 @@ template <> struct Frag<kTypeQ8_0> {
     }
 };
 
+template <> struct Raw<kTypeQ8_0Wide> {
+    uint4 q[4];
+    uint32_t d[4];
+    uint32_t live;   // bit j: part j's block lies inside the row (a short last chunk)
+    __device__ __forceinline__ void load(const RowPtr<kTypeQ8_0Wide> &rp, uint32_t blk_, int lane, uint32_t rel = 0) {
+        live = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            uint32_t b = blk_ + 32u * j;
+            if (b < rp.nb) live |= 1u << j;
+            else b = rp.nb - 1;   // in bounds, never used
+            const uint32_t blk = rel * rp.nb + b;
+            q[j] = *reinterpret_cast<const uint4 *>(rp.qs + (blk * 32u + 16u * (uint32_t)(lane & 1)));
+            d[j] = rp.d[blk];
+        }
+    }
+    __device__ __forceinline__ void zero() {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { q[j] = make_uint4(0, 0, 0, 0); d[j] = 0; }
+        live = 0;
+    }
+};
+
+template <> struct Frag<kTypeQ8_0Wide> {
+    uint32_t q[16];
+    float d[4];
+    uint32_t live;
+    __device__ __forceinline__ void unpack(const Raw<kTypeQ8_0Wide> &r, int) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            q[4 * j] = r.q[j].x; q[4 * j + 1] = r.q[j].y; q[4 * j + 2] = r.q[j].z; q[4 * j + 3] = r.q[j].w;
+            d[j] = h2f(r.d[j]);
+        }
+        live = r.live;
+    }
+};
+
 // ------------------------------------------------------------------------------------------
 // LDS image of staged quantized activations: MT rows, `kt` bytes of K each.
 struct XTile {
@@ -281,6 +327,34 @@ template <> struct Dot<kTypeQ8_0> {
 #pragma unroll
         for (int i = 0; i < 4; ++i) s = dot4(f.q[i], xq[i], s);
         return (float)s * (f.d * xd);
+    }
+};
+
+template <> struct Dot<kTypeQ8_0Wide> {
+    uint32_t xq[16];
+    float xd[4];
+    __device__ __forceinline__ void load_x(const XTile &x, int m, int c0, int lane) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int xo = c0 + 1024 * j + 16 * lane;
+            const uint4 a = *reinterpret_cast<const uint4 *>(x.qs + m * x.kt + xo);
+            xq[4 * j] = a.x; xq[4 * j + 1] = a.y; xq[4 * j + 2] = a.z; xq[4 * j + 3] = a.w;
+            xd[j] = x.d[m * (x.kt / 32) + (c0 >> 5) + 32 * j + (lane >> 1)];
+        }
+    }
+    // the parts are added in the order of K, as four steps of the narrow geometry would add them; a part past
+    // the end of the row is left out by selection (its activation bytes were never staged)
+    __device__ __forceinline__ float dot(const Frag<kTypeQ8_0Wide> &f) const {
+        float t = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int s = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s = dot4(f.q[4 * j + i], xq[4 * j + i], s);
+            const float term = (float)s * (f.d[j] * xd[j]);
+            t = j == 0 ? term : t + (((f.live >> j) & 1u) ? term : 0.f);
+        }
+        return t;
     }
 };
 

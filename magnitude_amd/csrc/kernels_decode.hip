@@ -42,7 +42,7 @@ __device__ __forceinline__ void stage_activations(uint8_t *smem, const GemvArgs 
                 if (first && ch < wave + kDecodeWaves * kPer)
                     v = first[m * kPer + (ch - wave) / kDecodeWaves];
                 else if (have && e0 < K) v = *reinterpret_cast<const float4 *>(x + e0);
-                if (QT == kTypeQ8_0) {
+                if (is_q8_0<QT>) {
                     int s;
                     float dd;
                     const uint32_t packed = wave_quantize_q8_32(v, s, dd);
@@ -68,7 +68,7 @@ __device__ __forceinline__ void stage_activations(uint8_t *smem, const GemvArgs 
             }
             for (int i = tid; i < K / BLK; i += kDecodeThreads)
                 sd[m * (kpad / BLK) + i] = have ? a.d[(int64_t)m * (K / BLK) + i] : 0.f;
-            if (QT != kTypeQ8_0)
+            if (!is_q8_0<QT>)
                 for (int i = tid; i < K / 16; i += kDecodeThreads)
                     sb[m * (kpad / 16) + i] = have ? a.bsums[(int64_t)m * (K / 16) + i] : (int16_t)0;
         }
@@ -387,7 +387,7 @@ hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
     }
     const int64_t K = a.t[0].w.K;
     const int kpad = (int)((K + CH - 1) / CH * CH);
-    const size_t smem = (size_t)MT * kpad + (size_t)MT * (kpad / BLK) * 4 + (QT != kTypeQ8_0 ? (size_t)MT * (kpad / 16) * 2 : 0);
+    const size_t smem = (size_t)MT * kpad + (size_t)MT * (kpad / BLK) * 4 + (!is_q8_0<QT> ? (size_t)MT * (kpad / 16) * 2 : 0);
     if (PAIR) a.n_targets = 2;
     auto kern = &gemv_decode_kernel<QT, MT, R, XREG, FUSE, PAIR>;
     if (smem > 48 * 1024) {
@@ -405,7 +405,9 @@ hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
 
 template <int QT, bool FUSE>
 hipError_t launch_decode_mt(const GemvArgs &args, int mt, hipStream_t s) {
-    const bool one_chunk = QT != kTypeQ8_0 && args.t[0].w.K <= Geo<QT>::kChunk;
+    // the wide Q8_0 geometry keeps its 20 activation registers a row only for one row and plain projections (two
+    // rows, or the gate/up pairing, would spill); otherwise it reads them from the LDS image like a longer K
+    const bool one_chunk = args.t[0].w.K <= Geo<QT>::kChunk && !(QT == kTypeQ8_0Wide && (mt > 1 || args.swiglu_pair));
     if (args.swiglu_pair) {
         if (mt == 1) return one_chunk ? launch_decode<QT, 1, 2, true, FUSE, true>(args, s) : launch_decode<QT, 1, 2, false, FUSE, true>(args, s);
         if (mt == 2) return one_chunk ? launch_decode<QT, 2, 2, true, FUSE, true>(args, s) : launch_decode<QT, 2, 2, false, FUSE, true>(args, s);
@@ -435,7 +437,7 @@ bool decode_kernel_norm_fits(int mt, int64_t K) {
 
 // the largest K whose activation rows fit the LDS image (mt rows)
 bool decode_kernel_fits(int type, int mt, int64_t K) {
-    const int ch = type == kTypeQ8_0 ? 1024 : 4096;
+    const int ch = 4096;
     const int blk = type == kTypeQ8_0 ? 32 : 256;
     const int64_t kpad = (K + ch - 1) / ch * ch;
     const int64_t smem = mt * kpad + mt * (kpad / blk) * 4 + (type != kTypeQ8_0 ? mt * (kpad / 16) * 2 : 0);
@@ -446,7 +448,7 @@ hipError_t launch_gemv_decode(const GemvArgs &args, int mt, bool fuse_quantize, 
     switch (args.t[0].w.type) {
     case kTypeQ4_K: return fuse_quantize ? launch_decode_mt<kTypeQ4_K, true>(args, mt, s) : launch_decode_mt<kTypeQ4_K, false>(args, mt, s);
     case kTypeQ6_K: return fuse_quantize ? launch_decode_mt<kTypeQ6_K, true>(args, mt, s) : launch_decode_mt<kTypeQ6_K, false>(args, mt, s);
-    case kTypeQ8_0: return fuse_quantize ? launch_decode_mt<kTypeQ8_0, true>(args, mt, s) : launch_decode_mt<kTypeQ8_0, false>(args, mt, s);
+    case kTypeQ8_0: return fuse_quantize ? launch_decode_mt<kTypeQ8_0Wide, true>(args, mt, s) : launch_decode_mt<kTypeQ8_0Wide, false>(args, mt, s);
     default: return hipErrorInvalidValue;
     }
 }
