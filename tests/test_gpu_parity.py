@@ -673,6 +673,66 @@ def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):
         c.close()
 
 
+# ---------------------------------------------------------------- seeded sweeps over random shapes
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_mul_mat_random_shapes_sweep(ctx, orc, seed):
+    """40 random (type, K, N, M, activation mode) cases a seed -- ragged row counts, K of one block up to 80
+    super-blocks, M across every kernel regime, outlier channels -- against the oracle in the same mode."""
+    from magnitude_amd import ACT_F32, ACT_GGML, ACT_Q8X32
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        qt = TYPES[rng.integers(3)]
+        if qt == Q8_0:
+            k = int(rng.choice([32, 64, 96, 1056, 2048, 4096, 4128, 5120, 8192, 256 * rng.integers(1, 40)]))
+        else:
+            k = int(256 * rng.choice([1, 2, 3, 5, 8, 16, 17, 32, 40, 56, 64, 80]))
+        n = int(rng.choice([1, 2, 3, 31, 32, 33, 63, 100, 255, 256, 257, 1000, 4097, rng.integers(1, 9000)]))
+        m = int(rng.choice([1, 1, 1, 2, 2, 3, 4, 5, 8, 9, 15, 16, 17, 31, 33, 48, 64, 65, 100, 128, 129, 200, 257]))
+        m = max(1, min(m, int(1.5e9 / (k * n))))
+        mode = ACT_GGML if rng.random() < 0.7 else (ACT_F32 if rng.random() < 0.5 else ACT_Q8X32)
+        if mode == ACT_Q8X32 and (qt != Q4_K or k % 256):
+            mode = ACT_GGML
+        blocks = orc.quantize(qt, (rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        if rng.random() < 0.2:
+            x[:, rng.integers(0, k, max(1, k // 100))] *= 20
+        w = ctx.upload(qt, k, n, blocks)
+        got = ctx.mul_mat(w, dev(x), mode).cpu().numpy()
+        want = orc.mul_mat(qt, blocks, k, x, {ACT_GGML: orc.ACT_GGML, ACT_F32: orc.ACT_F64, ACT_Q8X32: orc.ACT_Q8X32}[mode])
+        try:
+            close(got, want, 1e-4 if mode == ACT_F32 else 5e-5)
+        except AssertionError as e:
+            raise AssertionError(f"seed {seed} case {case}: type {qt} K {k} N {n} M {m} mode {mode}: {e}")
+        w.free()
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_mul_mat_id_random_shapes_sweep(ctx, orc, seed):
+    """20 random (type, experts, top-k, tokens, K, N, broadcast or per-slot rows) cases a seed against the oracle."""
+    from magnitude_amd import ACT_GGML
+    rng = np.random.default_rng(seed)
+    for case in range(20):
+        qt = TYPES[rng.integers(3)]
+        E = int(rng.choice([1, 2, 4, 8, 16, 60, 128]))
+        top = int(min(E, rng.choice([1, 2, 4, 8])))
+        B = int(rng.choice([1, 2, 3, 5, 8, 17, 64, 100]))
+        k = int(256 * rng.choice([1, 2, 3, 8, 16]))
+        n = int(rng.choice([32, 96, 100, 256, 768, 1000]))
+        nb1 = 1 if rng.random() < 0.5 else top
+        wb = orc.quantize(qt, (rng.standard_normal((E * n, k)) * 0.02).astype(np.float32))
+        ids = np.stack([rng.permutation(E)[:top] for _ in range(B)]).astype(np.int32)
+        x = rng.standard_normal((B, nb1, k)).astype(np.float32)
+        w = ctx.upload(qt, k, n, wb, n_expert=E)
+        got = ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML).cpu().numpy()
+        want = orc.mul_mat_id(qt, wb, k, n, E, x, ids, orc.ACT_GGML)
+        try:
+            close(got, want, 5e-5)
+        except AssertionError as e:
+            raise AssertionError(f"seed {seed} case {case}: type {qt} E {E} top {top} B {B} K {k} N {n} nb1 {nb1}: {e}")
+        w.free()
+
+
 # ---------------------------------------------------------------- full benchmark sizes
 
 @pytest.mark.parametrize("qtype,k,n", [(Q4_K, 4096, 14336), (Q6_K, 14336, 4096), (Q8_0, 4096, 4096)])
