@@ -280,11 +280,10 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     // (g, c) = (row group, chunk) cursors; the issue cursor runs one step ahead of the consume
     // cursor and stops on the last step, whose cache lines were just fetched, so every issue is
     // unconditional and no wait ever has to cover a maybe-issued load.
-    if constexpr (XREG && MT == 1) {  // one chunk per row, one activation row: the step index is the row group
+    if constexpr (XREG && MT <= 2) {  // one chunk per row, one or two activation rows: the step index is the row group
         // No load is issued twice (a repeated load of the last step, cheap as it looks, costs 0.4 us of the
-        // gate+up launch): the loop runs while two more steps follow, the last one or two steps are peeled,
-        // and every block still knows exactly which loads are outstanding.  (With two activation rows the
-        // peeled form measured slower, 19.8 against 17-18.7 us, and the plain loop below is kept.)
+        // gate+up launch at one activation row and 0.8 us at two): the loop runs while two more steps follow,
+        // the last one or two steps are peeled, and every block still knows exactly which loads are outstanding.
         int g = 0;
         for (; g + 2 < n_groups; g += 2) {
             issue_rows(buf_b, g + 1, 0);
