@@ -280,10 +280,12 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     // (g, c) = (row group, chunk) cursors; the issue cursor runs one step ahead of the consume
     // cursor and stops on the last step, whose cache lines were just fetched, so every issue is
     // unconditional and no wait ever has to cover a maybe-issued load.
-    if constexpr (XREG && MT <= 2) {  // one chunk per row, one or two activation rows: the step index is the row group
+    if constexpr (XREG && (MT == 1 || (MT == 2 && QT == kTypeQ4_K && FUSE && !PAIR))) {  // one chunk per row, one or two activation rows: the step index is the row group
         // No load is issued twice (a repeated load of the last step, cheap as it looks, costs 0.4 us of the
         // gate+up launch at one activation row and 0.8 us at two): the loop runs while two more steps follow,
         // the last one or two steps are peeled, and every block still knows exactly which loads are outstanding.
+        // (Two rows of the wider formats, of the gate/up pairing and of rows quantized earlier keep the plain loop
+        // below: peeled they run out of registers.)
         int g = 0;
         for (; g + 2 < n_groups; g += 2) {
             issue_rows(buf_b, g + 1, 0);
