@@ -7,7 +7,7 @@ namespace qproj {
 
 // Counting sort of (token, slot) pairs by expert id, one workgroup.  offsets[e]..offsets[e+1]
 // indexes the pairs of expert e inside order[]; active[0..active[n_expert]) lists the experts that
-// have pairs, ascending.  Ids outside [0, n_expert) raise *error_flag and
+// have pairs (those with more than pass_rows pairs first, ascending within both parts).  Ids outside [0, n_expert) raise *error_flag and
 // their pairs are left out (their outputs are not written).  Pairs of one expert keep ascending
 // pair order so repeated runs produce the same launch geometry.  Each of the 16 waves takes every
 // 16th expert and sweeps the pair list 64 ids at a time (consecutive lanes on consecutive ids):
@@ -20,7 +20,7 @@ constexpr int kGroupLdsIds = 8192;   // pair ids staged in LDS up to this many, 
 // cnt[e] = pairs of expert e on entry; on exit cnt[e] = offsets[e] = its first slot, active[] lists the
 // experts that have pairs.  All threads of the workgroup call it; the caller synchronizes afterwards.
 __device__ __forceinline__ void group_scan(int n_expert, int32_t *cnt, int32_t *wsum, int32_t *__restrict__ offsets,
-                                           int32_t *__restrict__ active) {
+                                           int32_t *__restrict__ active, int pass_rows) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // exclusive scans over the workgroup (shuffles inside a wave, wave totals through LDS) of the pair
     // counts (-> offsets) and of the non-empty flags (-> compact list of the experts that have work);
@@ -34,24 +34,39 @@ __device__ __forceinline__ void group_scan(int n_expert, int32_t *cnt, int32_t *
         local += tot[i];
         local_f += tot[i] > 0;
     }
-    int incl = local, incl_f = local_f;
+    // The experts with more pairs than one pass of the grouped kernels stages (two passes over their weights) go
+    // to the front of the list, everything else stays in ascending order: the grouped kernels hand their
+    // workgroups out in list order, and a two-pass expert then starts with the grid instead of stretching its
+    // tail.  A third scan, over the "heavy" flags, gives the positions.  (The whole list ordered by pair count
+    // evened the launches out as well but cost the ordinary case 3 us: neighbouring workgroups no longer read
+    // neighbouring experts.)
+    int local_h = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) local_h += pass_rows > 0 && tot[i] > pass_rows;
+    int incl = local, incl_f = local_f, incl_h = local_h;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
-        const int up = __shfl_up(incl, d), up_f = __shfl_up(incl_f, d);
+        const int up = __shfl_up(incl, d), up_f = __shfl_up(incl_f, d), up_h = __shfl_up(incl_h, d);
         if (lane >= d) {
             incl += up;
             incl_f += up_f;
+            incl_h += up_h;
         }
     }
     if (lane == 63) {
         wsum[wave] = incl;
         wsum[16 + wave] = incl_f;
+        wsum[32 + wave] = incl_h;
     }
     __syncthreads();
-    int before = incl - local, before_f = incl_f - local_f;
-    for (int w = 0; w < wave; ++w) {
-        before += wsum[w];
-        before_f += wsum[16 + w];
+    int before = incl - local, before_f = incl_f - local_f, before_h = incl_h - local_h, n_heavy = 0;
+    for (int w = 0; w < kGroupThreads / 64; ++w) {
+        if (w < wave) {
+            before += wsum[w];
+            before_f += wsum[16 + w];
+            before_h += wsum[32 + w];
+        }
+        n_heavy += wsum[32 + w];
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -60,7 +75,12 @@ __device__ __forceinline__ void group_scan(int n_expert, int32_t *cnt, int32_t *
             cnt[e] = before;   // from here on: the expert's first slot
             offsets[e] = before;
             before += tot[i];
-            if (tot[i] > 0) active[before_f++] = e;
+            if (tot[i] > 0) {
+                const bool heavy = pass_rows > 0 && tot[i] > pass_rows;
+                active[heavy ? before_h : n_heavy + (before_f - before_h)] = e;
+                ++before_f;
+                before_h += heavy;
+            }
         }
     }
     if (tid == kGroupThreads - 1) {
@@ -72,7 +92,7 @@ __device__ __forceinline__ void group_scan(int n_expert, int32_t *cnt, int32_t *
 template <bool STAGED>
 __device__ __forceinline__ void group_sweeps(const int32_t *__restrict__ ids, const int32_t *sid, int n_pairs, int n_expert,
                                              int32_t *cnt, int32_t *wsum, int32_t *__restrict__ order,
-                                             int32_t *__restrict__ offsets, int32_t *__restrict__ active) {
+                                             int32_t *__restrict__ offsets, int32_t *__restrict__ active, int pass_rows) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     constexpr int kWaves = kGroupThreads / 64;
     auto id_at = [&](int p) { return p < n_pairs ? (STAGED ? sid[p] : ids[p]) : -1; };
@@ -92,7 +112,7 @@ __device__ __forceinline__ void group_sweeps(const int32_t *__restrict__ ids, co
         }
     }
     __syncthreads();
-    group_scan(n_expert, cnt, wsum, offsets, active);
+    group_scan(n_expert, cnt, wsum, offsets, active, pass_rows);
     __syncthreads();
     // sweep 2: placement, ascending pair order inside every expert (cnt[e] = the expert's next free slot)
     for (int base = 0; base < n_pairs; base += 64 * kHeld) {
@@ -128,7 +148,7 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
                                                                   int32_t *__restrict__ offsets,
                                                                   int32_t *__restrict__ active,
                                                                   int32_t *__restrict__ error_flag, int by_block,
-                                                                  const RowQuantJob job) {
+                                                                  int pass_rows, const RowQuantJob job) {
     // Workgroups past the first have nothing to do with the grouping: they quantize the activation rows the
     // grouped projection is going to read (one 256-wide chunk a wave, ggml's quantize_row_q8_K as in the
     // standalone quantizer), so that the two passes, which depend only on the call's inputs, share a launch.
@@ -143,8 +163,8 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
     }
     extern __shared__ int32_t lds[];
     int32_t *cnt = lds;                 // [n_expert] pairs of the expert, then its first slot
-    int32_t *wsum = cnt + n_expert;     // [32] wave totals of the two scans
-    int32_t *tab = wsum + 32;           // by_block: blk[n_blocks][n_expert]; else the staged ids
+    int32_t *wsum = cnt + n_expert;     // [48] wave totals of the three scans
+    int32_t *tab = wsum + 48;           // by_block: blk[n_blocks][n_expert]; else the staged ids
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (!by_block) {
         const bool staged = n_pairs <= kGroupLdsIds;
@@ -157,8 +177,8 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
         for (int e = tid; e < n_expert; e += kGroupThreads) cnt[e] = 0;
         if (bad) atomicOr(error_flag, 1);
         __syncthreads();
-        if (staged) group_sweeps<true>(ids, tab, n_pairs, n_expert, cnt, wsum, order, offsets, active);
-        else group_sweeps<false>(ids, tab, n_pairs, n_expert, cnt, wsum, order, offsets, active);
+        if (staged) group_sweeps<true>(ids, tab, n_pairs, n_expert, cnt, wsum, order, offsets, active, pass_rows);
+        else group_sweeps<false>(ids, tab, n_pairs, n_expert, cnt, wsum, order, offsets, active, pass_rows);
         return;
     }
     const int n_blocks = (n_pairs + 63) / 64;
@@ -203,7 +223,7 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
         cnt[e] = run;
     }
     __syncthreads();
-    group_scan(n_expert, cnt, wsum, offsets, active);
+    group_scan(n_expert, cnt, wsum, offsets, active, pass_rows);
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < kBlocksPerWave; ++i) {
@@ -218,7 +238,7 @@ hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_exper
     if (n_expert > 8192 || n_pairs > 0x7fffffff) return hipErrorInvalidValue;
     const size_t table = (size_t)((n_pairs + 63) / 64) * (size_t)n_expert;
     const bool by_block = n_pairs <= 64 * 16 * kBlocksPerWave && table <= 24 * 1024;   // at most 96 KB of LDS
-    const size_t lds = ((size_t)n_expert + 32 + (by_block ? table : n_pairs <= kGroupLdsIds ? (size_t)n_pairs : 0)) * sizeof(int32_t);
+    const size_t lds = ((size_t)n_expert + 48 + (by_block ? table : n_pairs <= kGroupLdsIds ? (size_t)n_pairs : 0)) * sizeof(int32_t);
     static size_t allowed = 48 * 1024;
     if (lds > allowed) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(moe_group_kernel),
@@ -231,7 +251,8 @@ hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_exper
     const int64_t extra = (job.n_super + kGroupThreads / 64 - 1) / (kGroupThreads / 64);
     if (extra >= 0x7fffffff) return hipErrorInvalidValue;
     hipLaunchKernelGGL(moe_group_kernel, dim3((unsigned)(1 + extra)), dim3(kGroupThreads), lds, s, ids, (int)n_pairs,
-                       (int)n_expert, order, offsets, active, error_flag, by_block ? 1 : 0, job);
+                       (int)n_expert, order, offsets, active, error_flag, by_block ? 1 : 0,
+                       n_pairs <= 4 * n_expert ? 8 : 16 /* rows a pass of the grouped matrix-core kernel stages */, job);
     return hipGetLastError();
 }
 
