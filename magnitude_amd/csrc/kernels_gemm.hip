@@ -369,17 +369,41 @@ __device__ __forceinline__ uint32_t byte_to_u16x2(uint32_t word, int i) {
     return __builtin_amdgcn_perm(0u, word, 0x0c000c00u | (uint32_t)(i << 16) | (uint32_t)i);
 }
 
+// Up to three matrices that multiply the same activation rows (q/k/v, gate/up) ride in one launch: a matrix of
+// 1024 rows against 512 tokens is 64 tiles, an eighth of the workgroups the chip holds, and took as long alone
+// as the 4096-row one beside it.  Each matrix owns a run of workgroups that starts at a multiple of 8.
+struct DirectTargets {
+    int n;
+    WeightView w[3];
+    float *y[3];
+    int first_wg[3];
+};
+
 template <int NW>
-__global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const WeightView w, const ActView a, int64_t M,
-                                                                        float *__restrict__ y, float *__restrict__ part) {
+__global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const DirectTargets tg, const ActView a, int64_t M,
+                                                                        float *__restrict__ part) {
     constexpr int NT = 64 * NW, TN = 32 * NW;
     constexpr int PA = 1024 / NT;   // 16-byte activation pieces a thread moves per super-block
     extern __shared__ __align__(16) uint8_t smem_raw[];
     DirectSmem<NW> &sm = *reinterpret_cast<DirectSmem<NW> *>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    WeightView w = tg.w[0];
+    float *__restrict__ y = tg.y[0];
+    int first_wg = 0;
+#pragma unroll
+    for (int i = 1; i < 3; ++i)
+        if (i < tg.n && (int)blockIdx.x >= tg.first_wg[i]) {
+            w = tg.w[i];
+            y = tg.y[i];
+            first_wg = tg.first_wg[i];
+        }
     const int64_t N = w.N, K = w.K, nb = w.nb;
     int tile_n, tile_m;
-    tile_of_workgroup((int)((N + TN - 1) / TN), (int)((M + 63) / 64), tile_n, tile_m);
+    {
+        const int tiles_n = (int)((N + TN - 1) / TN), tiles_m = (int)((M + 63) / 64), pid = (int)blockIdx.x - first_wg;
+        if (pid >= tiles_n * tiles_m) return;   // padding between two matrices: the whole workgroup leaves
+        tile_of_workgroup(tiles_n, tiles_m, pid, tile_n, tile_m);
+    }
     const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * 64;
     const int l32 = lane & 31, lh = lane >> 5;
 
@@ -895,8 +919,52 @@ hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, flo
     if (attr != hipSuccess) return attr;
     const int n_split = scratch ? q8k_tile_splits(w.K, M, w.N) : 1;
     const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64)), (unsigned)n_split);
-    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, w, a, M, y, scratch);
+    DirectTargets tg{};
+    tg.n = 1;
+    tg.w[0] = w;
+    tg.y[0] = y;
+    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, tg, a, M, scratch);
     if (n_split > 1) return launch_sum_parts(scratch, n_split, (size_t)M * w.N, y, s);
+    return hipGetLastError();
+}
+
+// The same for n matrices over the same activation rows.  One launch where every matrix would take the
+// 64-token kernel with K in one stretch; otherwise one launch a matrix, as above.
+hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, int64_t M, float *const *y, float *scratch,
+                                 hipStream_t s) {
+    constexpr int NW = 4;
+    static const int wide_env = getenv("QPROJ_Q8K_WIDE") ? atoi(getenv("QPROJ_Q8K_WIDE")) : -1;
+    static const bool off = getenv("QPROJ_Q8K_NO_MULTI") != nullptr;
+    bool together = !off && n >= 2 && n <= 3 && wide_env < 0 && a.kind == kActKindQ8_K && a.msum && M > 0;
+    for (int i = 0; together && i < n; ++i) {
+        const int64_t wide_tiles = ((w[i].N + 255) / 256) * ((M + 127) / 128);
+        together = w[i].type == kTypeQ4_K && w[i].K == w[0].K && w[i].K <= (1 << 24) && wide_tiles < 192 &&
+                   (!scratch || q8k_tile_splits(w[i].K, M, w[i].N) == 1);
+    }
+    if (!together) {
+        for (int i = 0; i < n; ++i) {
+            hipError_t e = launch_gemm_q8k(w[i], a, M, y[i], scratch, s);
+            if (e != hipSuccess) return e;
+        }
+        return hipSuccess;
+    }
+    using Smem = DirectSmem<NW>;
+    static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_direct_kernel<NW>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
+    if (attr != hipSuccess) return attr;
+    DirectTargets tg{};
+    tg.n = n;
+    int64_t wg = 0;
+    for (int i = 0; i < n; ++i) {
+        tg.w[i] = w[i];
+        tg.y[i] = y[i];
+        tg.first_wg[i] = (int)wg;
+        wg += ((w[i].N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64);
+        wg = (wg + 7) / 8 * 8;   // the next matrix starts on XCD 0 again
+    }
+    if (wg >= 0x7fffffff) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, dim3((unsigned)wg), dim3(64 * NW), sizeof(Smem), s, tg, a, M,
+                       static_cast<float *>(nullptr));
     return hipGetLastError();
 }
 

@@ -325,6 +325,12 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
         return t->type == kTypeQ6_K && (M >= 112 || ((M + 63) / 64) * ((t->N + 127) / 128) >= 128);
     };
     if (tiled(w[0])) {
+        if (w[0]->type == kTypeQ4_K && n >= 2 && n <= 3) {   // q/k/v, gate/up: one launch where the tiles allow it
+            WeightView views[3];
+            for (int i = 0; i < n; ++i) views[i] = w[i]->view;
+            QP_HIP(ctx, launch_gemm_q8k_multi(n, views, a, M, y, scratch, ctx->stream));
+            return QPROJ_OK;
+        }
         for (int i = 0; i < n; ++i) {
             const int t = w[0]->type;
             QP_HIP(ctx, t == kTypeQ4_K   ? launch_gemm_q8k(w[i]->view, a, M, y[i], scratch, ctx->stream)

@@ -313,6 +313,25 @@ def test_mul_mat_multi_equals_separate_calls(ctx, orc):
         assert torch.equal(y, ctx.mul_mat(w, x, ACT_GGML))
 
 
+@pytest.mark.parametrize("m", [48, 130, 512])
+@pytest.mark.parametrize("ns", [(520, 130, 77), (1024, 256), (4096, 1024, 1024)])
+def test_mul_mat_multi_prefill_batches_equal_separate_calls(ctx, orc, ns, m):
+    """Prefill-sized batches: q/k/v (or gate/up) share one launch of the 64-token kernel, each matrix on its own
+    run of workgroups with idle ones in between -- bitwise what the matrices give one by one, ragged edges
+    included, and the oracle's values."""
+    from magnitude_amd import ACT_GGML
+    k = 1024
+    blocks = [make_weight(orc, Q4_K, n, k, seed=4100 + n) for n in ns]
+    ws = [ctx.upload(Q4_K, k, n, b) for n, b in zip(ns, blocks)]
+    x = np.random.default_rng(m + len(ns)).standard_normal((m, k)).astype(np.float32)
+    ys = ctx.mul_mat_multi(ws, dev(x), ACT_GGML)
+    for w, b, y in zip(ws, blocks, ys):
+        assert torch.equal(y, ctx.mul_mat(w, dev(x), ACT_GGML))
+    close(ys[-1].cpu().numpy(), orc.mul_mat(Q4_K, blocks[-1], k, x, orc.ACT_GGML), 5e-5)
+    for w in ws:
+        w.free()
+
+
 @pytest.mark.parametrize("qtype", TYPES)
 def test_mul_mat_special_inputs(ctx, orc, qtype):
     """zero in -> zero out; power-of-two scaling is exact; a one-hot row picks a dequantized column."""
