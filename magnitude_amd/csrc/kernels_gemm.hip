@@ -935,30 +935,37 @@ hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, i
     constexpr int NW = 4;
     static const int wide_env = getenv("QPROJ_Q8K_WIDE") ? atoi(getenv("QPROJ_Q8K_WIDE")) : -1;
     static const bool off = getenv("QPROJ_Q8K_NO_MULTI") != nullptr;
-    bool together = !off && n >= 2 && n <= 3 && wide_env < 0 && a.kind == kActKindQ8_K && a.msum && M > 0;
-    for (int i = 0; together && i < n; ++i) {
+    // the matrices that would take the 64-token kernel with K in one stretch go together; the others (128-token
+    // tiles, K cut into stretches) get their own launches first
+    const bool can = !off && n >= 2 && n <= 3 && wide_env < 0 && a.kind == kActKindQ8_K && a.msum && M > 0;
+    int joined[3], n_joined = 0;
+    for (int i = 0; i < n; ++i) {
         const int64_t wide_tiles = ((w[i].N + 255) / 256) * ((M + 127) / 128);
-        together = w[i].type == kTypeQ4_K && w[i].K == w[0].K && w[i].K <= (1 << 24) && wide_tiles < 192 &&
-                   (!scratch || q8k_tile_splits(w[i].K, M, w[i].N) == 1);
+        const bool fits = can && w[i].type == kTypeQ4_K && w[i].K == w[0].K && w[i].K <= (1 << 24) && wide_tiles < 192 &&
+                          (!scratch || q8k_tile_splits(w[i].K, M, w[i].N) == 1);
+        if (fits) joined[n_joined++] = i;
     }
-    if (!together) {
-        for (int i = 0; i < n; ++i) {
-            hipError_t e = launch_gemm_q8k(w[i], a, M, y[i], scratch, s);
-            if (e != hipSuccess) return e;
-        }
-        return hipSuccess;
+    if (n_joined < 2) n_joined = 0;
+    for (int i = 0; i < n; ++i) {
+        bool in = false;
+        for (int j = 0; j < n_joined; ++j) in = in || joined[j] == i;
+        if (in) continue;
+        hipError_t e = launch_gemm_q8k(w[i], a, M, y[i], scratch, s);
+        if (e != hipSuccess) return e;
     }
+    if (n_joined == 0) return hipSuccess;
     using Smem = DirectSmem<NW>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_direct_kernel<NW>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
     if (attr != hipSuccess) return attr;
     DirectTargets tg{};
-    tg.n = n;
+    tg.n = n_joined;
     int64_t wg = 0;
-    for (int i = 0; i < n; ++i) {
-        tg.w[i] = w[i];
-        tg.y[i] = y[i];
-        tg.first_wg[i] = (int)wg;
+    for (int j = 0; j < n_joined; ++j) {
+        const int i = joined[j];
+        tg.w[j] = w[i];
+        tg.y[j] = y[i];
+        tg.first_wg[j] = (int)wg;
         wg += ((w[i].N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64);
         wg = (wg + 7) / 8 * 8;   // the next matrix starts on XCD 0 again
     }
