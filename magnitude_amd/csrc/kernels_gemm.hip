@@ -860,9 +860,12 @@ hipError_t launch_sum_parts(const float *part, int n_split, size_t n, float *y, 
 int q8k_tile_splits(int64_t K, int64_t M, int64_t N) {
     static const int forced = getenv("QPROJ_Q8K_SPLITS") ? atoi(getenv("QPROJ_Q8K_SPLITS")) : 0;
     const int64_t tiles = ((N + 127) / 128) * ((M + 63) / 64);
-    int n = forced > 0 ? forced : tiles >= 384 ? 1 : tiles >= 192 ? 2 : 3;
+    int n = forced > 0 ? forced : tiles >= 384 ? 1 : tiles >= 192 ? 2 : tiles >= 96 ? 3 : 4;
     if ((M * N) % 4 != 0) n = 1;
-    while (n > 1 && K / 256 < 12 * n) --n;
+    // a stretch is at least 12 super-blocks (the pass that adds the partial tiles has to be earned), 4 where the
+    // grid is under a fifth of the workgroups the chip holds and a workgroup's K loop is pure latency
+    const int min_sb = tiles >= 192 ? 12 : 4;
+    while (n > 1 && K / 256 < min_sb * n) --n;
     return n;
 }
 size_t q8k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N) {
@@ -942,7 +945,8 @@ hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, i
     for (int i = 0; i < n; ++i) {
         const int64_t wide_tiles = ((w[i].N + 255) / 256) * ((M + 127) / 128);
         const bool fits = can && w[i].type == kTypeQ4_K && w[i].K == w[0].K && w[i].K <= (1 << 24) && wide_tiles < 192 &&
-                          (!scratch || q8k_tile_splits(w[i].K, M, w[i].N) == 1);
+                          (!scratch || q8k_tile_splits(w[i].K, M, w[i].N) == 1 ||
+                           ((w[i].N + 127) / 128) * ((M + 63) / 64) < 96);   // small ones are better off together than cut
         if (fits) joined[n_joined++] = i;
     }
     if (n_joined < 2) n_joined = 0;

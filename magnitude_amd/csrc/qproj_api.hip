@@ -314,15 +314,16 @@ bool dense_fuses_quantizer(const qproj_weight *w, int64_t M) {
 // x_f32: non-null when `a` carries no planes and the kernel quantizes these rows itself (small batches only)
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
                     float *const *y, float *scratch, const float *x_f32 = nullptr) {
-    static const int gemm_min_m = getenv("QPROJ_GEMM_MIN_M") ? atoi(getenv("QPROJ_GEMM_MIN_M")) : 48;
-    // prefill-sized batches: tiled product, weights reused across 64 tokens.  The Q6_K kernel is slow
-    // per workgroup (a vector multiply-add per output and sub-block): below 128 tiles of 64 x 128 it
-    // only pays from 112 tokens on, under that the small-batch kernel in steps of 16 is quicker.
+    static const int gemm_min_m = getenv("QPROJ_GEMM_MIN_M") ? atoi(getenv("QPROJ_GEMM_MIN_M")) : 17;
+    // Beyond the 16 rows one pass of the small-batch kernel takes: the tiled product, weights reused across 64
+    // tokens, K cut into stretches where the grid would leave the chip idle.  (Measured, 8B shapes: Q4_K 17..47
+    // rows 19-72 us in steps of 16 against 15-31 us tiled; Q6_K, whose workgroups are slow -- a vector
+    // multiply-add per output and sub-block --, pays from 32 rows on: 62-206 us in steps against 58-63 tiled.)
     const auto tiled = [&](const qproj_weight *t) {
         if (M < gemm_min_m) return false;
         if (t->type == kTypeQ4_K) return true;
         if (t->type == kTypeQ8_0) return t->K % 128 == 0 && M >= 64;
-        return t->type == kTypeQ6_K && (M >= 112 || ((M + 63) / 64) * ((t->N + 127) / 128) >= 128);
+        return t->type == kTypeQ6_K && M >= 32;
     };
     if (tiled(w[0])) {
         if (w[0]->type == kTypeQ4_K && n >= 2 && n <= 3) {   // q/k/v, gate/up: one launch where the tiles allow it
