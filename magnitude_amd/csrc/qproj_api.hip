@@ -286,8 +286,12 @@ size_t per32_scratch_max(int n, const qproj_weight *const *w, int64_t M) {   // 
     return need;
 }
 
+// Q8_0 takes the tiled product from 64 rows on, K a multiple of 128.  One predicate for the dispatch and for the
+// scratch sizing: the partial tiles of a K cut into stretches go to scratch that only this rule provides.
+bool q8_0_tiled(const qproj_weight *t, int64_t M) { return t->type == kTypeQ8_0 && t->K % 128 == 0 && M >= 64; }
+
 size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
-    if (w[0]->type == kTypeQ8_0 && M >= 64 && w[0]->K % 128 == 0) return per32_scratch_max(n, w, M);   // tiled Q8_0 product
+    if (q8_0_tiled(w[0], M)) return per32_scratch_max(n, w, M);
     size_t need = 0;
     if (M > 16 && w[0]->type != kTypeQ8_0)   // tiled Q4_K / Q6_K products with K cut into stretches
         for (int i = 0; i < n; ++i) need = std::max(need, q8k_tile_scratch_bytes(w[i]->K, M, w[i]->N));
@@ -314,7 +318,8 @@ bool dense_fuses_quantizer(const qproj_weight *w, int64_t M) {
 // x_f32: non-null when `a` carries no planes and the kernel quantizes these rows itself (small batches only)
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
                     float *const *y, float *scratch, const float *x_f32 = nullptr) {
-    static const int gemm_min_m = getenv("QPROJ_GEMM_MIN_M") ? atoi(getenv("QPROJ_GEMM_MIN_M")) : 17;
+    // (never under 17: the scratch for K cut into stretches is sized for more than 16 rows only)
+    static const int gemm_min_m = std::max(17, getenv("QPROJ_GEMM_MIN_M") ? atoi(getenv("QPROJ_GEMM_MIN_M")) : 17);
     // Beyond the 16 rows one pass of the small-batch kernel takes: the tiled product, weights reused across 64
     // tokens, K cut into stretches where the grid would leave the chip idle.  (Measured, 8B shapes: Q4_K 17..47
     // rows 19-72 us in steps of 16 against 15-31 us tiled; Q6_K, whose workgroups are slow -- a vector
@@ -322,7 +327,7 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
     const auto tiled = [&](const qproj_weight *t) {
         if (M < gemm_min_m) return false;
         if (t->type == kTypeQ4_K) return true;
-        if (t->type == kTypeQ8_0) return t->K % 128 == 0 && M >= 64;
+        if (t->type == kTypeQ8_0) return q8_0_tiled(t, M);
         return t->type == kTypeQ6_K && M >= 32;
     };
     if (tiled(w[0])) {
