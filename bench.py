@@ -96,16 +96,106 @@ def capture(torch, stream, fn):
         return None
 
 
+MAX_LINE_BYTES = 4000      # the final stdout line stays under this; everything else goes to the details file
+
+
+def source_digest(*rel):
+    """sha256 over the named source files (relative to the repository root), first 16 hex digits"""
+    import hashlib
+    h = hashlib.sha256()
+    for r in rel:
+        with open(os.path.join(ROOT, r), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+DECODE_KERNEL_SOURCES = ("magnitude_amd/csrc/kernels_decode.hip", "magnitude_amd/csrc/gemv_frags.h")
+
+
 def measured_traffic(summary="decode_gate_up_q4k.txt"):
-    """HBM bytes per launch of the dominant kernel, from the committed rocprofv3 counter summary
-    (FETCH_SIZE + WRITE_SIZE, each scaled by a copy kernel of known size); None if not recorded."""
+    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 counter summary (FETCH_SIZE +
+    WRITE_SIZE, each scaled by a copy kernel of known size).  The summary names the digest of the kernel sources
+    it was measured on; when the sources have changed since, the figure is withheld (None) and the source says so."""
+    path = os.path.join(ROOT, "profiles", summary)
+    traffic, digest = None, None
     try:
-        for line in open(os.path.join(ROOT, "profiles", summary)):
+        for line in open(path):
             if line.startswith("traffic_bytes_per_launch:"):
-                return int(line.split(":")[1])
+                traffic = int(line.split(":")[1])
+            if line.startswith("kernel_source_digest:"):
+                digest = line.split(":")[1].strip()
     except OSError:
-        pass
-    return None
+        return None, "not recorded"
+    if traffic is None:
+        return None, "not recorded"
+    now = source_digest(*DECODE_KERNEL_SOURCES)
+    if digest != now:
+        return None, f"profiles/{summary} is stale (kernel sources {now}, summary measured on {digest})"
+    return traffic, f"profiles/{summary} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel sources {digest})"
+
+
+def _r(v, nd=4):
+    return None if v is None else round(float(v), nd)
+
+
+def compact_line(out, details_path=None):
+    """The one JSON line the driver parses: the contract's fields, the roofline and CPU baseline objects and one
+    headline figure per other leg.  Per-shape tables, raw samples and the reference-shaped evidence rows are in the
+    details file (the reference keeps raw samples in evidence files too: inference/parity/README.md:110)."""
+    keep = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+            "vs_baseline", "dtype", "data")
+    line = {k: out.get(k) for k in keep}
+    line["value"], line["ms_per_step"] = _r(out.get("value"), 2), _r(out.get("ms_per_step"), 5)
+    cfg = out.get("config", {})
+    line["config"] = {k: cfg[k] for k in ("workload", "layers", "act_mode", "launch_route") if k in cfg}
+    for k in ("pct_hbm_peak", "tokens_per_s_projection_only"):
+        if out.get(k) is not None:
+            line[k] = _r(out[k], 2)
+    rf = out.get("roofline")
+    if rf:
+        line["roofline"] = {k: (_r(rf[k]) if isinstance(rf.get(k), float) else rf.get(k))
+                            for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "traffic_source", "kernel",
+                                      "bytes_per_launch", "us_per_launch", "launches_timed")}
+        line["decode_kernels_us"] = {k: _r(v["us_per_launch"], 2) for k, v in rf.get("other_kernels", {}).items()}
+    cb = out.get("cpu_baseline")
+    if cb:
+        line["cpu_baseline"] = {k: (_r(cb[k]) if isinstance(cb.get(k), float) else cb.get(k))
+                                for k in ("value", "unit", "cores", "kind", "sample", "host_cpus", "one_thread_GBps", "isa")
+                                if k in cb}
+    if "verify" in out:
+        line["verify_us"] = {f"M{r['M']}_{r['group']}": _r(r["us_per_launch"], 2) for r in out["verify"]["shapes"]}
+    if "q8_0" in out:
+        line["q8_0_gemv"] = {"us": _r(out["q8_0"]["us_per_launch"], 2), "frac_hbm_peak": _r(out["q8_0"]["frac_hbm_peak"])}
+    for key, tag in (("prefill", "prefill_q8x32"), ("prefill_ggml_acts", "prefill_q8k")):
+        if key in out:
+            pf = out[key]
+            line[tag] = {"headline_tops": _r(pf["headline_tops"], 1), "frac_int8_peak": _r(pf["headline_frac_int8_peak"]),
+                         "peak_tops": INT8_PEAK_TOPS, "shape": "M4096 K4096 N14336 Q4_K",
+                         "tops": {f"{r.get('type', 'Q4_K')}_M{r['M']}_K{r['K']}_N{r['N']}": _r(r["gemm_tops"], 0)
+                                  for r in pf["shapes"]}}
+    if "moe" in out:
+        line["moe_ffn"] = {f"B{r['B']}": {"us": _r(r["ms"] * 1e3, 1), "GBps": _r(r["GBps"], 0),
+                                          "MB_cycled": _r(r.get("bytes_cycled", 0) / 1e6, 0)}
+                           for r in out["moe"]["batches"]}
+    if "llama_bench" in out:
+        med = lambda v: sorted(v)[len(v) // 2]
+        toks = {r["output"]["operation"].split(".")[1]: med(r["measurements"][1]["samples"]) for r in out["llama_bench"]}
+        line["llama_bench_projections_only"] = {"pp512_tok_s": _r(toks.get("prompt-processing"), 0),
+                                                "tg128_tok_s": _r(toks.get("token-generation"), 1)}
+    if details_path:
+        line["details"] = details_path
+    text = json.dumps(line, separators=(",", ":"))
+    if len(text) > MAX_LINE_BYTES:      # never lose the contract's fields to a long tail: drop the optional tables first
+        for k in ("prefill_q8k", "prefill_q8x32", "verify_us", "moe_ffn", "decode_kernels_us"):
+            if isinstance(line.get(k), dict) and "tops" in line[k]:
+                line[k].pop("tops")
+            else:
+                line.pop(k, None)
+            text = json.dumps(line, separators=(",", ":"))
+            if len(text) <= MAX_LINE_BYTES:
+                break
+    assert len(text) <= MAX_LINE_BYTES, len(text)
+    return text
 
 
 def main():
@@ -123,6 +213,9 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0)
     ap.add_argument("--evidence-sql", default=None,
                     help="also write the per-kernel rows as test-backend-ops SQL INSERT lines to this file")
+    ap.add_argument("--details-json", default=os.path.join("gpurun_out", "bench_details.json"),
+                    help="per-shape tables, raw samples and the reference-shaped evidence rows go to this file "
+                         "('' = nowhere); stdout carries one compact line")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (no sharding, no collectives); use --gpus 1", file=sys.stderr)
@@ -272,8 +365,9 @@ def main():
             ev_meas.append(evidence.measurement(f"decode.{grp[0]}.launch", "us", samples))
             ev_cal.append(evidence.calibration_metric(qt0, False, nbytes, samples, launch_us=2.0))
         dom = per["gate_up"]
+        traffic, traffic_source = measured_traffic()
         out["roofline"] = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                           "frac": dom["frac_hbm_peak"], "traffic": measured_traffic(),
+                           "frac": dom["frac_hbm_peak"], "traffic": traffic, "traffic_source": traffic_source,
                            "kernel": "gemv_decode_kernel<Q4_K, M=1>: gate+up (2 x 4096->14336) in one launch, "
                                      "activation quantized in the prologue",
                            "bytes_per_launch": dom["bytes_per_launch"], "us_per_launch": dom["us_per_launch"],
@@ -472,43 +566,75 @@ def main():
 
     # ------------------------------------------------------------------ MoE leg (config 5)
     if "moe" in legs:
-        E, top, dm, dff = 128, 8, 2048, 768
-        exps = {}
-        for i, (name, n, k) in enumerate((("gate", dff, dm), ("up", dff, dm), ("down", dm, dff))):
-            blocks = synth.random_weight(Q4_K, E * n, k, seed=500 + i, device=dev)
-            exps[name] = ctx.upload_from_device(Q4_K, k, n, blocks, n_expert=E)
-            del blocks
+        # Three distinct sets of expert weights (3 x 340 MB) and several draws of expert ids are rotated through, so
+        # that more than a gigabyte of experts cycles between two uses of the same bytes: the 256 MB Infinity Cache
+        # cannot hold them and the rate is an HBM rate.  One id draw replayed on one set (at most 340 MB, 21 MB at
+        # B = 1) is reported beside it as the cache-resident figure.
+        E, top, dm, dff, ncopy = 128, 8, 2048, 768, 3
+        sets = []
+        for c in range(ncopy):
+            exps = {}
+            for i, (name, n, k) in enumerate((("gate", dff, dm), ("up", dff, dm), ("down", dm, dff))):
+                blocks = synth.random_weight(Q4_K, E * n, k, seed=500 + 10 * c + i, device=dev)
+                exps[name] = ctx.upload_from_device(Q4_K, k, n, blocks, n_expert=E)
+                del blocks
+            sets.append(exps)
         per_expert = 2 * gguf_bytes(Q4_K, dff, dm) + gguf_bytes(Q4_K, dm, dff)
         res = []
         for B in (1, 8, 64):
-            ids = torch.stack([torch.randperm(E, generator=g, device=dev)[:top] for _ in range(B)]).to(torch.int32)
+            ndraw = {1: 16, 8: 4, 64: 2}[B]
+            if B == 1:      # sixteen disjoint draws of eight experts cover all 128
+                perm = torch.randperm(E, generator=g, device=dev).to(torch.int32)
+                draws = [perm[top * d: top * (d + 1)].reshape(1, top).contiguous() for d in range(ndraw)]
+            else:
+                draws = [torch.stack([torch.randperm(E, generator=g, device=dev)[:top] for _ in range(B)]).to(torch.int32)
+                         for _ in range(ndraw)]
             wts = torch.softmax(torch.randn((B, top), generator=g, device=dev), dim=1)
             x = torch.randn((B, dm), generator=g, device=dev)
-            distinct = int(torch.unique(ids).numel())
+            calls = [(c, d) for d in range(ndraw) for c in range(ncopy)]
+            distinct = [int(torch.unique(draws[d]).numel()) for c, d in calls]
+            cycled = ncopy * int(torch.unique(torch.cat([d.flatten() for d in draws])).numel()) * per_expert
             torch.cuda.synchronize()
             yb = torch.empty((B, dm), device=dev)
-            f = lambda: ctx.moe_ffn(exps["gate"], exps["up"], exps["down"], x, ids, wts, ACT_GGML, out=yb, sync=False)
-            f(); ctx.sync()
-            run = (None if args.no_graph else capture(torch, stream, f)) or f
+
+            def rotation():
+                for c, d in calls:
+                    ctx.moe_ffn(sets[c]["gate"], sets[c]["up"], sets[c]["down"], x, draws[d], wts, ACT_GGML, out=yb, sync=False)
+
+            def resident():
+                ctx.moe_ffn(sets[0]["gate"], sets[0]["up"], sets[0]["down"], x, draws[0], wts, ACT_GGML, out=yb, sync=False)
+
+            rotation(); ctx.sync()
+            run = (None if args.no_graph else capture(torch, stream, rotation)) or rotation
             run(); torch.cuda.synchronize()
-            sm_ = timer.samples_ms(run, 20)          # raw samples for the records (an event pair around each call)
-            ms = timer.time_ms(run, 100)             # the figure: 100 calls back to back between one event pair
-            byts = distinct * per_expert + B * dm * 4 * 2
+            reps = max(2, 96 // len(calls))
+            sm_ = [s_ / len(calls) for s_ in timer.samples_ms(run, reps)]     # ms per call, one sample per rotation
+            ms = sum(sm_) / len(sm_)
+            byts = sum(distinct) / len(calls) * per_expert + B * dm * 4 * 2  # mean distinct-expert bytes of a call
+            run1 = (None if args.no_graph else capture(torch, stream, resident)) or resident
+            run1(); torch.cuda.synchronize()
+            ms1 = timer.time_ms(run1, 100)
+            byts1 = distinct[0] * per_expert + B * dm * 4 * 2
             ev_rows.append(evidence.backend_ops_row("MUL_MAT_ID", evidence.mul_mat_id_params(Q4_K, dff, dm, E, top, B) +
-                                                    ",fused=moe_ffn(gate,up,swiglu,down,combine)", [s * 1e3 for s in sm_],
+                                                    ",fused=moe_ffn(gate,up,swiglu,down,combine)", [s_ * 1e3 for s_ in sm_],
                                                     flops=2.0 * B * top * 3 * dm * dff, bytes_moved=byts,
-                                                    memory_kb=byts // 1024, device=props.name))
-            ev_cal.append(evidence.calibration_metric(Q4_K, True, byts, [s * 1e3 for s in sm_], launch_us=2.0))
-            res.append({"B": B, "distinct_experts": distinct, "ms": ms, "GBps": byts / (ms * 1e-3) / 1e9,
-                        "frac_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
-            log(f"[bench] moe B={B}: {ms * 1e3:.1f} us, {distinct} experts, {res[-1]['GBps']:.0f} GB/s")
+                                                    memory_kb=int(byts) // 1024, device=props.name))
+            ev_cal.append(evidence.calibration_metric(Q4_K, True, byts, [s_ * 1e3 for s_ in sm_], launch_us=2.0))
+            res.append({"B": B, "distinct_experts_mean": sum(distinct) / len(calls), "calls_in_rotation": len(calls),
+                        "bytes_cycled": cycled, "ms": ms, "GBps": byts / (ms * 1e-3) / 1e9,
+                        "frac_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        "cache_resident": {"ms": ms1, "GBps": byts1 / (ms1 * 1e-3) / 1e9, "bytes": byts1}})
+            log(f"[bench] moe B={B}: {ms * 1e3:.1f} us a call over a rotation of {len(calls)} calls cycling {cycled / 1e6:.0f} MB "
+                f"({res[-1]['GBps']:.0f} GB/s from HBM); one draw replayed: {ms1 * 1e3:.1f} us ({res[-1]['cache_resident']['GBps']:.0f} GB/s, "
+                f"{byts1 / 1e6:.0f} MB, may sit in the Infinity Cache)")
         out["moe"] = {"experts": E, "top": top, "d_model": dm, "d_ff": dff, "batches": res,
                       "note": "3 to 6 launches per call ([quantize,] [group,] gate/up+SwiGLU, [quantize,] down, combine: the grouped "
                               "kernel quantizes its own rows when experts have few pairs, and skips the grouping pass for "
-                              "up to 16 pairs), replayed as a HIP graph, 100 calls back to back; "
-                              "the same experts every replay, so weights may sit in the Infinity Cache"}
-        for w in exps.values():
-            w.free()
+                              "up to 16 pairs); the rotation over three weight sets and several id draws is replayed as one "
+                              "HIP graph; GBps counts the distinct experts of each call"}
+        for exps in sets:
+            for w in exps.values():
+                w.free()
 
     # ------------------------------------------------------------------ CPU baseline (oracle, host cores)
     if "cpu" in legs:
@@ -581,7 +707,16 @@ def main():
         if args.evidence_sql:
             with open(args.evidence_sql, "w") as f:
                 f.write("\n".join(evidence.backend_ops_sql(r) for r in ev_rows) + "\n")
-    print(json.dumps(out), flush=True)
+    details = None
+    if args.details_json:
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(args.details_json)), exist_ok=True)
+            with open(args.details_json, "w") as f:
+                json.dump(out, f, indent=1)
+            details = args.details_json
+        except OSError as e:
+            log(f"[bench] details file not written: {e}")
+    print(compact_line(out, details), flush=True)
     return 0
 
 
