@@ -103,7 +103,9 @@ int qproj_dequantize(qproj_ctx *ctx, const qproj_weight *w, float *out_dev);
  *           (msum: d * (sum of the 32 codes of a sub-block) / 16 as an fp16 pair, the 8 high parts of
  *           a super-block, then the 8 low parts; operand of the prefill kernel's min term)
  *   Q8X32 : int8 qs[M][K] | f32 d[M][K/32]  | int32 isum[M][K/32] | f16 msum[M][K/256][16] (as above)
- * each plane starting at a 256-byte aligned offset, in that order. */
+ * each plane starting at a 256-byte aligned offset, in that order.  K must be a multiple of 32 for Q8_0 and of
+ * 256 for Q8_K and Q8X32 (both carry one msum record per 256 weights of a row); qproj_act_bytes returns 0 and
+ * qproj_quantize_activations QPROJ_ERR_INVALID_ARG otherwise. */
 size_t qproj_act_bytes(int kind, int wtype, int64_t M, int64_t K);
 int qproj_quantize_activations(qproj_ctx *ctx, int kind, int wtype, const float *x_dev, int64_t M,
                                int64_t K, void *out_dev);

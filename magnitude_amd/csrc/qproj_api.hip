@@ -627,7 +627,9 @@ size_t qproj_act_bytes(int kind, int wtype, int64_t M, int64_t K) {
     if (M <= 0 || K <= 0) return 0;
     if (kind != kActGGML && kind != kActQ8X32) return 0;
     const int k = act_kind_for(kind, wtype);
-    if (K % (k == kActKindQ8_K ? 256 : 32) != 0) return 0;
+    // The per-32 format carries one min-term record (msum) per 256 weights of a row, like Q8_K, and its quantizer
+    // walks 256 floats at a time: K must be a whole number of super-blocks for both.
+    if (K % (k == kActKindQ8_0 ? 32 : 256) != 0) return 0;
     return act_planes(k, M, K).total;
 }
 

@@ -101,24 +101,35 @@ def load_library(path: Optional[str] = None) -> C.CDLL:
     return lib
 
 
-def probe_eligibility() -> dict:
-    """The backend eligibility entry a HIP backend would add to the server's report, in the contract's
-    serialised shape (/root/reference/inference/crates/icn-contracts/src/bootstrap_protocol.rs:14-39: tag
-    "state" in lowercase, camelCase fields): {"state": "usable", "driverApi", "architectures",
-    "driverLibrary"} or {"state": "absent" | "failed", "diagnostic"}.  "hardwareLabels" and "runtimeApi"
-    ride along for usable devices (the reference keeps its hardware labels beside the report,
-    /root/reference/inference/crates/icn-server/src/cuda_driver.rs:78)."""
+def _probe() -> Eligibility:
     e = Eligibility()
     st = load_library().qproj_probe_eligibility(C.byref(e))
     if st:
         raise QprojError(st, "qproj_probe_eligibility")
+    return e
+
+
+def probe_eligibility() -> dict:
+    """The backend eligibility entry a HIP backend would add to the server's report, in exactly the contract's
+    serialised shape (/root/reference/inference/crates/icn-contracts/src/bootstrap_protocol.rs:14-39: tag
+    "state" in lowercase, camelCase fields, unknown fields denied): {"state": "usable", "driverApi",
+    "architectures", "driverLibrary"} or {"state": "absent" | "failed", "diagnostic"}."""
+    e = _probe()
     if e.state == 0:
-        n = e.n_devices
-        return {"state": "usable", "driverApi": e.driver_api, "runtimeApi": e.runtime_api,
-                "architectures": [e.architectures[i].value.decode() for i in range(n)],
-                "hardwareLabels": [e.hardware_labels[i].value.decode(errors="replace") for i in range(n)],
+        return {"state": "usable", "driverApi": e.driver_api,
+                "architectures": [e.architectures[i].value.decode() for i in range(e.n_devices)],
                 "driverLibrary": e.runtime_library.decode(errors="replace")}
     return {"state": "absent" if e.state == 1 else "failed", "diagnostic": e.diagnostic.decode(errors="replace")}
+
+
+def probe_hardware() -> dict:
+    """What the probe learns beside the contract entry: one hardware label per device and the runtime version
+    (the reference keeps its hardware labels beside the report as well,
+    /root/reference/inference/crates/icn-server/src/cuda_driver.rs:78).  Empty lists when no device is usable."""
+    e = _probe()
+    n = e.n_devices if e.state == 0 else 0
+    return {"runtimeApi": e.runtime_api if e.state == 0 else 0,
+            "hardwareLabels": [e.hardware_labels[i].value.decode(errors="replace") for i in range(n)]}
 
 
 def row_bytes(qtype: int, k: int) -> int:
@@ -405,6 +416,10 @@ class Context:
                 weights: torch.Tensor, act: int = ACT_GGML, out: torch.Tensor = None,
                 sync: bool = True) -> torch.Tensor:
         """y[b] = sum_j weights[b, j] * down_e(silu(gate_e x_b) * up_e x_b), e = ids[b, j]."""
+        if ids.dtype != torch.int32 or x.dtype != torch.float32 or weights.dtype != torch.float32:
+            raise ValueError("ids must be int32, x and weights float32")
+        if ids.dim() != 2 or tuple(weights.shape) != tuple(ids.shape) or x.shape[0] != ids.shape[0]:
+            raise ValueError("ids and weights must be [B, n_used] and x [B, d_model]")
         b, n_used = ids.shape
         y = out if out is not None else torch.empty((b, gate.K), dtype=torch.float32, device=x.device)
         if sync:

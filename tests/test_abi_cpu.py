@@ -41,6 +41,12 @@ def test_version_and_sizes(lib):
     assert lib.qproj_act_bytes(2, 12, 2, 4096) == 8192 + 1024 + 1024 + 1024   # qs | d | isum | fp16 min-term plane
     assert lib.qproj_act_bytes(0, 12, 1, 4000) == 0
     assert lib.qproj_act_bytes(1, 12, 1, 4096) == 0  # fp32 activations are not quantized
+    # the per-32 format keeps one min-term record per 256 weights of a row: K must be whole super-blocks, or the
+    # quantizer would write records the msum plane has no room for
+    for k in (32, 288, 4096 + 32):
+        assert lib.qproj_act_bytes(2, 12, 1000, k) == 0
+        assert lib.qproj_act_bytes(0, 12, 1000, k) == 0
+    assert lib.qproj_act_bytes(0, 8, 1, 288) == 512 + 256   # Q8_0 blocks need K % 32 only
 
 
 def test_null_and_no_device_errors_do_not_crash(lib):
@@ -72,13 +78,16 @@ def test_eligibility_probe_answers_in_the_contract_shape(lib):
     rc = lib.qproj_device_count(C.byref(n))
     if r["state"] == "usable":
         assert rc == 0 and n.value >= 1
-        assert set(r) == {"state", "driverApi", "runtimeApi", "architectures", "hardwareLabels", "driverLibrary"}
+        # exactly the contract's fields: its deserialiser denies unknown ones (bootstrap_protocol.rs:16-21)
+        assert set(r) == {"state", "driverApi", "architectures", "driverLibrary"}
         assert r["driverApi"] > 0 and "gfx950" in r["architectures"]
-        assert len(r["architectures"]) == len(r["hardwareLabels"]) >= n.value
+        hw = qproj.probe_hardware()
+        assert len(r["architectures"]) == len(hw["hardwareLabels"]) >= n.value and hw["runtimeApi"] > 0
         assert r["driverLibrary"]
     else:
         assert rc == 5      # whatever keeps the probe from "usable" also keeps contexts from being created
         assert set(r) == {"state", "diagnostic"}
+        assert qproj.probe_hardware() == {"runtimeApi": 0, "hardwareLabels": []}
         d = r["diagnostic"]
         assert 0 < len(d) <= 240 and "\n" not in d and "\r" not in d
 

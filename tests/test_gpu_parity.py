@@ -113,10 +113,12 @@ def test_eligibility_probe_reports_the_gfx950_device(ctx):
     from magnitude_amd import qproj
     r = qproj.probe_eligibility()
     assert r["state"] == "usable", r
-    assert r["driverApi"] > 0 and r["runtimeApi"] > 0
+    assert set(r) == {"state", "driverApi", "architectures", "driverLibrary"}   # the contract denies unknown fields
+    hw = qproj.probe_hardware()
+    assert r["driverApi"] > 0 and hw["runtimeApi"] > 0
     assert r["architectures"][0] == "gfx950"
-    assert len(r["architectures"]) == len(r["hardwareLabels"]) == torch.cuda.device_count()
-    assert r["hardwareLabels"][0].strip() == r["hardwareLabels"][0] != ""
+    assert len(r["architectures"]) == len(hw["hardwareLabels"]) == torch.cuda.device_count()
+    assert hw["hardwareLabels"][0].strip() == hw["hardwareLabels"][0] != ""
     assert "amdhip64" in r["driverLibrary"]
 
 
@@ -198,6 +200,19 @@ def test_quantize_q8x32_bit_exact(ctx, orc):
     ms = got["msum"].cpu().numpy()
     assert np.array_equal(ms[:, :, 0].view(np.uint16), hi.reshape(m, k // 256, 8).view(np.uint16))
     assert np.array_equal(ms[:, :, 1].view(np.uint16), lo.reshape(m, k // 256, 8).view(np.uint16))
+
+
+def test_quantize_q8x32_rejects_rows_that_are_not_whole_super_blocks(ctx):
+    """The per-32 format keeps one min-term record per 256 weights of a row; with K % 256 != 0 the quantizer
+    would write records the msum plane has no room for, so the ABI refuses before anything is launched."""
+    from magnitude_amd import ACT_Q8X32
+    for m, k in ((1000, 32), (3, 288)):
+        assert ctx.lib.qproj_act_bytes(ACT_Q8X32, Q4_K, m, k) == 0
+        x = torch.zeros((m, k), device="cuda")
+        buf = torch.empty(m * k * 4 + 4096, dtype=torch.uint8, device="cuda")
+        rc = ctx.lib.qproj_quantize_activations(ctx.handle, ACT_Q8X32, Q4_K, x.data_ptr(), m, k, buf.data_ptr())
+        assert rc == 1                      # QPROJ_ERR_INVALID_ARG
+        assert b"shape" in ctx.lib.qproj_last_error(ctx.handle)
 
 
 # ---------------------------------------------------------------- mul_mat, decode and small M
