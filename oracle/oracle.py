@@ -56,8 +56,9 @@ def lib() -> C.CDLL:
         L.orc_get_scale_min_k4.argtypes = [i32, vp, vp, vp]
         L.orc_pack_scale_min_k4.argtypes = [vp, vp, vp]
         L.orc_dequantize_row.argtypes = [i32, vp, f32p, i64]
-        L.orc_quantize_row.argtypes = [i32, f32p, vp, i64]
+        L.orc_quantize_rows.restype = i32
         L.orc_quantize_rows.argtypes = [i32, f32p, vp, i64, i64, i32]
+        L.orc_quantize_row_q8_0.argtypes = [f32p, vp, i64]
         L.orc_quantize_row_q8_K.argtypes = [f32p, vp, i64]
         L.orc_quantize_row_q8x32.argtypes = [f32p, vp, i64]
         for name in ("orc_vec_dot_q8_0_q8_0", "orc_vec_dot_q4_K_q8_K", "orc_vec_dot_q6_K_q8_K"):
@@ -97,11 +98,13 @@ def fp16_to_fp32(h: int) -> float:
 
 
 def quantize(qtype: int, w: np.ndarray, nthreads: int = 8) -> np.ndarray:
-    """float32 [N, K] -> uint8 [N, row_bytes] of GGUF blocks."""
+    """float32 [N, K] -> uint8 [N, row_bytes] of GGUF Q8_0 blocks (quantize_row_q8_0_ref).  The oracle makes no
+    Q4_K / Q6_K weight blocks: those are inputs of the path (tests/kquant_encoders.py encodes test inputs)."""
     w = np.ascontiguousarray(w, dtype=np.float32)
     n, k = w.shape
     out = np.zeros((n, row_bytes(qtype, k)), dtype=np.uint8)
-    lib().orc_quantize_rows(qtype, _p(w), _p(out), k, n, nthreads)
+    if lib().orc_quantize_rows(qtype, _p(w), _p(out), k, n, nthreads) != 0:
+        raise ValueError("the oracle quantizes weights to Q8_0 only (K a multiple of 32)")
     return out
 
 
@@ -130,7 +133,7 @@ def quantize_q8_0_act(x: np.ndarray) -> np.ndarray:
     rows = x.reshape(-1, k)
     out = np.zeros((rows.shape[0], k // 32 * 34), dtype=np.uint8)
     for r in range(rows.shape[0]):
-        lib().orc_quantize_row(TYPE_Q8_0, _p(rows[r]), _p(out[r]), k)
+        lib().orc_quantize_row_q8_0(_p(rows[r]), _p(out[r]), k)
     return out
 
 

@@ -5,8 +5,7 @@
  * Upstream functions restated here live in llama.cpp @ 0b1bad14 (absent from
  * /root/reference; pinned by /root/reference/inference/native-pin.toml:11-14):
  *   ggml/src/ggml-common.h      block_q8_0, block_q4_K, block_q6_K, block_q8_K
- *   ggml/src/ggml-quants.c      quantize_row_*_ref, dequantize_row_*, make_qkx2_quants,
- *                               make_qx_quants, nearest_int, get_scale_min_k4
+ *   ggml/src/ggml-quants.c      quantize_row_q8_0_ref, dequantize_row_*, nearest_int, get_scale_min_k4
  *   ggml/src/ggml-cpu/quants.c  ggml_vec_dot_*_generic, quantize_row_q8_K
  *   ggml/src/ggml-cpu/ggml-cpu.c ggml_compute_forward_mul_mat{,_id}
  *   src/llama-graph.cpp         build_moe_ffn
@@ -322,238 +321,17 @@ void orc_quantize_row_q8_K(const float *x, orc_block_q8_K *y, int64_t k) {
     }
 }
 
-/* ggml-quants.c make_qkx2_quants: weighted affine fit (scale, min<=0) of n
- * values onto 0..nmax, refined over nstep+1 candidate inverse scales. */
-static float fit_affine_qkx2(int n, int nmax, const float *x, const float *w, uint8_t *L,
-                             float *the_min, uint8_t *Laux, float rmin, float rdelta, int nstep) {
-    float lo = x[0], hi = x[0];
-    float sum_w = w[0];
-    float sum_x = sum_w * x[0];
-    for (int i = 1; i < n; ++i) {
-        if (x[i] < lo) lo = x[i];
-        if (x[i] > hi) hi = x[i];
-        sum_w += w[i];
-        sum_x += w[i] * x[i];
-    }
-    if (lo > 0) lo = 0;
-    if (hi == lo) {
-        for (int i = 0; i < n; ++i) L[i] = 0;
-        *the_min = -lo;
-        return 0.f;
-    }
-    float iscale = nmax / (hi - lo);
-    float scale = 1 / iscale;
-    float best = 0;
-    for (int i = 0; i < n; ++i) {
-        int l = nearest_int(iscale * (x[i] - lo));
-        L[i] = (uint8_t)ORC_MAX(0, ORC_MIN(nmax, l));
-        float diff = scale * L[i] + lo - x[i];
-        best += w[i] * (diff * diff);
-    }
-    for (int is = 0; is <= nstep; ++is) {
-        iscale = (rmin + rdelta * is + nmax) / (hi - lo);
-        float sum_l = 0, sum_l2 = 0, sum_xl = 0;
-        for (int i = 0; i < n; ++i) {
-            int l = nearest_int(iscale * (x[i] - lo));
-            l = ORC_MAX(0, ORC_MIN(nmax, l));
-            Laux[i] = (uint8_t)l;
-            sum_l += w[i] * l;
-            sum_l2 += w[i] * l * l;
-            sum_xl += w[i] * l * x[i];
-        }
-        const float D = sum_w * sum_l2 - sum_l * sum_l;
-        if (D > 0) {
-            float this_scale = (sum_w * sum_xl - sum_x * sum_l) / D;
-            float this_min = (sum_l2 * sum_x - sum_l * sum_xl) / D;
-            if (this_min > 0) {
-                this_min = 0;
-                this_scale = sum_xl / sum_l2;
-            }
-            float err = 0;
-            for (int i = 0; i < n; ++i) {
-                float diff = this_scale * Laux[i] + this_min - x[i];
-                err += w[i] * (diff * diff);
-            }
-            if (err < best) {
-                for (int i = 0; i < n; ++i) L[i] = Laux[i];
-                best = err;
-                scale = this_scale;
-                lo = this_min;
-            }
-        }
-    }
-    *the_min = -lo;
-    return scale;
-}
-
-/* ggml-quants.c quantize_row_q4_K_ref */
-void orc_quantize_row_q4_K(const float *x, orc_block_q4_K *y, int64_t k) {
-    const int64_t nb = k / ORC_QK_K;
-    uint8_t L[ORC_QK_K], Laux[32];
-    float weights[32], mins[8], scales[8];
-    for (int64_t i = 0; i < nb; ++i) {
-        float max_scale = 0, max_min = 0;
-        for (int j = 0; j < 8; ++j) {
-            float sum_x2 = 0;
-            for (int l = 0; l < 32; ++l) sum_x2 += x[32 * j + l] * x[32 * j + l];
-            const float av_x = sqrtf(sum_x2 / 32);
-            for (int l = 0; l < 32; ++l) weights[l] = av_x + fabsf(x[32 * j + l]);
-            scales[j] = fit_affine_qkx2(32, 15, x + 32 * j, weights, L + 32 * j, &mins[j], Laux, -1.f,
-                                        0.1f, 20);
-            if (scales[j] > max_scale) max_scale = scales[j];
-            if (mins[j] > max_min) max_min = mins[j];
-        }
-        const float inv_scale = max_scale > 0 ? 63.f / max_scale : 0.f;
-        const float inv_min = max_min > 0 ? 63.f / max_min : 0.f;
-        uint8_t ls8[8], lm8[8];
-        for (int j = 0; j < 8; ++j) {
-            int ls = nearest_int(inv_scale * scales[j]);
-            int lm = nearest_int(inv_min * mins[j]);
-            ls8[j] = (uint8_t)ORC_MIN(63, ls);
-            lm8[j] = (uint8_t)ORC_MIN(63, lm);
-        }
-        orc_pack_scale_min_k4(ls8, lm8, y[i].scales);
-        y[i].d = orc_fp32_to_fp16(max_scale / 63.f);
-        y[i].dmin = orc_fp32_to_fp16(max_min / 63.f);
-        for (int j = 0; j < 8; ++j) {
-            uint8_t sc, m;
-            orc_get_scale_min_k4(j, y[i].scales, &sc, &m);
-            const float d = orc_fp16_to_fp32(y[i].d) * sc;
-            if (!d) continue;
-            const float dm = orc_fp16_to_fp32(y[i].dmin) * m;
-            for (int ii = 0; ii < 32; ++ii) {
-                int l = nearest_int((x[32 * j + ii] + dm) / d);
-                l = ORC_MAX(0, ORC_MIN(15, l));
-                L[32 * j + ii] = (uint8_t)l;
-            }
-        }
-        uint8_t *q = y[i].qs;
-        for (int j = 0; j < ORC_QK_K; j += 64) {
-            for (int l = 0; l < 32; ++l) q[l] = (uint8_t)(L[j + l] | (L[j + l + 32] << 4));
-            q += 32;
-        }
-        x += ORC_QK_K;
-    }
-}
-
-/* ggml-quants.c make_qx_quants with rmse_type = 1 (weights x^2), no external weights */
-static float fit_symmetric_qx(int n, int nmax, const float *x, int8_t *L) {
-    float max = 0, amax = 0;
-    for (int i = 0; i < n; ++i) {
-        float ax = fabsf(x[i]);
-        if (ax > amax) {
-            amax = ax;
-            max = x[i];
-        }
-    }
-    if (amax < ORC_GROUP_MAX_EPS) {
-        for (int i = 0; i < n; ++i) L[i] = 0;
-        return 0.f;
-    }
-    float iscale = -nmax / max;
-    float sumlx = 0, suml2 = 0;
-    for (int i = 0; i < n; ++i) {
-        int l = nearest_int(iscale * x[i]);
-        l = ORC_MAX(-nmax, ORC_MIN(nmax - 1, l));
-        L[i] = (int8_t)(l + nmax);
-        float w = x[i] * x[i];
-        sumlx += w * x[i] * l;
-        suml2 += w * l * l;
-    }
-    float scale = suml2 ? sumlx / suml2 : 0.0f;
-    float best = scale * sumlx;
-    for (int is = -9; is <= 9; ++is) {
-        if (is == 0) continue;
-        iscale = -(nmax + 0.1f * is) / max;
-        sumlx = suml2 = 0;
-        for (int i = 0; i < n; ++i) {
-            int l = nearest_int(iscale * x[i]);
-            l = ORC_MAX(-nmax, ORC_MIN(nmax - 1, l));
-            float w = x[i] * x[i];
-            sumlx += w * x[i] * l;
-            suml2 += w * l * l;
-        }
-        if (suml2 > 0 && sumlx * sumlx > best * suml2) {
-            for (int i = 0; i < n; ++i) {
-                int l = nearest_int(iscale * x[i]);
-                L[i] = (int8_t)(nmax + ORC_MAX(-nmax, ORC_MIN(nmax - 1, l)));
-            }
-            scale = sumlx / suml2;
-            best = scale * sumlx;
-        }
-    }
-    return scale;
-}
-
-/* ggml-quants.c quantize_row_q6_K_ref */
-void orc_quantize_row_q6_K(const float *x, orc_block_q6_K *y, int64_t k) {
-    const int64_t nb = k / ORC_QK_K;
-    int8_t L[ORC_QK_K];
-    float scales[16];
-    for (int64_t i = 0; i < nb; ++i) {
-        float max_scale = 0, max_abs_scale = 0;
-        for (int ib = 0; ib < 16; ++ib) {
-            const float scale = fit_symmetric_qx(16, 32, x + 16 * ib, L + 16 * ib);
-            scales[ib] = scale;
-            const float a = fabsf(scale);
-            if (a > max_abs_scale) {
-                max_abs_scale = a;
-                max_scale = scale;
-            }
-        }
-        if (max_abs_scale < ORC_GROUP_MAX_EPS) {
-            memset(&y[i], 0, sizeof(y[i]));
-            x += ORC_QK_K;
-            continue;
-        }
-        const float iscale = -128.f / max_scale;
-        y[i].d = orc_fp32_to_fp16(1 / iscale);
-        for (int ib = 0; ib < 16; ++ib)
-            y[i].scales[ib] = (int8_t)ORC_MIN(127, nearest_int(iscale * scales[ib]));
-        for (int j = 0; j < 16; ++j) {
-            const float d = orc_fp16_to_fp32(y[i].d) * y[i].scales[j];
-            if (!d) continue;
-            for (int ii = 0; ii < 16; ++ii) {
-                int l = nearest_int(x[16 * j + ii] / d);
-                l = ORC_MAX(-32, ORC_MIN(31, l));
-                L[16 * j + ii] = (int8_t)(l + 32);
-            }
-        }
-        uint8_t *ql = y[i].ql;
-        uint8_t *qh = y[i].qh;
-        for (int j = 0; j < ORC_QK_K; j += 128) {
-            for (int l = 0; l < 32; ++l) {
-                const uint8_t q1 = L[j + l + 0] & 0xF;
-                const uint8_t q2 = L[j + l + 32] & 0xF;
-                const uint8_t q3 = L[j + l + 64] & 0xF;
-                const uint8_t q4 = L[j + l + 96] & 0xF;
-                ql[l + 0] = (uint8_t)(q1 | (q3 << 4));
-                ql[l + 32] = (uint8_t)(q2 | (q4 << 4));
-                qh[l] = (uint8_t)((L[j + l] >> 4) | ((L[j + l + 32] >> 4) << 2) |
-                                  ((L[j + l + 64] >> 4) << 4) | ((L[j + l + 96] >> 4) << 6));
-            }
-            ql += 64;
-            qh += 32;
-        }
-        x += ORC_QK_K;
-    }
-}
-
-void orc_quantize_row(int type, const float *x, void *blocks, int64_t k) {
-    switch (type) {
-    case ORC_TYPE_Q8_0: orc_quantize_row_q8_0(x, (orc_block_q8_0 *)blocks, k); break;
-    case ORC_TYPE_Q4_K: orc_quantize_row_q4_K(x, (orc_block_q4_K *)blocks, k); break;
-    case ORC_TYPE_Q6_K: orc_quantize_row_q6_K(x, (orc_block_q6_K *)blocks, k); break;
-    default: break;
-    }
-}
-
-void orc_quantize_rows(int type, const float *x, void *blocks, int64_t k, int64_t nrows, int nthreads) {
+/* Weight-side quantizer of the oracle: Q8_0 only (the one the benchmark configuration defines completely).
+ * Q4_K / Q6_K weight blocks are INPUTS of this path -- models arrive quantized -- and the tests make them with the
+ * format-valid encoders of tests/kquant_encoders.c, which are not part of the oracle. */
+int orc_quantize_rows(int type, const float *x, void *blocks, int64_t k, int64_t nrows, int nthreads) {
+    if (type != ORC_TYPE_Q8_0 || k % ORC_QK8_0 != 0) return -1;
     const size_t rb = orc_row_bytes(type, k);
     if (nthreads < 1) nthreads = 1;
 #pragma omp parallel for num_threads(nthreads) schedule(static)
     for (int64_t r = 0; r < nrows; ++r)
-        orc_quantize_row(type, x + r * k, (char *)blocks + (size_t)r * rb, k);
+        orc_quantize_row_q8_0(x + r * k, (orc_block_q8_0 *)((char *)blocks + (size_t)r * rb), k);
+    return 0;
 }
 
 /* ---------------------------------------------------------------- dot products */

@@ -23,18 +23,22 @@
  *   dequantize_row_{q8_0,q4_K,q6_K} pinned: closed forms on hand-built blocks
  *                                 and an independent numpy restatement.
  *   quantize_row_q8_0 ........... pinned: fully specified by the benchmark
- *                                 config (d = amax/127 as fp16, q = round(w/d)).
+ *                                 config (d = amax/127 as fp16, q = round(w/d));
+ *                                 roundf's half-away-from-zero ties and the zero
+ *                                 block by hand-computed vectors.
  *   vec_dot_* integer partials .. pinned: brute force in int64/fp64 from the
  *                                 dequantized values; one-hot and linearity.
- *   quantize_row_q8_K ........... PARITY UNPINNED against ggml (tie behaviour
- *                                 and the -127 constant are recalled, no
- *                                 reference-held vector exists); it is pinned
- *                                 only as "a valid per-256 int8 quantizer".
- *   quantize_row_q4_K / q6_K .... PARITY UNPINNED against ggml (search
- *                                 heuristics recalled); format-valid and
- *                                 quality-bounded only.  They produce test
- *                                 inputs; both sides of every parity test
- *                                 consume the same blocks.
+ *   quantize_row_q8_K ........... pinned to the published algorithm by hand-computed
+ *                                 vectors that a plausible variant fails: half-to-even
+ *                                 ties of nearest_int (roundf differs), the -127
+ *                                 constant (-128 differs), "first element of the
+ *                                 strictly largest magnitude" (last-wins differs),
+ *                                 d = 1/iscale bit for bit (-max/127 differs), the
+ *                                 clamp at 127, 16-wide block sums.  No reference-held
+ *                                 vector exists for it (llama.cpp is not vendored).
+ *   Q4_K / Q6_K weight quantizers  NOT PART OF THE ORACLE: weight blocks are inputs of
+ *                                 the path.  The tests make them with the format-valid
+ *                                 encoders of tests/kquant_encoders.c.
  *   fp32 association in vec_dot . follows ggml's generic C code; ggml's own
  *                                 SIMD paths associate differently, so GPU
  *                                 comparisons use a tolerance, integers exact.
@@ -98,11 +102,9 @@ void orc_dequantize_row_q8_0(const orc_block_q8_0 *x, float *y, int64_t k);
 void orc_dequantize_row_q4_K(const orc_block_q4_K *x, float *y, int64_t k);
 void orc_dequantize_row_q6_K(const orc_block_q6_K *x, float *y, int64_t k);
 
-void orc_quantize_row(int type, const float *x, void *blocks, int64_t k);
-void orc_quantize_rows(int type, const float *x, void *blocks, int64_t k, int64_t nrows, int nthreads);
+/* Q8_0 only (returns -1 otherwise): Q4_K / Q6_K weight blocks are inputs of the path, not made by the oracle */
+int orc_quantize_rows(int type, const float *x, void *blocks, int64_t k, int64_t nrows, int nthreads);
 void orc_quantize_row_q8_0(const float *x, orc_block_q8_0 *y, int64_t k);
-void orc_quantize_row_q4_K(const float *x, orc_block_q4_K *y, int64_t k);
-void orc_quantize_row_q6_K(const float *x, orc_block_q6_K *y, int64_t k);
 void orc_quantize_row_q8_K(const float *x, orc_block_q8_K *y, int64_t k);
 void orc_quantize_row_q8x32(const float *x, orc_block_q8x32 *y, int64_t k);
 

@@ -11,6 +11,8 @@ import numpy as np
 import pytest
 import torch
 
+from kquant_encoders import encode
+
 pytestmark = pytest.mark.gpu
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
@@ -80,7 +82,7 @@ def make_weight(orc, qtype, n, k, seed):
 def _make_weight(orc, qtype, n, k, seed):
     rng = np.random.default_rng(seed)
     w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
-    return orc.quantize(qtype, w)
+    return encode(qtype, w)
 
 
 # ---------------------------------------------------------------- dequantize / upload
@@ -389,7 +391,7 @@ def test_prefill_gemm_q8x32_matches_oracle(ctx, orc, m, k, n):
 def moe(orc):
     d_model, d_ff, E = 2048, 768, 16
     rng = np.random.default_rng(8)
-    q = lambda rows, cols, s: orc.quantize(Q4_K, (np.random.default_rng(s).standard_normal((E * rows, cols)) * 0.02).astype(np.float32)).reshape(E, rows, -1)
+    q = lambda rows, cols, s: encode(Q4_K, (np.random.default_rng(s).standard_normal((E * rows, cols)) * 0.02).astype(np.float32)).reshape(E, rows, -1)
     return dict(d_model=d_model, d_ff=d_ff, E=E, gate=q(d_ff, d_model, 81), up=q(d_ff, d_model, 82),
                 down=q(d_model, d_ff, 83), rng=rng)
 
@@ -428,7 +430,7 @@ def test_mul_mat_id_grouping_of_many_pairs(ctx, orc, E, B):
     the grouped kernel also runs its several-passes-per-expert loop."""
     from magnitude_amd import ACT_GGML
     k, n, top = 256, 32, 8
-    blocks = orc.quantize(Q4_K, (np.random.default_rng(E + B).standard_normal((E * n, k)) * 0.02).astype(np.float32)).reshape(E, n, -1)
+    blocks = encode(Q4_K, (np.random.default_rng(E + B).standard_normal((E * n, k)) * 0.02).astype(np.float32)).reshape(E, n, -1)
     rng = np.random.default_rng(7 * E + B)
     ids, _ = routing(rng, B, top, E)
     w = ctx.upload(Q4_K, k, n, blocks, n_expert=E)
@@ -727,7 +729,7 @@ def test_mul_mat_random_shapes_sweep(ctx, orc, seed):
         mode = ACT_GGML if rng.random() < 0.7 else (ACT_F32 if rng.random() < 0.5 else ACT_Q8X32)
         if mode == ACT_Q8X32 and (qt != Q4_K or k % 256):
             mode = ACT_GGML
-        blocks = orc.quantize(qt, (rng.standard_normal((n, k)) * 0.02).astype(np.float32))
+        blocks = encode(qt, (rng.standard_normal((n, k)) * 0.02).astype(np.float32))
         x = rng.standard_normal((m, k)).astype(np.float32)
         if rng.random() < 0.2:
             x[:, rng.integers(0, k, max(1, k // 100))] *= 20
@@ -754,7 +756,7 @@ def test_mul_mat_id_random_shapes_sweep(ctx, orc, seed):
         k = int(256 * rng.choice([1, 2, 3, 8, 16]))
         n = int(rng.choice([32, 96, 100, 256, 768, 1000]))
         nb1 = 1 if rng.random() < 0.5 else top
-        wb = orc.quantize(qt, (rng.standard_normal((E * n, k)) * 0.02).astype(np.float32))
+        wb = encode(qt, (rng.standard_normal((E * n, k)) * 0.02).astype(np.float32))
         ids = np.stack([rng.permutation(E)[:top] for _ in range(B)]).astype(np.int32)
         x = rng.standard_normal((B, nb1, k)).astype(np.float32)
         w = ctx.upload(qt, k, n, wb, n_expert=E)

@@ -8,11 +8,13 @@ and brute force in int64/fp64.  Each check is chosen so that a dropped term, a
 wrong shift or a swapped nibble fails it.
 """
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
 
 import np_ref
+from kquant_encoders import encode
 
 Q8_0, Q4_K, Q6_K = 8, 12, 14
 
@@ -206,7 +208,7 @@ def test_quantize_q8_0_matches_spec(orc):
     w = (rng.standard_normal((64, 4096)) * 0.02).astype(np.float32)
     w[3, 32:64] = 0.0                      # an all-zero block
     w[5, 0:32] = np.float32(0.02)          # constant block
-    got = orc.quantize(Q8_0, w)
+    got = encode(Q8_0, w)
     want = np_ref.quant_q8_0(w).reshape(64, -1)
     assert np.array_equal(got, want)
     deq = orc.dequantize(Q8_0, got, 4096)
@@ -217,11 +219,13 @@ def test_quantize_q8_0_matches_spec(orc):
 
 
 @pytest.mark.parametrize("qtype,rmse_max", [(Q4_K, 0.002), (Q6_K, 0.002), (Q8_0, 0.002)])
-def test_quantizer_round_trip_quality(orc, qtype, rmse_max):
-    """ggml's own test-quantize-fns bound (recalled): array_rmse <= 0.002 on 0.1 + 2cos(i)."""
+def test_encoder_round_trip_quality(orc, qtype, rmse_max):
+    """The tests' weight encoders (kquant_encoders.c; Q8_0: the oracle's quantizer) against the bound ggml's own
+    test-quantize-fns uses (recalled): array_rmse <= 0.002 on 0.1 + 2cos(i).  A quality check of test inputs,
+    decoded by the oracle's pinned dequantizer -- not a parity pin."""
     i = np.arange(4096, dtype=np.float32)
     x = (0.1 + 2.0 * np.cos(i + 0.0)).astype(np.float32)[None, :]
-    blocks = orc.quantize(qtype, x)
+    blocks = encode(qtype, x)
     y = orc.dequantize(qtype, blocks, 4096)
     # upstream array_rmse is sqrt(sum of squared differences) / n, threshold 0.002
     err = np.sqrt(np.sum((x.astype(np.float64) - y) ** 2)) / x.size
@@ -230,16 +234,35 @@ def test_quantizer_round_trip_quality(orc, qtype, rmse_max):
 
 
 @pytest.mark.parametrize("qtype", [Q4_K, Q6_K])
-def test_k_quantizer_outputs_are_valid_and_close(orc, qtype):
+def test_encoder_outputs_are_valid_and_close(orc, qtype):
     rng = np.random.default_rng(21)
     w = (rng.standard_normal((32, 2048)) * 0.02).astype(np.float32)
-    blocks = orc.quantize(qtype, w)
+    blocks = encode(qtype, w)
     y = orc.dequantize(qtype, blocks, 2048)
     rel = np.linalg.norm(y - w) / np.linalg.norm(w)
     assert rel < (0.08 if qtype == Q4_K else 0.02), rel
     # all-zero input -> all-zero output
-    z = orc.quantize(qtype, np.zeros((1, 256), np.float32))
+    z = encode(qtype, np.zeros((1, 256), np.float32))
     assert np.array_equal(orc.dequantize(qtype, z, 256), np.zeros((1, 256), np.float32))
+
+
+def test_the_oracle_makes_no_k_quant_weights(orc):
+    """Q4_K / Q6_K weight blocks are inputs of the path; nothing under oracle/ claims to restate ggml's offline
+    quantizer for them."""
+    with pytest.raises(ValueError):
+        orc.quantize(Q4_K, np.zeros((1, 256), np.float32))
+    with pytest.raises(ValueError):
+        orc.quantize(Q6_K, np.zeros((1, 256), np.float32))
+    src = open(os.path.join(os.path.dirname(orc.__file__), "qproj_oracle.c")).read()
+    assert "orc_quantize_row_q4_K" not in src and "orc_quantize_row_q6_K" not in src and "make_qkx2" not in src
+
+
+def _q8_K(orc, x):
+    raw = orc.quantize_q8_K(np.asarray(x, np.float32))[0].reshape(-1, 292)
+    d = raw[:, 0:4].copy().view(np.float32)[:, 0]
+    qs = raw[:, 4:260].view(np.int8).astype(np.int32)
+    bs = raw[:, 260:292].copy().view(np.int16).astype(np.int32)
+    return d, qs, bs
 
 
 def test_quantize_q8_K_properties(orc):
@@ -248,10 +271,7 @@ def test_quantize_q8_K_properties(orc):
     rng = np.random.default_rng(3)
     x = rng.standard_normal(1024).astype(np.float32)
     x[256:512] = 0.0
-    raw = orc.quantize_q8_K(x)[0].reshape(4, 292)
-    d = raw[:, 0:4].copy().view(np.float32)[:, 0]
-    qs = raw[:, 4:260].view(np.int8).astype(np.int32)
-    bs = raw[:, 260:292].copy().view(np.int16).astype(np.int32)
+    d, qs, bs = _q8_K(orc, x)
     assert d[1] == 0 and not qs[1].any() and not bs[1].any()
     for b in (0, 2, 3):
         xb = x[256 * b: 256 * b + 256]
@@ -260,6 +280,98 @@ def test_quantize_q8_K_properties(orc):
         assert np.isclose(d[b], -xb[imax] / 127.0, rtol=1e-6)
         assert np.all(np.abs(qs[b] - xb / d[b]) <= 0.5 + 1e-4)
         assert np.array_equal(bs[b], qs[b].reshape(16, 16).sum(axis=1))
+
+
+def test_quantize_q8_K_ties_round_half_to_even(orc):
+    """Hand-computed from the published algorithm (quantize_row_q8_K: iscale = -127/max, q = nearest_int(iscale*x),
+    nearest_int = round half to even through the 2^23 + 2^22 addend).  With max = 127 the inverse scale is exactly
+    -1, so the codes are the negated inputs rounded: +-0.5 -> 0, +-1.5 -> -+2, +-2.5 -> -+2, +-3.5 -> -+4.
+    roundf (half away from zero) would give -+1, -+2, -+3, -+4 and fails here."""
+    x = np.zeros(256, np.float32)
+    x[0] = 127.0
+    ties = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 3.5, -3.5, 126.5, -126.5, 0.49999997, 0.50000006]
+    want = [0, 0, -2, 2, -2, 2, -4, 4, -126, 126, 0, -1]
+    x[16:16 + len(ties)] = ties
+    d, qs, bs = _q8_K(orc, x)
+    assert d[0].view(np.uint32) == np.float32(-1.0).view(np.uint32)          # d = 1/iscale = 1/(-1)
+    assert qs[0, 0] == -127
+    assert qs[0, 16:16 + len(ties)].tolist() == want
+    assert bs[0, 0] == -127 and bs[0, 1] == sum(want) and not bs[0, 2:].any()
+
+
+def test_quantize_q8_K_first_largest_magnitude_sets_the_sign(orc):
+    """`if (ax > amax)` is strict: of several elements of the same largest magnitude the FIRST one is `max`.
+    x[3] = -8, x[10] = +8: max = -8, iscale = -127/-8 = 15.875, d = 1/15.875, q[3] = -127, q[10] = +127.
+    A last-wins (or positive-wins) rule gives iscale = -15.875, d < 0 and the two codes swapped."""
+    x = np.zeros(256, np.float32)
+    x[3], x[10], x[200] = -8.0, 8.0, 4.0
+    d, qs, _ = _q8_K(orc, x)
+    assert d[0].view(np.uint32) == (np.float32(1.0) / np.float32(15.875)).view(np.uint32) and d[0] > 0
+    assert qs[0, 3] == -127 and qs[0, 10] == 127 and qs[0, 200] == 64        # 63.5 -> 64: half to even
+    x[3], x[10] = 8.0, -8.0
+    d, qs, _ = _q8_K(orc, x)
+    assert d[0] < 0 and qs[0, 3] == -127 and qs[0, 10] == 127 and qs[0, 200] == -64
+
+
+def test_quantize_q8_K_constant_is_127_and_d_is_the_reciprocal_of_iscale(orc):
+    """The pinned revision scales by -127/max (older ones by -128/max) and stores d = 1/iscale, two roundings,
+    which is not always the one rounding of -max/127: both are told apart bit for bit."""
+    m127 = np.float32(-127.0)
+    differ = 0
+    for mx in np.float32([3.0, 0.7, 1.6625982522964478, 60.667510986328125, 2.841683864593506, 12.437085151672363,
+                          1e-3, 123.456, 7e4, 13.518299102783203]):
+        x = np.zeros(256, np.float32)
+        x[77] = mx
+        x[5] = -mx * np.float32(0.5)
+        d, qs, _ = _q8_K(orc, x)
+        iscale = m127 / mx                                   # fp32 division, as in the C source
+        want_d = np.float32(1.0) / iscale
+        assert d[0].view(np.uint32) == want_d.view(np.uint32), mx
+        assert qs[0, 77] == -127                              # -128 with the older constant
+        # the half-size element: iscale * x is computed in fp32, then rounded half to even
+        prod = np.float32(iscale * x[5])
+        assert qs[0, 5] == int(np.rint(prod)) and abs(int(qs[0, 5]) - 63.5) <= 0.5
+        differ += want_d.view(np.uint32) != (-mx / np.float32(127.0)).view(np.uint32)
+    assert differ >= 5          # the vectors do separate 1/iscale from -max/127
+
+
+def test_quantize_q8_K_clamps_at_127(orc):
+    """`MIN(127, v)`: an element of the opposite sign and (almost) the same magnitude lands on +127, never 128.
+    max = x[0] = -1 (iscale = 127): x[1] = 0.99999994 -> 126.99999 -> 127; x[2] = +1 cannot be `max` (not strictly
+    larger) and gives exactly 127."""
+    x = np.zeros(256, np.float32)
+    x[0], x[1], x[2] = -1.0, np.float32(0.99999994), 1.0
+    d, qs, _ = _q8_K(orc, x)
+    assert qs[0, :3].tolist() == [-127, 127, 127] and qs.max() == 127 and qs.min() == -127
+    assert d[0].view(np.uint32) == (np.float32(1.0) / np.float32(127.0)).view(np.uint32)
+
+
+def test_quantize_q8_0_ties_round_half_away_from_zero(orc):
+    """quantize_row_q8_0_ref: d = amax/127, id = 1/d, q = roundf(x*id).  With amax = 127 both are exactly 1, so the
+    codes are the inputs rounded half AWAY from zero (+-0.5 -> +-1, +-2.5 -> +-3), where the K-quant activation
+    quantizer's nearest_int would give 0 and +-2; d is stored as fp16 1.0 = 0x3C00.  Same vector through the
+    activation-side entry point, which is the same function."""
+    x = np.zeros((1, 64), np.float32)
+    x[0, 0] = -127.0
+    ties = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 126.5, -126.5, 0.49999997]
+    want = [1, -1, 2, -2, 3, -3, 127, -127, 0]
+    x[0, 1:1 + len(ties)] = ties
+    for raw in (orc.quantize(Q8_0, x), orc.quantize_q8_0_act(x[0])):
+        blk = raw.reshape(2, 34)
+        assert blk[0, 0:2].copy().view(np.uint16)[0] == 0x3C00
+        q = blk[0, 2:].view(np.int8)
+        assert q[0] == -127 and q[1:1 + len(ties)].tolist() == want and not q[1 + len(ties):].any()
+        assert not blk[1].any()                               # the all-zero block: d = 0, id = 0, codes 0
+    # d is rounded to fp16 but the codes use the unrounded fp32 scale: amax = 1 -> d = 1/127, id = 1/d
+    y = np.zeros((1, 32), np.float32)
+    y[0, 0], y[0, 1], y[0, 2] = 1.0, np.float32(0.5), np.float32(63.5 / 127)
+    d32 = np.float32(1.0) / np.float32(127.0)
+    idv = np.float32(1.0) / d32
+    blk = orc.quantize(Q8_0, y).reshape(34)
+    assert blk[0:2].copy().view(np.uint16)[0] == np.float16(d32).view(np.uint16)
+    for j in range(3):
+        v = np.float32(y[0, j] * idv)
+        assert blk[2:].view(np.int8)[j] == int(np.sign(v) * np.floor(np.abs(v) + np.float32(0.5)))
 
 
 def test_quantize_q8x32_properties(orc):
@@ -295,7 +407,7 @@ def test_vec_dot_q4_K_q8_K_brute_force(orc, k):
     rng = np.random.default_rng(k)
     w = (rng.standard_normal((1, k)) * 0.02).astype(np.float32)
     x = rng.standard_normal(k).astype(np.float32)
-    wb = orc.quantize(Q4_K, w)
+    wb = encode(Q4_K, w)
     q, sc, mn, d, dmin = np_ref.q4_K_ints(wb)
     ax = orc.quantize_q8_K(x)[0]
     dx, a = _act_q8_K_parts(ax, k)
@@ -315,7 +427,7 @@ def test_vec_dot_q6_K_q8_K_brute_force(orc, k):
     rng = np.random.default_rng(k + 1)
     w = (rng.standard_normal((1, k)) * 0.02).astype(np.float32)
     x = rng.standard_normal(k).astype(np.float32)
-    wb = orc.quantize(Q6_K, w)
+    wb = encode(Q6_K, w)
     q, sc, d = np_ref.q6_K_ints(wb)
     ax = orc.quantize_q8_K(x)[0]
     dx, a = _act_q8_K_parts(ax, k)
@@ -330,7 +442,7 @@ def test_vec_dot_q8_0_q8_0_brute_force(orc, k):
     rng = np.random.default_rng(k + 2)
     w = (rng.standard_normal((1, k)) * 0.02).astype(np.float32)
     x = rng.standard_normal(k).astype(np.float32)
-    wb = orc.quantize(Q8_0, w)
+    wb = encode(Q8_0, w)
     ab = orc.quantize_q8_0_act(x)[0]
     W = wb.reshape(-1, 34)
     A = ab.reshape(-1, 34)
@@ -350,7 +462,7 @@ def test_vec_dot_q8x32_brute_force(orc, qtype):
     w = (rng.standard_normal((3, k)) * 0.02).astype(np.float32)
     x = rng.standard_normal((2, k)).astype(np.float32)
     x[:, 5] *= 20
-    wb = orc.quantize(qtype, w)
+    wb = encode(qtype, w)
     wd = orc.dequantize(qtype, wb, k).astype(np.float64)
     raw = orc.quantize_q8x32(x).reshape(2, k // 32, 40)
     d = raw[:, :, 0:4].copy().view(np.float32)[:, :, 0].astype(np.float64)
@@ -368,7 +480,7 @@ def test_mul_mat_one_hot_selects_dequantized_weight(orc, qtype):
     k = 512
     rng = np.random.default_rng(9)
     w = (rng.standard_normal((8, k)) * 0.02).astype(np.float32)
-    wb = orc.quantize(qtype, w)
+    wb = encode(qtype, w)
     wd = orc.dequantize(qtype, wb, k)
     for kk in (0, 15, 16, 31, 32, 63, 64, 100, 255, 256, 300, 511):
         x = np.zeros((1, k), np.float32)
@@ -387,7 +499,7 @@ def test_mul_mat_linearity_and_zero(orc, qtype):
     rng = np.random.default_rng(10)
     w = (rng.standard_normal((16, k)) * 0.02).astype(np.float32)
     x = rng.standard_normal((1, k)).astype(np.float32)
-    wb = orc.quantize(qtype, w)
+    wb = encode(qtype, w)
     y1 = orc.mul_mat(qtype, wb, k, x, orc.ACT_GGML)
     y4 = orc.mul_mat(qtype, wb, k, 4 * x, orc.ACT_GGML)
     assert np.array_equal(4 * y1, y4)
@@ -406,7 +518,7 @@ def test_ggml_activation_noise_is_what_the_design_notes_say(orc):
     rng = np.random.default_rng(12)
     w = (rng.standard_normal((n, k)) * 0.02).astype(np.float32)
     x = rng.standard_normal((1, k)).astype(np.float32)
-    wb = orc.quantize(Q4_K, w)
+    wb = encode(Q4_K, w)
     yq = orc.mul_mat(Q4_K, wb, k, x, orc.ACT_GGML)[0]
     ye = orc.mul_mat_f64(Q4_K, wb, k, x)[0]
     big = np.abs(ye) >= 1
@@ -420,7 +532,7 @@ def test_mul_mat_id_equals_loop_of_dense(orc):
     k, n, E, B, top = 512, 24, 6, 5, 3
     rng = np.random.default_rng(13)
     w = (rng.standard_normal((E * n, k)) * 0.02).astype(np.float32)
-    wb = orc.quantize(Q4_K, w).reshape(E, n, -1)
+    wb = encode(Q4_K, w).reshape(E, n, -1)
     ids = np.stack([rng.permutation(E)[:top] for _ in range(B)]).astype(np.int32)
     x1 = rng.standard_normal((B, 1, k)).astype(np.float32)
     xt = rng.standard_normal((B, top, k)).astype(np.float32)
@@ -440,7 +552,7 @@ def test_mul_mat_id_equals_loop_of_dense(orc):
 def test_moe_ffn_equals_explicit_numpy(orc):
     d_model, d_ff, E, B, top = 512, 256, 8, 4, 3
     rng = np.random.default_rng(14)
-    q = lambda rows, cols: orc.quantize(Q4_K, (rng.standard_normal((E * rows, cols)) * 0.02).astype(np.float32)).reshape(E, rows, -1)
+    q = lambda rows, cols: encode(Q4_K, (rng.standard_normal((E * rows, cols)) * 0.02).astype(np.float32)).reshape(E, rows, -1)
     gate, up, down = q(d_ff, d_model), q(d_ff, d_model), q(d_model, d_ff)
     ids = np.stack([rng.permutation(E)[:top] for _ in range(B)]).astype(np.int32)
     logits = rng.standard_normal((B, top)).astype(np.float32)
