@@ -152,6 +152,12 @@ int qproj_mul_mat(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int
 int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev,
                         int64_t M, float *const *y_dev, int act);
 
+/* Scratch bytes qproj_mul_mat_multi reserves for n tensors of `type` with rows N[0..n) sharing K, M activation
+ * rows and activation mode `act` (0 for the decode regime, which needs none).  Needs no device: it walks the
+ * library's own dispatch for that shape without launching, and checks on the way that every kernel launcher it
+ * picks accepts a buffer of exactly that size and refuses a smaller one; *status (may be null) is QPROJ_OK then. */
+size_t qproj_workspace_bytes(int type, int64_t K, int n, const int64_t *N, int64_t M, int act, int *status);
+
 /* The second half of a MUL_MAT on its own: `act_dev` holds M rows already quantized by
  * qproj_quantize_activations(kind, type of w[0], ...).  ggml converts src1 once per MUL_MAT; a
  * caller that feeds one activation to several weights (q/k/v) converts once and calls this. */

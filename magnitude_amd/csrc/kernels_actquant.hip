@@ -37,6 +37,7 @@ hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, i
                                int16_t *bsums, uint16_t *msum, int32_t *isum, hipStream_t s) {
     const int64_t n = M * K;
     if (n == 0) return hipSuccess;
+    if (dry_run()) return kind == kActKindQ8_K || kind == kActKindQ8_0 || kind == kActKindQ8X32 ? hipSuccess : hipErrorInvalidValue;
     const int64_t chunks = (n + 255) / 256;
     const dim3 grid((unsigned)((chunks + 3) / 4)), block(256);
     if (kind == kActKindQ8_K) {

@@ -349,11 +349,6 @@ int cu_count() {
     return n;
 }
 
-int env_int(const char *name, int dflt) {
-    const char *e = getenv(name);
-    return e && *e ? atoi(e) : dflt;
-}
-
 template <int QT, int MT, int R, bool XREG, bool FUSE, bool PAIR = false>
 hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
     constexpr int CH = Geo<QT>::kChunk;
@@ -367,7 +362,7 @@ hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
     for (int i = 0; i < a.n_targets; ++i) rows_total += a.t[i].w.N;
     if (rows_total == 0) return hipSuccess;
     // one workgroup per CU, fewer when there are not enough rows to give every wave one
-    static const int wgs_per_cu = env_int("QPROJ_DECODE_WGS_PER_CU", 1);
+    static const int wgs_per_cu = tuning_int("QPROJ_DECODE_WGS_PER_CU", 1);
     int64_t grid = (int64_t)cu_count() * wgs_per_cu;
     const int64_t need = (rows_total + kDecodeWaves - 1) / kDecodeWaves;  // at least one row per wave
     if (grid > need) grid = need;
@@ -390,6 +385,7 @@ hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
     const int kpad = (int)((K + CH - 1) / CH * CH);
     const size_t smem = (size_t)MT * kpad + (size_t)MT * (kpad / BLK) * 4 + (!is_q8_0<QT> ? (size_t)MT * (kpad / 16) * 2 : 0);
     if (PAIR) a.n_targets = 2;
+    if (dry_run()) return hipSuccess;
     auto kern = &gemv_decode_kernel<QT, MT, R, XREG, FUSE, PAIR>;
     if (smem > 48 * 1024) {
         static size_t allowed = 0;

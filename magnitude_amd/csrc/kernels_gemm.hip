@@ -831,23 +831,26 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(const float *__restrict_
 }
 
 template <int QT>
-hipError_t launch_per32(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s) {
+hipError_t launch_per32(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &sc, hipStream_t s) {
+    const int n_split = sc.p ? per32_splits(w.K, M, w.N) : 1;
+    if (n_split > 1 && (size_t)n_split * M * w.N * 4 > sc.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
+    if (dry_run()) return hipSuccess;
     const auto kern = &gemm_per32_kernel<QT>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem));
     if (attr != hipSuccess) return attr;
-    const int n_split = scratch ? per32_splits(w.K, M, w.N) : 1;
     const dim3 grid((unsigned)(((w.N + BN - 1) / BN) * ((M + BM - 1) / BM)), (unsigned)n_split);
-    hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y, scratch);
+    hipLaunchKernelGGL(kern, grid, dim3(kGemmThreads), sizeof(GemmSmem), s, w, a, M, y, sc.p);
     if (n_split > 1) {
         const size_t n4 = (size_t)M * w.N / 4;
-        hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, scratch, n_split, n4, y);
+        hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, sc.p, n_split, n4, y);
     }
     return hipGetLastError();
 }
 }  // namespace
 
 hipError_t launch_sum_parts(const float *part, int n_split, size_t n, float *y, hipStream_t s) {
+    if (dry_run()) return hipSuccess;
     const size_t n4 = n / 4;   // callers only split when n is a multiple of 4
     hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, part, n_split, n4, y);
     return hipGetLastError();
@@ -858,7 +861,7 @@ hipError_t launch_sum_parts(const float *part, int n_split, size_t n, float *y, 
 // stretch (K = 4096 cut in two measured slower than whole: the pass that adds the partial tiles costs more
 // than the fuller grid gains).
 int q8k_tile_splits(int64_t K, int64_t M, int64_t N) {
-    static const int forced = getenv("QPROJ_Q8K_SPLITS") ? atoi(getenv("QPROJ_Q8K_SPLITS")) : 0;
+    static const int forced = tuning_int("QPROJ_Q8K_SPLITS", 0);
     const int64_t tiles = ((N + 127) / 128) * ((M + 63) / 64);
     int n = forced > 0 ? forced : tiles >= 384 ? 1 : tiles >= 192 ? 2 : tiles >= 96 ? 3 : 4;
     if ((M * N) % 4 != 0) n = 1;
@@ -876,7 +879,7 @@ size_t q8k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N) {
 // A grid of fewer than 192 tiles leaves the 256 compute units (two workgroups each) mostly idle and a
 // workgroup's K loop is latency-bound: K is then cut into 2 or 3 stretches done by different workgroups.
 int per32_splits(int64_t K, int64_t M, int64_t N) {
-    static const int forced = getenv("QPROJ_PER32_SPLITS") ? atoi(getenv("QPROJ_PER32_SPLITS")) : 0;
+    static const int forced = tuning_int("QPROJ_PER32_SPLITS", 0);
     const int64_t tiles = ((N + BN - 1) / BN) * ((M + BM - 1) / BM);
     int n = forced > 0 ? forced : tiles >= 192 ? 1 : tiles >= 96 ? 2 : 3;
     if ((M * N) % 4 != 0) n = 1;
@@ -888,25 +891,26 @@ size_t per32_scratch_bytes(int64_t K, int64_t M, int64_t N) {
     return n > 1 ? (size_t)n * M * N * 4 : 0;
 }
 
-hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s) {
+hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s) {
     if (w.type != kTypeQ4_K || w.K % 256 != 0 || M <= 0 || !a.msum) return hipErrorInvalidValue;
     return launch_per32<kTypeQ4_K>(w, a, M, y, scratch, s);
 }
 
 // Q8_0 weights x ggml Q8_0 activation blocks (planes in `a`), K a multiple of 128
-hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s) {
+hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s) {
     if (w.type != kTypeQ8_0 || a.kind != kActKindQ8_0 || w.K % BK != 0 || M <= 0) return hipErrorInvalidValue;
     return launch_per32<kTypeQ8_0>(w, a, M, y, scratch, s);
 }
 
 // ggml-format activations (Q8_K planes in `a`, including the min-term plane), Q4_K weights, any M
-hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s) {
+hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s) {
     if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || !a.msum || M <= 0) return hipErrorInvalidValue;
     if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 64 token rows of K bytes, 32 weight rows of K*144/256
     // large batches: 128 tokens x 256 weight rows per workgroup, one workgroup per compute unit
-    static const int wide_env = getenv("QPROJ_Q8K_WIDE") ? atoi(getenv("QPROJ_Q8K_WIDE")) : -1;
+    static const int wide_env = tuning_int("QPROJ_Q8K_WIDE", -1);
     const int64_t wide_tiles = ((w.N + 255) / 256) * ((M + 127) / 128);
     if (wide_env >= 0 ? wide_env != 0 : wide_tiles >= 192) {
+        if (dry_run()) return hipSuccess;
         using Smem = WideSmem<8>;
         const auto kern = &gemm_q4k_q8k_wide_kernel<8>;
         static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -917,27 +921,29 @@ hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, flo
     }
     constexpr int NW = 4;   // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit
     using Smem = DirectSmem<NW>;
+    const int n_split = scratch.p ? q8k_tile_splits(w.K, M, w.N) : 1;
+    if (n_split > 1 && (size_t)n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
+    if (dry_run()) return hipSuccess;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_direct_kernel<NW>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
     if (attr != hipSuccess) return attr;
-    const int n_split = scratch ? q8k_tile_splits(w.K, M, w.N) : 1;
     const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64)), (unsigned)n_split);
     DirectTargets tg{};
     tg.n = 1;
     tg.w[0] = w;
     tg.y[0] = y;
-    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, tg, a, M, scratch);
-    if (n_split > 1) return launch_sum_parts(scratch, n_split, (size_t)M * w.N, y, s);
+    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, tg, a, M, scratch.p);
+    if (n_split > 1) return launch_sum_parts(scratch.p, n_split, (size_t)M * w.N, y, s);
     return hipGetLastError();
 }
 
 // The same for n matrices over the same activation rows.  One launch where every matrix would take the
 // 64-token kernel with K in one stretch; otherwise one launch a matrix, as above.
-hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, int64_t M, float *const *y, float *scratch,
-                                 hipStream_t s) {
+hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, int64_t M, float *const *y,
+                                 const Scratch &scratch, hipStream_t s) {
     constexpr int NW = 4;
-    static const int wide_env = getenv("QPROJ_Q8K_WIDE") ? atoi(getenv("QPROJ_Q8K_WIDE")) : -1;
-    static const bool off = getenv("QPROJ_Q8K_NO_MULTI") != nullptr;
+    static const int wide_env = tuning_int("QPROJ_Q8K_WIDE", -1);
+    static const bool off = tuning_int("QPROJ_Q8K_NO_MULTI", 0) != 0;
     // the matrices that would take the 64-token kernel with K in one stretch go together; the others (128-token
     // tiles, K cut into stretches) get their own launches first
     const bool can = !off && n >= 2 && n <= 3 && wide_env < 0 && a.kind == kActKindQ8_K && a.msum && M > 0;
@@ -945,7 +951,7 @@ hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, i
     for (int i = 0; i < n; ++i) {
         const int64_t wide_tiles = ((w[i].N + 255) / 256) * ((M + 127) / 128);
         const bool fits = can && w[i].type == kTypeQ4_K && w[i].K == w[0].K && w[i].K <= (1 << 24) && wide_tiles < 192 &&
-                          (!scratch || q8k_tile_splits(w[i].K, M, w[i].N) == 1 ||
+                          (!scratch.p || q8k_tile_splits(w[i].K, M, w[i].N) == 1 ||
                            ((w[i].N + 127) / 128) * ((M + 63) / 64) < 96);   // small ones are better off together than cut
         if (fits) joined[n_joined++] = i;
     }
@@ -957,7 +963,7 @@ hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, i
         hipError_t e = launch_gemm_q8k(w[i], a, M, y[i], scratch, s);
         if (e != hipSuccess) return e;
     }
-    if (n_joined == 0) return hipSuccess;
+    if (n_joined == 0 || dry_run()) return hipSuccess;
     using Smem = DirectSmem<NW>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_direct_kernel<NW>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));

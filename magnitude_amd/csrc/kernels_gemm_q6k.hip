@@ -280,6 +280,7 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
 namespace {
 template <int NW, int JT>
 hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, int n_split, hipStream_t s) {
+    if (dry_run()) return hipSuccess;
     using Smem = Q6Smem<NW, JT>;
     const auto kern = &gemm_q6k_q8k_kernel<NW, JT>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -293,14 +294,15 @@ hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y
 }  // namespace
 
 // ggml-format activations (Q8_K planes in `a`), Q6_K weights, any M
-hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s) {
+hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s) {
     if (w.type != kTypeQ6_K || a.kind != kActKindQ8_K || !a.bsums || M <= 0) return hipErrorInvalidValue;
     if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 64 token rows of K bytes, 32 weight rows of K/2
     // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit.  A grid of such tiles that
     // would leave compute units idle is filled by cutting K into stretches (partial tiles added afterwards);
     // where K is too short for that, 32-token tiles double the number of workgroups instead.
-    const int n_split = scratch ? q8k_tile_splits(w.K, M, w.N) : 1;
-    if (n_split > 1 || ((w.N + 127) / 128) * ((M + 63) / 64) >= 384) return launch_q6k<4, 2>(w, a, M, y, scratch, n_split, s);
+    const int n_split = scratch.p ? q8k_tile_splits(w.K, M, w.N) : 1;
+    if (n_split > 1 && (size_t)n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
+    if (n_split > 1 || ((w.N + 127) / 128) * ((M + 63) / 64) >= 384) return launch_q6k<4, 2>(w, a, M, y, scratch.p, n_split, s);
     return launch_q6k<4, 1>(w, a, M, y, nullptr, 1, s);
 }
 

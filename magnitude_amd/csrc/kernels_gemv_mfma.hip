@@ -681,6 +681,7 @@ __global__ __launch_bounds__(256) void sum_chunks_kernel(const MfmaArgs g) {
 
 template <int QT, int NI, int W, int MODE>
 hipError_t launch_one(const MfmaArgs &g, hipStream_t s) {
+    if (dry_run()) return hipSuccess;
     const Layout L = layout<QT, 8 * NI, W>(g.chunk_sb);
     auto kern = gemv_mfma_kernel<QT, NI, W, MODE>;
     static int allowed = 0;
@@ -702,8 +703,7 @@ hipError_t launch_one(const MfmaArgs &g, hipStream_t s) {
 
 int waves_per_wg(int type) {
     static const int w = [] {
-        const char *e = getenv("QPROJ_MFMA_WAVES");
-        const int v = e ? atoi(e) : 8;
+        const int v = tuning_int("QPROJ_MFMA_WAVES", 8);
         return v == 4 || v == 16 ? v : 8;
     }();
     return w == 16 && type != kTypeQ4_K ? 8 : w;   // 16 regions of the larger formats do not fit LDS
@@ -761,7 +761,7 @@ size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, in
     return p.n_chunks > 1 ? (size_t)p.n_chunks * (size_t)M * (size_t)sum_n * 4 : 0;
 }
 
-hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s) {
+hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStream_t s) {
     MfmaArgs g{};
     g.n_targets = args.n_targets;
     g.a = args.a;
@@ -782,7 +782,7 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s)
     for (int i = 0; i < args.n_targets; ++i) {
         g.t[i].w = args.t[i].w;
         g.t[i].y = args.t[i].y;
-        g.t[i].part = scratch ? scratch + part_off : nullptr;
+        g.t[i].part = scratch.p ? scratch.p + part_off : nullptr;
         part_off += (size_t)g.n_chunks * args.M * args.t[i].w.N;
         const int n_rg = (int)((args.t[i].w.N + 31) / 32);
         g.t[i].n_rowsets = (n_rg + g.rw - 1) / g.rw;
@@ -790,7 +790,8 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s)
         wg += g.t[i].n_rowsets * g.n_chunks;
     }
     g.n_wgs = wg;
-    if (g.n_chunks > 1 && !scratch) return hipErrorInvalidValue;
+    // the per-chunk results of all targets lie one behind the other in the scratch: refuse what would not fit
+    if (g.n_chunks > 1 && (!scratch.p || part_off * sizeof(float) > scratch.bytes)) return hipErrorInvalidValue;
     return launch_typed<kDense>(g, args.t[0].w.type, args.M <= 8, W, s);
 }
 
@@ -830,7 +831,7 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
     // the 128-expert FFN's down projection (K = 768): worth it for a grid of one to three workgroups per
     // compute unit (416 workgroups: the FFN at B = 8 goes from 61.6 to 55.3 us), neutral above (992
     // workgroups, B = 64), harmful below (64 workgroups, B = 1: 24 -> 31 us), and four in a row always lose.
-    static const int forced_loop = getenv("QPROJ_MOE_RG_LOOP") ? atoi(getenv("QPROJ_MOE_RG_LOOP")) : 0;
+    static const int forced_loop = tuning_int("QPROJ_MOE_RG_LOOP", 0);
     {
         const int64_t wgs1 = (args.ids ? n_pairs : std::min<int64_t>(w.E, n_pairs)) * ((rg_e + g.rw - 1) / g.rw);
         const int64_t cus = 256;

@@ -280,7 +280,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ g
 }
 
 hipError_t launch_swiglu(const float *g, const float *u, size_t n, float *h, hipStream_t s) {
-    if (n == 0) return hipSuccess;
+    if (n == 0 || dry_run()) return hipSuccess;
     hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, g, u, n, h);
     return hipGetLastError();
 }

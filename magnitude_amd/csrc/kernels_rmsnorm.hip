@@ -89,6 +89,7 @@ hipError_t launch_rms_norm(int kind, const float *x, const float *gamma, float e
                            int8_t *qs, float *d, int16_t *bsums, uint16_t *msum, int32_t *isum, hipStream_t s) {
     if (M == 0) return hipSuccess;
     if (K <= 0 || K % 32 != 0) return hipErrorInvalidValue;
+    if (dry_run()) return hipSuccess;
     const dim3 grid((unsigned)M), block(kNormThreads);
     if (kind < 0) {
         hipLaunchKernelGGL(rms_norm_kernel<0>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, msum, isum);

@@ -14,6 +14,24 @@
 
 using namespace qproj;
 
+namespace qproj {
+namespace {
+thread_local bool g_dry_run = false;
+}
+bool dry_run() { return g_dry_run; }
+void set_dry_run(bool on) { g_dry_run = on; }
+
+int tuning_int(const char *name, int dflt) {
+#ifdef QPROJ_TUNING
+    const char *e = getenv(name);
+    return e && *e ? atoi(e) : dflt;
+#else
+    (void)name;
+    return dflt;
+#endif
+}
+}  // namespace qproj
+
 struct qproj_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -76,6 +94,37 @@ int ensure_ws(qproj_ctx *ctx, size_t bytes) {
     const size_t want = align_up(bytes + bytes / 4);
     QP_HIP(ctx, hipMalloc((void **)&ctx->ws, want));
     ctx->ws_bytes = want;
+    return QPROJ_OK;
+}
+
+// Where an operator call keeps its scratch: the context's growable buffer (reserve may allocate), or a fixed
+// buffer that is never grown.
+struct Workspace {
+    uint8_t *base;
+    size_t cap;
+    bool fixed;
+    size_t reserved = 0;   // what the call asked for (the largest request)
+};
+
+int reserve(qproj_ctx *ctx, Workspace &ws, size_t bytes) {
+    ws.reserved = std::max(ws.reserved, bytes);
+    if (dry_run() && !ws.fixed) {   // sizes only: any non-null base will do, nothing is dereferenced
+        ws.base = reinterpret_cast<uint8_t *>(uintptr_t(256));
+        ws.cap = bytes;
+        return QPROJ_OK;
+    }
+    if (ws.fixed) {
+        if (bytes > ws.cap) {
+            char buf[160];
+            snprintf(buf, sizeof buf, "this call needs %zu bytes of scratch, the fixed buffer holds %zu", bytes, ws.cap);
+            return fail(ctx, QPROJ_ERR_INVALID_ARG, buf);
+        }
+        return QPROJ_OK;
+    }
+    int rc = ensure_ws(ctx, bytes);
+    if (rc) return rc;
+    ws.base = ctx->ws;
+    ws.cap = ctx->ws_bytes;
     return QPROJ_OK;
 }
 
@@ -264,18 +313,18 @@ int upload_common(qproj_ctx *ctx, int type, int64_t K, int64_t N, int64_t n_expe
 
 // dense mul_mat over quantized activations already sitting in `a` (M rows)
 bool use_decode_kernel(int type, int64_t M, int64_t K) {
-    static const bool off = getenv("QPROJ_NO_DECODE_KERNEL") != nullptr;
+    static const bool off = tuning_int("QPROJ_NO_DECODE_KERNEL", 0) != 0;
     return !off && M <= 4 && decode_kernel_fits(type, pow2_ceil(M), K);
 }
 
 bool use_mfma_grouped(int type, int64_t K) {
-    static const bool off = getenv("QPROJ_NO_MFMA_GEMV") != nullptr;
+    static const bool off = tuning_int("QPROJ_NO_MFMA_GEMV", 0) != 0;
     return !off && mfma_grouped_fits(type, K);
 }
 
 bool use_mfma_kernel(int type, int64_t M, int64_t K) {
-    static const bool off = getenv("QPROJ_NO_MFMA_GEMV") != nullptr;
-    static const int min_m = getenv("QPROJ_MFMA_MIN_M") ? atoi(getenv("QPROJ_MFMA_MIN_M")) : 3;
+    static const bool off = tuning_int("QPROJ_NO_MFMA_GEMV", 0) != 0;
+    static const int min_m = tuning_int("QPROJ_MFMA_MIN_M", 3);
     return !off && M >= min_m && mfma_gemv_fits(type, std::min<int64_t>(M, 16), K);
 }
 
@@ -311,15 +360,15 @@ size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
 // rows, which costs more than the separate quantizer launch saves (gate+up, M = 4 / 8 / 16: 22.1 /
 // 26.9 / 38.5 us fused against 20.5 / 20.8 / 22.7 us).
 bool dense_fuses_quantizer(const qproj_weight *w, int64_t M) {
-    static const bool on = getenv("QPROJ_FUSED_QUANT_DENSE") && atoi(getenv("QPROJ_FUSED_QUANT_DENSE"));
+    static const bool on = tuning_int("QPROJ_FUSED_QUANT_DENSE", 0) != 0;
     return on && M <= 16 && use_mfma_kernel(w->type, M, w->K);
 }
 
 // x_f32: non-null when `a` carries no planes and the kernel quantizes these rows itself (small batches only)
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
-                    float *const *y, float *scratch, const float *x_f32 = nullptr) {
+                    float *const *y, const Scratch &sc, const float *x_f32 = nullptr) {
     // (never under 17: the scratch for K cut into stretches is sized for more than 16 rows only)
-    static const int gemm_min_m = std::max(17, getenv("QPROJ_GEMM_MIN_M") ? atoi(getenv("QPROJ_GEMM_MIN_M")) : 17);
+    static const int gemm_min_m = std::max(17, tuning_int("QPROJ_GEMM_MIN_M", 17));
     // Beyond the 16 rows one pass of the small-batch kernel takes: the tiled product, weights reused across 64
     // tokens, K cut into stretches where the grid would leave the chip idle.  (Measured, 8B shapes: Q4_K 17..47
     // rows 19-72 us in steps of 16 against 15-31 us tiled; Q6_K, whose workgroups are slow -- a vector
@@ -334,14 +383,14 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
         if (w[0]->type == kTypeQ4_K && n >= 2 && n <= 3) {   // q/k/v, gate/up: one launch where the tiles allow it
             WeightView views[3];
             for (int i = 0; i < n; ++i) views[i] = w[i]->view;
-            QP_HIP(ctx, launch_gemm_q8k_multi(n, views, a, M, y, scratch, ctx->stream));
+            QP_HIP(ctx, launch_gemm_q8k_multi(n, views, a, M, y, sc, ctx->stream));
             return QPROJ_OK;
         }
         for (int i = 0; i < n; ++i) {
             const int t = w[0]->type;
-            QP_HIP(ctx, t == kTypeQ4_K   ? launch_gemm_q8k(w[i]->view, a, M, y[i], scratch, ctx->stream)
-                        : t == kTypeQ6_K ? launch_gemm_q6k_q8k(w[i]->view, a, M, y[i], scratch, ctx->stream)
-                                         : launch_gemm_q8_0(w[i]->view, a, M, y[i], scratch, ctx->stream));
+            QP_HIP(ctx, t == kTypeQ4_K   ? launch_gemm_q8k(w[i]->view, a, M, y[i], sc, ctx->stream)
+                        : t == kTypeQ6_K ? launch_gemm_q6k_q8k(w[i]->view, a, M, y[i], sc, ctx->stream)
+                                         : launch_gemm_q8_0(w[i]->view, a, M, y[i], sc, ctx->stream));
         }
         return QPROJ_OK;
     }
@@ -358,7 +407,7 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
             g.x = x_f32;   // (only with M <= 16: a single pass)
             g.M = (int)mc;
             g.x_div = 1;
-            QP_HIP(ctx, launch_gemv_mfma(g, scratch, ctx->stream));
+            QP_HIP(ctx, launch_gemv_mfma(g, sc, ctx->stream));
         }
         return QPROJ_OK;
     }
@@ -395,14 +444,14 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
 // (every workgroup of the expert repeats that work): two launches less per MoE layer, 40.5 -> 33.7 us
 // at one token, 73 -> 68 us at eight, no difference any more at four pairs an expert
 bool grouped_fuses_quantizer(int type, int64_t K, int64_t n_pairs, int64_t E) {
-    static const bool on = !(getenv("QPROJ_NO_FUSED_QUANT") && atoi(getenv("QPROJ_NO_FUSED_QUANT")));
+    static const bool on = tuning_int("QPROJ_NO_FUSED_QUANT", 0) == 0;
     return on && use_mfma_grouped(type, K) && n_pairs <= 2 * E;
 }
 
 // a handful of pairs (one or two decode tokens): no grouping pass, a set of workgroups per pair; an expert
 // that does come twice is simply read twice
 bool grouped_pair_mode(int type, int64_t K, int64_t n_pairs, int64_t E) {
-    static const bool on = !(getenv("QPROJ_NO_PAIR_MODE") && atoi(getenv("QPROJ_NO_PAIR_MODE")));
+    static const bool on = tuning_int("QPROJ_NO_PAIR_MODE", 0) == 0;
     return on && grouped_fuses_quantizer(type, K, n_pairs, E) && n_pairs <= 16;
 }
 
@@ -682,7 +731,7 @@ struct NormSpec {   // RMS norm (+ weights) applied to the rows before they are 
 }  // namespace
 
 static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
-                              float *const *y_dev, int act, const NormSpec *norm) {
+                              float *const *y_dev, int act, const NormSpec *norm, Workspace &wsp) {
     if (!ctx) return QPROJ_ERR_INVALID_ARG;
     if (n <= 0 || n > kMaxTargets || !w || !y_dev || !x_dev)
         return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: null argument or more than 4 tensors");
@@ -694,7 +743,7 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
             return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat_multi: tensors must share K and type");
     }
     if (M == 0) return QPROJ_OK;
-    QP_HIP(ctx, hipSetDevice(ctx->device));
+    if (!dry_run()) QP_HIP(ctx, hipSetDevice(ctx->device));
     const int64_t K = w[0]->K;
     if (act == kActGGML && !use_mfma_kernel(w[0]->type, M, K) && use_decode_kernel(w[0]->type, M, K) &&
         (!norm || decode_kernel_norm_fits(pow2_ceil(M), K))) {
@@ -718,43 +767,44 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
         if (act == kActQ8X32 && w[0]->type != kTypeQ4_K)
             return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat: the per-32 int8 path is built for Q4_K weights");
         if (act == kActGGML && !norm && dense_fuses_quantizer(w[0], M)) {
-            int rc = ensure_ws(ctx, dense_scratch_bytes(n, w, M));
+            const size_t extra = dense_scratch_bytes(n, w, M);
+            int rc = reserve(ctx, wsp, extra);
             if (rc) return rc;
             ActView a{};
             a.kind = act_kind_for(act, w[0]->type);
             a.K = K;
-            return run_dense_q8act(ctx, n, w, a, M, y_dev, reinterpret_cast<float *>(ctx->ws), x_dev);
+            return run_dense_q8act(ctx, n, w, a, M, y_dev, Scratch{reinterpret_cast<float *>(wsp.base), extra}, x_dev);
         }
         const ActPlanes p = act_planes(act_kind_for(act, w[0]->type), M, K);
         const size_t extra = act == kActGGML ? dense_scratch_bytes(n, w, M) : per32_scratch_max(n, w, M);
-        int rc = ensure_ws(ctx, p.total + extra);
+        int rc = reserve(ctx, wsp, p.total + extra);
         if (rc) return rc;
+        uint8_t *ws = wsp.base;
         if (norm) {   // norm, weights and quantizer in one launch
             if (p.kind == kActKindQ8X32 && K % 256 != 0)
                 return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_rms_norm_mul_mat: the per-32 format needs K % 256 == 0");
             QP_HIP(ctx, launch_rms_norm(p.kind, x_dev, norm->gamma, norm->eps, M, K, nullptr,
-                                        reinterpret_cast<int8_t *>(ctx->ws + p.off_qs), reinterpret_cast<float *>(ctx->ws + p.off_d),
-                                        reinterpret_cast<int16_t *>(ctx->ws + p.off_aux),
-                                        reinterpret_cast<uint16_t *>(ctx->ws + p.off_msum),
-                                        reinterpret_cast<int32_t *>(ctx->ws + p.off_aux), ctx->stream));
+                                        reinterpret_cast<int8_t *>(ws + p.off_qs), reinterpret_cast<float *>(ws + p.off_d),
+                                        reinterpret_cast<int16_t *>(ws + p.off_aux),
+                                        reinterpret_cast<uint16_t *>(ws + p.off_msum),
+                                        reinterpret_cast<int32_t *>(ws + p.off_aux), ctx->stream));
         } else {
-            QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, M, K));
+            QP_HIP(ctx, run_quantize(ctx, p, ws, x_dev, M, K));
         }
-        const ActView a = act_view(p, ctx->ws, K);
-        if (act == kActGGML)
-            return run_dense_q8act(ctx, n, w, a, M, y_dev, reinterpret_cast<float *>(ctx->ws + p.total));
-        for (int i = 0; i < n; ++i)
-            QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], extra ? reinterpret_cast<float *>(ctx->ws + p.total) : nullptr,
-                                          ctx->stream));
+        const ActView a = act_view(p, ws, K);
+        // the partial results lie behind the activation planes; `extra` is all a launcher may use of it
+        const Scratch sc{extra ? reinterpret_cast<float *>(ws + p.total) : nullptr, extra};
+        if (act == kActGGML) return run_dense_q8act(ctx, n, w, a, M, y_dev, sc);
+        for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], sc, ctx->stream));
         return QPROJ_OK;
     }
     if (act == kActF32) {
         if (norm) {   // normalised rows to the workspace, then the fp32 kernel reads them
-            int rc = ensure_ws(ctx, (size_t)M * K * 4);
+            int rc = reserve(ctx, wsp, (size_t)M * K * 4);
             if (rc) return rc;
-            QP_HIP(ctx, launch_rms_norm(-1, x_dev, norm->gamma, norm->eps, M, K, reinterpret_cast<float *>(ctx->ws), nullptr,
+            QP_HIP(ctx, launch_rms_norm(-1, x_dev, norm->gamma, norm->eps, M, K, reinterpret_cast<float *>(wsp.base), nullptr,
                                         nullptr, nullptr, nullptr, nullptr, ctx->stream));
-            x_dev = reinterpret_cast<const float *>(ctx->ws);
+            x_dev = reinterpret_cast<const float *>(wsp.base);
         }
         for (int64_t m0 = 0; m0 < M; m0 += 4) {
             const int64_t mc = std::min<int64_t>(4, M - m0);
@@ -774,15 +824,58 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
     return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: unknown activation mode");
 }
 
+static Workspace ctx_workspace(qproj_ctx *ctx) { return Workspace{ctx ? ctx->ws : nullptr, ctx ? ctx->ws_bytes : 0, false}; }
+
 int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
                         float *const *y_dev, int act) {
-    return mul_mat_multi_impl(ctx, n, w, x_dev, M, y_dev, act, nullptr);
+    Workspace wsp = ctx_workspace(ctx);
+    return mul_mat_multi_impl(ctx, n, w, x_dev, M, y_dev, act, nullptr, wsp);
+}
+
+size_t qproj_workspace_bytes(int type, int64_t K, int n, const int64_t *N, int64_t M, int act, int *status) {
+    // Walks the dispatch of qproj_mul_mat_multi for this shape without touching a device: the same code that serves
+    // a call sizes its scratch, hands it to the launchers it picks, and every launcher checks its own demand against
+    // what it was given.  *status is QPROJ_OK when all of them were satisfied.
+    if (status) *status = QPROJ_ERR_INVALID_ARG;
+    if (!type_ok(type) || n <= 0 || n > kMaxTargets || !N || M < 0 || K <= 0 || K % block_elems(type) != 0) return 0;
+    qproj_ctx ctx;
+    qproj_weight ws[kMaxTargets];
+    const qproj_weight *wp[kMaxTargets];
+    float *yp[kMaxTargets];
+    for (int i = 0; i < n; ++i) {
+        if (N[i] <= 0) return 0;
+        ws[i].type = type;
+        ws[i].K = K;
+        ws[i].N = N[i];
+        ws[i].E = 1;
+        ws[i].dev = reinterpret_cast<uint8_t *>(uintptr_t(256));
+        make_view(&ws[i]);
+        wp[i] = &ws[i];
+        yp[i] = reinterpret_cast<float *>(uintptr_t(256));
+    }
+    const float *fake_x = reinterpret_cast<const float *>(uintptr_t(256));
+    set_dry_run(true);
+    Workspace sized{nullptr, 0, false};
+    int rc = mul_mat_multi_impl(&ctx, n, wp, fake_x, M, yp, act, nullptr, sized);
+    const size_t total = sized.reserved;
+    if (rc == QPROJ_OK) {   // against a fixed buffer of exactly that size every launcher must be satisfied ...
+        Workspace exact{reinterpret_cast<uint8_t *>(uintptr_t(256)), total, true};
+        rc = mul_mat_multi_impl(&ctx, n, wp, fake_x, M, yp, act, nullptr, exact);
+    }
+    if (rc == QPROJ_OK && total > 0) {   // ... and one byte less must be refused, not overrun
+        Workspace less{reinterpret_cast<uint8_t *>(uintptr_t(256)), total - 1, true};
+        if (mul_mat_multi_impl(&ctx, n, wp, fake_x, M, yp, act, nullptr, less) == QPROJ_OK) rc = QPROJ_ERR_HIP;
+    }
+    set_dry_run(false);
+    if (status) *status = rc;
+    return rc == QPROJ_OK ? total : 0;
 }
 
 int qproj_rms_norm_mul_mat(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, const float *gamma_dev,
                            float eps, int64_t M, float *const *y_dev, int act) {
     const NormSpec norm{gamma_dev, eps};
-    return mul_mat_multi_impl(ctx, n, w, x_dev, M, y_dev, act, &norm);
+    Workspace wsp = ctx_workspace(ctx);
+    return mul_mat_multi_impl(ctx, n, w, x_dev, M, y_dev, act, &norm, wsp);
 }
 
 // silu(gate . x) * (up . x), optionally behind an RMS norm: one launch where the decode kernel serves
@@ -819,7 +912,8 @@ static int ffn_gate_up_impl(qproj_ctx *ctx, const qproj_weight *gate, const qpro
     if (rc) return rc;
     float *gu[2] = {reinterpret_cast<float *>(ctx->ws2), reinterpret_cast<float *>(ctx->ws2) + (size_t)M * N};
     const qproj_weight *ws[2] = {gate, up};
-    rc = mul_mat_multi_impl(ctx, 2, ws, x_dev, M, gu, act, norm);
+    Workspace wsp = ctx_workspace(ctx);
+    rc = mul_mat_multi_impl(ctx, 2, ws, x_dev, M, gu, act, norm, wsp);
     if (rc) return rc;
     QP_HIP(ctx, launch_swiglu(gu[0], gu[1], (size_t)M * N, h_dev, ctx->stream));
     return QPROJ_OK;
@@ -854,16 +948,12 @@ int qproj_mul_mat_quantized(qproj_ctx *ctx, int n, const qproj_weight *const *w,
     const int64_t K = w[0]->K;
     const ActPlanes p = act_planes(act_kind_for(kind, w[0]->type), M, K);
     const ActView a = act_view(p, static_cast<uint8_t *>(const_cast<void *>(act_dev)), K);
-    if (kind == kActGGML) {
-        int rc = ensure_ws(ctx, dense_scratch_bytes(n, w, M));
-        if (rc) return rc;
-        return run_dense_q8act(ctx, n, w, a, M, y_dev, reinterpret_cast<float *>(ctx->ws));
-    }
-    const size_t extra = per32_scratch_max(n, w, M);
+    const size_t extra = kind == kActGGML ? dense_scratch_bytes(n, w, M) : per32_scratch_max(n, w, M);
     int rc = ensure_ws(ctx, extra);
     if (rc) return rc;
-    for (int i = 0; i < n; ++i)
-        QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], extra ? reinterpret_cast<float *>(ctx->ws) : nullptr, ctx->stream));
+    const Scratch sc{extra ? reinterpret_cast<float *>(ctx->ws) : nullptr, extra};
+    if (kind == kActGGML) return run_dense_q8act(ctx, n, w, a, M, y_dev, sc);
+    for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], sc, ctx->stream));
     return QPROJ_OK;
 }
 

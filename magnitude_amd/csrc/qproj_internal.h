@@ -82,6 +82,25 @@ struct GemvArgs {
     int32_t *error_flag;
 };
 
+// Scratch memory handed to a launcher: where the partial results of a K cut into stretches (tiled kernels) or
+// chunks (small-batch kernel) go before a second small kernel adds them.  A launcher works out what its own split
+// needs from the variables that pick the split, and answers hipErrorInvalidValue instead of launching when that
+// is more than `bytes`.  {nullptr, 0}: K is never cut (the tiled kernels) / the launch is refused if it must be.
+struct Scratch {
+    float *p;
+    size_t bytes;
+};
+
+// Dry run: every launcher does its argument and capacity checks and returns without touching the device.  The
+// host-side tests walk the dispatch of whole operator calls with it (no GPU needed) to show that the scratch the
+// library reserves covers what the launchers it picks ask for.  Thread-local, off by default.
+bool dry_run();
+void set_dry_run(bool on);
+
+// Tuning knobs read from the environment exist only in builds made with -DQPROJ_TUNING (kernel-selection sweeps in
+// the lab); in the shipped library this returns `dflt` and no environment variable can change a numerics path.
+int tuning_int(const char *name, int dflt);
+
 // ---- launchers (each returns the hipError_t of the launch) ----
 hipError_t launch_dequantize(const WeightView &w, float *out, hipStream_t s);
 hipError_t launch_repack_to_planes(int type, const uint8_t *gguf, uint8_t *planes_base, const WeightView &w,
@@ -101,7 +120,7 @@ hipError_t launch_gemv_decode(const GemvArgs &args, int mt, bool fuse_quantize, 
 // results when K > 4096 (mfma_gemv_scratch_bytes, 0 if none is needed)
 bool mfma_gemv_fits(int type, int64_t M, int64_t K);
 size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, int64_t total_row_groups);
-hipError_t launch_gemv_mfma(const GemvArgs &args, float *scratch, hipStream_t s);
+hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStream_t s);
 // expert-grouped form (args.order / args.offsets); K / 256 must not exceed 16 (mfma_grouped_fits)
 bool mfma_grouped_fits(int type, int64_t K);
 hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool swiglu, hipStream_t s);
@@ -123,19 +142,19 @@ hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_exper
 hipError_t launch_moe_swiglu_gemv(const GemvArgs &gate_up, int mt, int n_experts_grid, hipStream_t s);
 hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, int64_t n_used, int64_t N,
                               float *y, hipStream_t s);
-// `scratch`: per32_scratch_bytes(K, M, N) bytes (may be null: then K is never split)
+// `scratch`: per32_scratch_bytes(K, M, N) bytes (null: K is never split)
 int per32_splits(int64_t K, int64_t M, int64_t N);
 size_t per32_scratch_bytes(int64_t K, int64_t M, int64_t N);
-hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s);
+hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s);
 // Q4_K weights x ggml Q8_K activations (`a`), large M
-// `scratch`: q8k_tile_scratch_bytes(K, M, N) bytes (may be null: then K is never split)
+// `scratch`: q8k_tile_scratch_bytes(K, M, N) bytes (null: K is never split)
 int q8k_tile_splits(int64_t K, int64_t M, int64_t N);
 size_t q8k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N);
 hipError_t launch_sum_parts(const float *part, int n_split, size_t n, float *y, hipStream_t s);
-hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s);
-hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, int64_t M, float *const *y, float *scratch,
-                                 hipStream_t s);
-hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s);
-hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, hipStream_t s);
+hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s);
+hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, int64_t M, float *const *y,
+                                 const Scratch &scratch, hipStream_t s);
+hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s);
+hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s);
 
 }  // namespace qproj

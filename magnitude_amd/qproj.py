@@ -54,6 +54,7 @@ SYMBOLS = {
     "qproj_rms_norm_quantize": (_i32, [_vp, _i32, _i32, _vp, _vp, C.c_float, _i64, _i64, _vp]),
     "qproj_mul_mat": (_i32, [_vp, _vp, _vp, _i64, _vp, _i32]),
     "qproj_mul_mat_multi": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i64, C.POINTER(_vp), _i32]),
+    "qproj_workspace_bytes": (_sz, [_i32, _i64, _i32, C.POINTER(_i64), _i64, _i32, C.POINTER(C.c_int)]),
     "qproj_mul_mat_quantized": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i32, _i64, C.POINTER(_vp)]),
     "qproj_mul_mat_id": (_i32, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _i32]),
     "qproj_moe_ffn": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i32]),
@@ -130,6 +131,17 @@ def probe_hardware() -> dict:
     n = e.n_devices if e.state == 0 else 0
     return {"runtimeApi": e.runtime_api if e.state == 0 else 0,
             "hardwareLabels": [e.hardware_labels[i].value.decode(errors="replace") for i in range(n)]}
+
+
+def workspace_bytes(qtype: int, k: int, ns: Sequence[int], m: int, act: int = ACT_GGML) -> int:
+    """Scratch bytes mul_mat_multi reserves for this shape; raises when the library's walk of its own dispatch
+    finds a launcher that the reserved scratch would not satisfy.  Needs no GPU."""
+    arr = (_i64 * len(ns))(*ns)
+    st = C.c_int(0)
+    nbytes = int(load_library().qproj_workspace_bytes(qtype, k, len(ns), arr, m, act, C.byref(st)))
+    if st.value:
+        raise QprojError(st.value, f"qproj_workspace_bytes(type {qtype}, K {k}, N {list(ns)}, M {m}, act {act})")
+    return nbytes
 
 
 def row_bytes(qtype: int, k: int) -> int:

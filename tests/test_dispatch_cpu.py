@@ -1,0 +1,69 @@
+"""The scratch the library reserves for a MUL_MAT covers what the kernel launchers it picks ask for.
+
+qproj_workspace_bytes walks the library's own dispatch (the code that serves qproj_mul_mat_multi) without
+launching: every launcher works out its demand from the variables that pick its split and refuses a buffer that is
+too small, so a sizing rule and a dispatch rule that disagree show up here, on the CPU, as a non-zero status --
+not as a write past a device buffer."""
+import itertools
+
+import pytest
+
+from magnitude_amd import qproj
+
+Q8_0, Q4_K, Q6_K = 8, 12, 14
+GGML, F32, Q8X32 = 0, 1, 2
+
+MS = [1, 2, 3, 4, 5, 8, 9, 15, 16, 17, 20, 31, 32, 33, 47, 48, 63, 64, 65, 96, 127, 128, 129, 200, 255, 256, 333, 511, 512,
+      513, 1000, 1024, 2048, 4096]
+KS = [256, 512, 768, 1024, 2048, 3072, 4096, 5120, 6144, 8192, 11008, 14336, 28672]
+NS = [(1,), (5,), (32,), (77,), (128,), (256,), (1024,), (4096,), (14336,), (4096, 1024, 1024), (14336, 14336), (768, 768),
+      (130, 5), (1024, 1024, 1024, 1024), (32000,)]
+
+
+@pytest.mark.parametrize("qtype", [Q4_K, Q6_K, Q8_0])
+def test_every_launcher_is_satisfied_by_the_reserved_scratch(qtype):
+    checked = 0
+    for m, k, ns in itertools.product(MS, KS, NS):
+        nbytes = qproj.workspace_bytes(qtype, k, ns, m, GGML)       # raises on a launcher that would be refused
+        if m <= 2:
+            assert nbytes == 0, (m, k, ns)                            # decode regime: the kernel quantizes its own rows
+        else:
+            assert nbytes >= qproj.load_library().qproj_act_bytes(GGML, qtype, m, k) > 0
+        checked += 1
+    assert checked == len(MS) * len(KS) * len(NS)
+
+
+def test_q8_0_rows_of_whole_blocks_only():
+    for m, k in itertools.product([1, 3, 16, 17, 64, 100, 512], [32, 96, 288, 1056, 4096 + 32]):
+        qproj.workspace_bytes(Q8_0, k, (77,), m, GGML)
+
+
+def test_per32_and_fp32_modes():
+    for m, k, ns in itertools.product([1, 3, 17, 64, 200, 512, 2048], [256, 4096, 14336], [(4096,), (14336,), (130,)]):
+        nbytes = qproj.workspace_bytes(Q4_K, k, ns, m, Q8X32)
+        assert nbytes >= qproj.load_library().qproj_act_bytes(Q8X32, Q4_K, m, k)
+        assert qproj.workspace_bytes(Q4_K, k, ns, m, F32) == 0
+    with pytest.raises(qproj.QprojError):
+        qproj.workspace_bytes(Q6_K, 4096, (4096,), 64, Q8X32)        # the per-32 path is built for Q4_K weights
+
+
+def test_known_sizes():
+    al = lambda v: (v + 255) // 256 * 256
+    planes = lambda m, k: al(m * k) + al(m * (k // 256) * 4) + al(m * (k // 16) * 2) + al(m * (k // 256) * 32)
+    # down projection of the 8B layer at 512 tokens: 256 tiles of 64 x 128 for 512 places on the chip, K is cut in two
+    assert qproj.workspace_bytes(Q6_K, 14336, (4096,), 512, GGML) == planes(512, 14336) + 2 * 512 * 4096 * 4
+    # gate/up at 4096 tokens: the grid is full, nothing beyond the activation planes
+    assert qproj.workspace_bytes(Q4_K, 4096, (14336, 14336), 4096, GGML) == planes(4096, 4096)
+    # small batch, K = 14336 at 16 rows: per-chunk results of the small-batch kernel
+    assert qproj.workspace_bytes(Q6_K, 14336, (4096,), 16, GGML) > planes(16, 14336)
+
+
+def test_bad_shapes_are_refused():
+    lib = qproj.load_library()
+    import ctypes as C
+    st = C.c_int(0)
+    arr = (C.c_int64 * 1)(4096)
+    assert lib.qproj_workspace_bytes(Q4_K, 4100, 1, arr, 4, GGML, C.byref(st)) == 0 and st.value == 1
+    assert lib.qproj_workspace_bytes(2, 4096, 1, arr, 4, GGML, C.byref(st)) == 0 and st.value == 1
+    assert lib.qproj_workspace_bytes(Q4_K, 4096, 5, arr, 4, GGML, C.byref(st)) == 0 and st.value == 1
+    assert lib.qproj_workspace_bytes(Q4_K, 4096, 1, None, 4, GGML, None) == 0
