@@ -152,6 +152,20 @@ int qproj_mul_mat(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int
 int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev,
                         int64_t M, float *const *y_dev, int act);
 
+/* qproj_mul_mat_multi for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (ggml's backends allocate their
+ * compute buffers up front through the graph allocator); it exists for those callers.  Same arguments, same
+ * kernels and bit-identical results, but the call's scratch -- the quantized activation planes and the partial
+ * results of a K cut into stretches or chunks -- lives in one fixed buffer of QPROJ_NOALLOC_SCRATCH_BYTES inside
+ * the library (one copy per GPU, held until the process ends) instead of the context's growable workspace, and the
+ * call issues no hipMalloc / hipFree.  A call that needs more answers QPROJ_ERR_INVALID_ARG and launches nothing
+ * (qproj_workspace_bytes tells the need beforehand; M <= 2 needs none; the 8B-class shapes fit up to M = 512).
+ * All contexts on one GPU share that buffer, which keeps the last call's contents (every byte a kernel reads
+ * was written earlier in the same call): calls that overlap in time on one GPU race. */
+#define QPROJ_NOALLOC_SCRATCH_BYTES (64u << 20)
+int qproj_mul_mat_multi_noalloc(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev,
+                                int64_t M, float *const *y_dev, int act);
+
 /* Scratch bytes qproj_mul_mat_multi reserves for n tensors of `type` with rows N[0..n) sharing K, M activation
  * rows and activation mode `act` (0 for the decode regime, which needs none).  Needs no device: it walks the
  * library's own dispatch for that shape without launching, and checks on the way that every kernel launcher it

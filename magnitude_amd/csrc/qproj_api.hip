@@ -32,6 +32,17 @@ int tuning_int(const char *name, int dflt) {
 }
 }  // namespace qproj
 
+// Scratch of the allocation-free entry point (qproj_mul_mat_multi_noalloc): quantized activation planes and the
+// partial results of a K cut into stretches or chunks.  One copy per GPU the library runs on, held until the
+// process ends; its device address is looked up once per device in qproj_ctx_create (the name below is a host-side
+// stand-in, never a device address).
+static __device__ __align__(256) unsigned char scratch[QPROJ_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+uint8_t *g_noalloc_ptr[kMaxDevices] = {};   // device address of `scratch` on each device, null until looked up
+}  // namespace
+
 struct qproj_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -98,7 +109,7 @@ int ensure_ws(qproj_ctx *ctx, size_t bytes) {
 }
 
 // Where an operator call keeps its scratch: the context's growable buffer (reserve may allocate), or a fixed
-// buffer that is never grown.
+// buffer that is never grown (the allocation-free entry point).
 struct Workspace {
     uint8_t *base;
     size_t cap;
@@ -566,6 +577,17 @@ int qproj_ctx_create(int device, void *stream, qproj_ctx **out) {
         }
         ctx->own_stream = true;
     }
+    // the fixed scratch of the allocation-free entry point: each device holds its own copy at its own address
+    if (device < kMaxDevices && !g_noalloc_ptr[device]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+            (void)hipGetLastError();
+            if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
+            delete ctx;
+            return QPROJ_ERR_HIP;
+        }
+        g_noalloc_ptr[device] = static_cast<uint8_t *>(ptr);
+    }
     if (hipMalloc((void **)&ctx->flag_dev, 256) != hipSuccess ||
         hipMemsetAsync(ctx->flag_dev, 0, 256, ctx->stream) != hipSuccess ||
         hipStreamSynchronize(ctx->stream) != hipSuccess) {
@@ -829,6 +851,15 @@ static Workspace ctx_workspace(qproj_ctx *ctx) { return Workspace{ctx ? ctx->ws 
 int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
                         float *const *y_dev, int act) {
     Workspace wsp = ctx_workspace(ctx);
+    return mul_mat_multi_impl(ctx, n, w, x_dev, M, y_dev, act, nullptr, wsp);
+}
+
+int qproj_mul_mat_multi_noalloc(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
+                                float *const *y_dev, int act) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (ctx->device < 0 || ctx->device >= kMaxDevices || !g_noalloc_ptr[ctx->device])
+        return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat_multi_noalloc: the fixed scratch was not set up for this device");
+    Workspace wsp{g_noalloc_ptr[ctx->device], (size_t)QPROJ_NOALLOC_SCRATCH_BYTES, true};
     return mul_mat_multi_impl(ctx, n, w, x_dev, M, y_dev, act, nullptr, wsp);
 }
 

@@ -54,6 +54,7 @@ SYMBOLS = {
     "qproj_rms_norm_quantize": (_i32, [_vp, _i32, _i32, _vp, _vp, C.c_float, _i64, _i64, _vp]),
     "qproj_mul_mat": (_i32, [_vp, _vp, _vp, _i64, _vp, _i32]),
     "qproj_mul_mat_multi": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i64, C.POINTER(_vp), _i32]),
+    "qproj_mul_mat_multi_noalloc": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i64, C.POINTER(_vp), _i32]),
     "qproj_workspace_bytes": (_sz, [_i32, _i64, _i32, C.POINTER(_i64), _i64, _i32, C.POINTER(C.c_int)]),
     "qproj_mul_mat_quantized": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i32, _i64, C.POINTER(_vp)]),
     "qproj_mul_mat_id": (_i32, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _i32]),
@@ -131,6 +132,9 @@ def probe_hardware() -> dict:
     n = e.n_devices if e.state == 0 else 0
     return {"runtimeApi": e.runtime_api if e.state == 0 else 0,
             "hardwareLabels": [e.hardware_labels[i].value.decode(errors="replace") for i in range(n)]}
+
+
+NOALLOC_SCRATCH_BYTES = 64 << 20
 
 
 def workspace_bytes(qtype: int, k: int, ns: Sequence[int], m: int, act: int = ACT_GGML) -> int:
@@ -292,8 +296,10 @@ class Context:
         return y
 
     def mul_mat_multi(self, ws: Sequence[Weight], x: torch.Tensor, act: int = ACT_GGML,
-                      outs: Optional[Sequence[torch.Tensor]] = None, sync: bool = True):
-        """Several MUL_MATs sharing one activation (q/k/v or gate/up) in one launch."""
+                      outs: Optional[Sequence[torch.Tensor]] = None, sync: bool = True, noalloc: bool = False):
+        """Several MUL_MATs sharing one activation (q/k/v or gate/up) in one launch.  noalloc: through the entry
+        point that keeps its scratch in the library's fixed buffer and allocates nothing (the outputs must be
+        passed in then, or they are made here before the call)."""
         x2 = x.reshape(-1, ws[0].K).contiguous()
         m = x2.shape[0]
         ys = list(outs) if outs is not None else [
@@ -303,7 +309,8 @@ class Context:
         ya = (_vp * n)(*[_ptr(y) for y in ys])
         if sync:
             torch.cuda.current_stream().synchronize()
-        self._check(self.lib.qproj_mul_mat_multi(self.handle, n, wa, _ptr(x2), m, ya, act))
+        fn = self.lib.qproj_mul_mat_multi_noalloc if noalloc else self.lib.qproj_mul_mat_multi
+        self._check(fn(self.handle, n, wa, _ptr(x2), m, ya, act))
         if sync:
             self.sync()
         return ys

@@ -67,3 +67,14 @@ def test_bad_shapes_are_refused():
     assert lib.qproj_workspace_bytes(2, 4096, 1, arr, 4, GGML, C.byref(st)) == 0 and st.value == 1
     assert lib.qproj_workspace_bytes(Q4_K, 4096, 5, arr, 4, GGML, C.byref(st)) == 0 and st.value == 1
     assert lib.qproj_workspace_bytes(Q4_K, 4096, 1, None, 4, GGML, None) == 0
+
+
+def test_the_8b_layer_fits_the_fixed_scratch_up_to_512_tokens():
+    """The allocation-free entry point keeps its scratch in a fixed 64 MiB buffer: every projection group of the
+    8B-class layer must fit for the batches the engine issues (n_batch 512,
+    /root/reference/inference/crates/icn-engine/src/lib.rs:93-96)."""
+    groups = [(Q4_K, 4096, (4096, 1024, 1024)), (Q4_K, 4096, (4096,)), (Q4_K, 4096, (14336, 14336)), (Q6_K, 14336, (4096,))]
+    for m in (1, 2, 4, 8, 16, 64, 128, 512):
+        for qt, k, ns in groups:
+            assert qproj.workspace_bytes(qt, k, ns, m, GGML) <= qproj.NOALLOC_SCRATCH_BYTES, (m, qt, k, ns)
+    assert qproj.workspace_bytes(Q6_K, 14336, (4096,), 4096, GGML) > qproj.NOALLOC_SCRATCH_BYTES   # and larger ones are refused
