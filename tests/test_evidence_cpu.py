@@ -69,3 +69,92 @@ def test_llama_bench_record_has_the_probe_result_shape():
         evidence.llama_bench_record("llama-bench.prompt-processing", 512, 1, 0, 0, [0.0], {}, [])  # zero duration
     with pytest.raises(ValueError):
         evidence.llama_bench_record("decode", 1, 1, 0, 0, [1.0], {}, [])
+
+
+# ---------------------------------------------------------------- against the reference-held sample row
+
+def _decode_backend_ops_sql(text):
+    """The reference decoder's rules for `test-backend-ops perf --output sql` rows, restated
+    (icn-parity/src/decode.rs:542-640 and the value parser at :731-762): lines starting with the INSERT prefix,
+    values single-quoted with '' as the escape, exactly 16 of them in the pinned field order, test_mode perf, a
+    resolved tool / backend identity, booleans as 1/0/true/false, numeric fields that parse, and a supported row
+    with passed, a finite positive time and n_runs > 0."""
+    import math
+    rows = []
+    for line in text.splitlines():
+        if not line.startswith("INSERT INTO test_backend_ops"):
+            continue
+        before, sep, suffix = line.partition("VALUES (")
+        assert sep and suffix.endswith(");"), "malformed backend-ops SQL INSERT"
+        body, values, i = suffix[:-2], [], 0
+        while True:
+            while i < len(body) and (body[i].isspace() or body[i] == ","):
+                i += 1
+            if i >= len(body):
+                break
+            assert body[i] == "'", "backend-ops SQL values must be single-quoted"
+            i += 1
+            value = ""
+            while True:
+                assert i < len(body), "unterminated backend-ops SQL value"
+                if body[i] == "'" and i + 1 < len(body) and body[i + 1] == "'":
+                    value += "'"
+                    i += 2
+                elif body[i] == "'":
+                    i += 1
+                    break
+                else:
+                    value += body[i]
+                    i += 1
+            values.append(value)
+        assert len(values) == 16
+        f = dict(zip(ev.BACKEND_OPS_FIELDS, values))
+        assert f["test_mode"] == "perf"
+        assert f["build_commit"].strip() and f["backend_name"].strip()
+        assert f["backend_name"].lower() not in ("unknown", "auto")
+        as_bool = {"1": True, "true": True, "0": False, "false": False}
+        supported, passed = as_bool[f["supported"]], as_bool[f["passed"]]
+        time_us, flops, bw = float(f["time_us"]), float(f["flops"]), float(f["bandwidth_gb_s"])
+        memory_kb, n_runs = int(f["memory_kb"]), int(f["n_runs"])
+        assert memory_kb >= 0 and n_runs >= 0 and "-" not in f["memory_kb"] + f["n_runs"]      # u64 in the reference
+        if supported:
+            assert passed and math.isfinite(time_us) and time_us > 0.0 and n_runs > 0
+        rows.append((before, f, time_us, flops, bw))
+    assert rows, "backend-ops SQL contains no result rows"
+    return rows
+
+
+def _golden_row():
+    import os
+    return open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "backend_ops_row.sql")).read()
+
+
+def test_the_reference_held_sample_row_decodes():
+    (before, f, time_us, flops, bw), = _decode_backend_ops_sql(_golden_row())
+    assert f["op_name"] == "SOFT_MAX" and f["backend_name"] == "MTL0" and f["build_commit"] == "9e3b928fd"
+    assert (time_us, flops, bw) == (222.961055, 0.0, 2.737648)
+    assert f["device_description"] == "" and f["backend_reg_name"] == ""
+
+
+def test_emitted_rows_have_the_sample_rows_column_list_quoting_and_value_syntax():
+    golden = _golden_row().strip()
+    g_before, g_f, *_ = _decode_backend_ops_sql(golden)[0]
+    rows = [ev.backend_ops_row("MUL_MAT", ev.mul_mat_params(12, 28672, 1, 4096), [14.6, 14.7, 14.9], flops=2.0 * 28672 * 4096,
+                               bytes_moved=66_191_360, memory_kb=64640, device="AMD Instinct MI355X"),
+            ev.backend_ops_row("MUL_MAT_ID", ev.mul_mat_id_params(12, 768, 2048, 128, 8, 64), [114.0], flops=1.0,
+                               bytes_moved=334e6, memory_kb=326000, device="it's a 'quoted' name")]
+    text = "\n".join(ev.backend_ops_sql(r) for r in rows)
+    decoded = _decode_backend_ops_sql(text)
+    assert len(decoded) == 2
+    for (before, f, time_us, flops, bw), row in zip(decoded, rows):
+        assert before == g_before                                   # the statement up to VALUES, byte for byte
+        assert list(f) == list(g_f) == list(ev.BACKEND_OPS_FIELDS)
+        assert f["device_description"] == row["device_description"]  # the '' escape round-trips
+        # the same value syntax as the sample: fixed notation with six decimals, integers bare, booleans 1/0
+        for key in ("time_us", "flops", "bandwidth_gb_s"):
+            assert re.fullmatch(r"\d+\.\d{6}", f[key]) and re.fullmatch(r"\d+\.\d{6}", g_f[key])
+        for key in ("memory_kb", "n_runs"):
+            assert re.fullmatch(r"\d+", f[key]) and re.fullmatch(r"\d+", g_f[key])
+        assert f["supported"] == g_f["supported"] == "1" and f["passed"] == "1"
+        assert re.fullmatch(r"\d{4}-\d\d-\d\dT\d\d:\d\d:\d\dZ", f["test_time"]) and re.fullmatch(r"\d{4}-\d\d-\d\dT\d\d:\d\d:\d\dZ", g_f["test_time"])
+    assert text.endswith(");") and golden.endswith(");")

@@ -841,6 +841,48 @@ def test_full_size_prefill_gemm_against_device_fp64(ctx):
     err = ((y.double() - ref).abs() / ref.abs().clamp(min=1.0)).max().item()
     assert err <= 5e-5, err
 
+BENCHED_PREFILL = (   # every (mode, type, K, N) x M the benchmark's prefill leg times (config 4 and the layer's other formats)
+    [("q8x32", Q4_K, k, n) for (k, n) in ((4096, 14336), (14336, 4096), (4096, 4096))] +
+    [("ggml", Q4_K, k, n) for (k, n) in ((4096, 14336), (14336, 4096), (4096, 4096))] +
+    [("ggml", Q6_K, 14336, 4096), ("ggml", Q8_0, 4096, 4096)])
+
+
+@pytest.mark.parametrize("m", [512, 2048, 4096])
+@pytest.mark.parametrize("mode,qtype,k,n", BENCHED_PREFILL)
+def test_every_benchmarked_prefill_shape_against_device_fp64(ctx, mode, qtype, k, n, m):
+    """Config 4's whole grid (M in {512, 2048, 4096} x the three K x N shapes, per-32 and ggml activation formats)
+    plus the Q6_K down projection and the Q8_0 matrix at the same M, on the dispatch path the benchmark times
+    (quantize, then qproj_mul_mat_quantized: wide tiles, 64-token tiles, K cut into stretches where the grid is
+    small).  Reference: fp64 product, on the device, of the dequantized weights and the dequantized quantized
+    activations, both of which are proven bit-exact against the oracle at small sizes; outlier channels as in
+    config 4."""
+    from magnitude_amd import ACT_GGML, ACT_Q8X32, synth
+    act = ACT_Q8X32 if mode == "q8x32" else ACT_GGML
+    blocks = synth.random_weight(qtype, n, k, seed=77 + n + qtype, device="cuda")
+    w = ctx.upload_from_device(qtype, k, n, blocks)
+    del blocks
+    g = torch.Generator(device="cuda").manual_seed(m + k + n)
+    x = torch.randn((m, k), generator=g, device="cuda", dtype=torch.float32)
+    x[:, torch.randperm(k, generator=g, device="cuda")[: k // 100]] *= 20.0
+    print(f"prefill parity {mode} type {qtype} M {m} K {k} N {n}", flush=True)
+    qb = ctx.quantize_activations_raw(x, act, qtype)
+    y = torch.empty((m, n), device="cuda")
+    ctx.mul_mat_quantized([w], qb, act, m, [y])
+    a = ctx.quantize_activations(x, act, qtype)
+    blk = 256 if (mode == "ggml" and qtype != Q8_0) else 32
+    xq = (a["qs"].double().view(m, k // blk, blk) * a["d"].double()[:, :, None]).view(m, k)
+    del a, qb, x
+    wd = ctx.dequantize(w).double()
+    worst = 0.0
+    for m0 in range(0, m, 1024):                    # the fp64 reference 1024 tokens at a time
+        ref = xq[m0:m0 + 1024] @ wd.T
+        worst = max(worst, ((y[m0:m0 + 1024].double() - ref).abs() / ref.abs().clamp(min=1.0)).max().item())
+        del ref
+    w.free()
+    del wd, xq
+    torch.cuda.empty_cache()
+    assert worst <= 5e-5, worst
+
 
 # ---------------------------------------------------------------- GGUF file -> library
 
