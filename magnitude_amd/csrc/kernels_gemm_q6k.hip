@@ -2,24 +2,27 @@
 //
 //   y[m][n] = sum_sb d_n * dx_m * sum_{s<16} sc_{n,s} * sum_{k in s} (q_k - 32) * a_k
 //
-// A Q6_K sub-block is 16 weights with a signed 8-bit scale: sc*q does not fit an int8 operand in
-// any two-way split, so each sub-block gets one v_mfma_i32_32x32x16_i8 on the raw 6-bit codes
-// (0..63) and the vector ALU multiplies the 16 results of a lane by the lane's scale into an
-// int32 sum that lives for the whole super-block (one mad per output and sub-block).  The -32 of
-// every code is taken out exactly with the activation block sums the quantizer already wrote:
-// sum_s sc_s * bsum_s is a K=16 product per super-block, run as two more matrix instructions with
-// the 12-bit sums split into a signed high byte and a 6-bit low byte (bsum = 64*hi + lo).  The
-// vector ALU touches floating point once per 256 weights.
+// A Q6_K sub-block is 16 weights with a signed 8-bit scale.  The scale does not split into parts that stay
+// int8 after the multiply, but the PRODUCT does: w = sc * (q - 32) lies in [-4096, 4064], and
+//     w = 256 * hi + lo,   lo = the low byte of w read as a signed byte, in [-128, 127],   hi = (w + 128) >> 8, in [-16, 16]
+// are two int8 operands.  Each lane converts the 128 weights of its half super-block once into both operands
+// (packed 16-bit multiply-add: w + 128 = sc * q + (128 - 32 * sc); the high bytes of that are hi, its low bytes
+// with bit 7 flipped are lo) and both chains then stay inside the matrix cores for the whole super-block:
+// eight v_mfma_i32_32x32x32_i8 per chain and 32 x 32 tile, (I_hi << 8) + I_lo is the exact integer sum that
+// ggml's vec_dot forms, and the vector ALU touches the outputs once per 256 weights.  Because both chains run
+// over the whole super-block the order of its 256 products is free: step t of lane (row l%32, half f = l/32) is
+// sub-block 8f + t, sixteen consecutive weights, against the sixteen activations at the same place.  No block
+// sums are needed: the -32 is inside the operand.
 //
-// Layout of the work is that of the Q4_K kernel for the same activations: 64 tokens x 32*NW weight
-// rows per workgroup, each wave 64 tokens x 32 rows (one weight operand feeds both token tiles);
-// each wave fetches the ql/qh/scale planes of its 32 rows with consecutive lanes on consecutive
-// 16-byte pieces and parks them in wave-private LDS strips, from which every lane picks the eight
-// bytes of its own row it needs per sub-block; LDS otherwise holds one super-block of
-// activations, double-buffered, so there is one workgroup barrier per 256 weights.
+// Layout of the work: 32*JT tokens x 32*NW weight rows per workgroup, each wave 32 rows x all tokens of the tile
+// (a converted operand feeds every token tile in turn).  Each wave fetches the ql / qh / scale planes of its 32
+// rows with consecutive lanes on consecutive 16-byte pieces and parks them in wave-private LDS strips (row
+// strides of 144 and 80 bytes: conflict-free for 16-byte reads by consecutive rows); LDS otherwise holds one
+// super-block of activations, double-buffered: one workgroup barrier per 256 weights.
 #include "qproj_device.h"
 #include "qproj_internal.h"
 #include "gemm_tiles.h"
+#include "lds_direct.h"
 
 namespace qproj {
 
@@ -31,30 +34,58 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 constexpr int LA = 256 + 16;   // activation row stride in LDS (bytes)
-constexpr int SQL = 128 + 8;   // strip row strides: conflict-free for 8-byte reads by consecutive rows
-constexpr int SQH = 64 + 8;
+constexpr int SQL = 128 + 16;  // strip row strides
+constexpr int SQH = 64 + 16;
 
 template <int NW, int JT>   // NW waves of 32 weight rows each, JT token tiles of 32
 struct Q6Smem {
-    // activations of one super-block, per token: the first eight bytes of the 16 sub-blocks, then
-    // the second eight bytes of the 16 sub-blocks (a lane's operands of two neighbouring
-    // sub-blocks are then one 16-byte read)
-    int8_t a[2][32 * JT * LA];
-    int16_t bs[2][32 * JT * 16];   // activation block sums per 16
-    float dx[2][32 * JT];
+    int8_t a[2][32 * JT * LA];   // activations of one super-block [token][256 (+16)]
+    float dx[2][32 * JT];        // activation scale of the super-block
     uint8_t ql[NW][32 * SQL];
     uint8_t qh[NW][32 * SQH];
     int8_t sc[NW][32 * 16];
 };
 
-__device__ __forceinline__ long as_i64(uint32_t lo, uint32_t hi) { return (long)(((uint64_t)hi << 32) | lo); }
+// two 16-bit lanes: x * s + c, each lane modulo 2^16
+__device__ __forceinline__ uint32_t pk_mad_u16(uint32_t x, uint32_t s, uint32_t c) {
+    uint32_t r;
+    asm("v_pk_mad_u16 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(s), "v"(c));
+    return r;
+}
+
+// The 16 + 16 weights that one 16-byte piece of ql (group gl of the half, bytes 16e .. 16e+15) holds in its low and
+// high nibbles, with the matching piece of qh, into both int8 operands.  Step t of a lane is sub-block 8f + t of its
+// half f = group g = t/2 (ql byte 32*(g%2) + l, nibble g/2, qh bits 2g and 2g+1), bytes l = 16*(t%2) .. +15; `scq`
+// holds the eight scales of the half.
+__device__ __forceinline__ void convert_pieces(const v4i &lq, const v4i &hq, const v2i &scq, int gl, int e, v4i (&cl)[8], v4i (&ch)[8]) {
+#pragma unroll
+    for (int nib = 0; nib < 2; ++nib) {
+        const int g = gl + 2 * nib, t = 2 * g + e;
+        const int s = (int)(int8_t)((uint32_t)scq[t >> 2] >> (8 * (t & 3)));
+        const uint32_t s16 = __builtin_amdgcn_perm((uint32_t)s, (uint32_t)s, 0x01000100u);
+        const int cc = 128 - 32 * s;
+        const uint32_t c16 = __builtin_amdgcn_perm((uint32_t)cc, (uint32_t)cc, 0x01000100u);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t lw = (uint32_t)lq[c], hw = (uint32_t)hq[c];
+            const uint32_t x = nib ? (lw >> 4) & 0x0f0f0f0fu : lw & 0x0f0f0f0fu;
+            const uint32_t hs = g == 0 ? hw << 4 : g == 1 ? hw << 2 : g == 2 ? hw : hw >> 2;
+            const uint32_t q = (hs & 0x30303030u) | x;                          // four codes 0..63
+            const uint32_t e0 = q & 0x00ff00ffu, e1 = (q >> 8) & 0x00ff00ffu;   // codes 0, 2 and 1, 3 in 16-bit lanes
+            const uint32_t w0 = pk_mad_u16(e0, s16, c16), w1 = pk_mad_u16(e1, s16, c16);   // sc * (q - 32) + 128
+            // low bytes (bit 7 flipped: minus 128 modulo 256) and high bytes, back in the order of the codes
+            cl[t][c] = (int)(__builtin_amdgcn_perm(w1, w0, 0x06020400u) ^ 0x80808080u);
+            ch[t][c] = (int)__builtin_amdgcn_perm(w1, w0, 0x07030501u);
+        }
+    }
+}
 
 template <int NW, int JT>
 __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightView w, const ActView a, int64_t M,
-                                                                 float *__restrict__ y, float *__restrict__ part) {
+                                                                              float *__restrict__ y, float *__restrict__ part) {
     constexpr int NT = 64 * NW, TN = 32 * NW, TM = 32 * JT;
     constexpr int PA = TM * 16 / NT;   // 16-byte activation pieces a thread moves per super-block
-    static_assert(PA >= 1 && TM * 2 <= NT, "tile does not fit the staging scheme");
+    static_assert(PA >= 1 && TM <= NT, "tile does not fit the staging scheme");
     extern __shared__ __align__(16) uint8_t smem_raw[];
     Q6Smem<NW, JT> &sm = *reinterpret_cast<Q6Smem<NW, JT> *>(smem_raw);
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -95,7 +126,7 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
     const int myrow = l32 < wrow_cap ? l32 : wrow_cap;
     const uint32_t scoff = (uint32_t)(myrow * (int)nb * 16);   // 32 pieces of scales: row l%32 (both halves store)
     const uint32_t doff = (uint32_t)(myrow * (int)nb);
-    // activations: piece id = tid + NT*p -> token id / 16, sub-block id % 16
+    // activations: piece id = tid + NT*p -> token id / 16, 16-byte segment id % 16
     const int mrow_cap = (int)(M - 1 - m0 < TM - 1 ? M - 1 - m0 : TM - 1);
     const int8_t *abase = a.qs + m0 * K;
     uint32_t aoffg[PA];
@@ -104,22 +135,17 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
     for (int p = 0; p < PA; ++p) {
         const int id = tid + NT * p, row = id >> 4, seg = id & 15;
         aoffg[p] = (uint32_t)((row < mrow_cap ? row : mrow_cap) * (int)K + 16 * seg);
-        aoffl[p] = row * LA + 8 * seg;
+        aoffl[p] = row * LA + 16 * seg;
     }
-    // block sums: TM tokens x 32 bytes, thread t (mod 2*TM) moves 16 bytes; scale: thread t (mod TM)
-    const uint8_t *bsbase = reinterpret_cast<const uint8_t *>(a.bsums) + m0 * nb * 32;
-    const int bsrow = (tid & (2 * TM - 1)) >> 1;
-    const uint32_t bsoffg = (uint32_t)((bsrow < mrow_cap ? bsrow : mrow_cap) * (int)nb * 32 + 16 * (tid & 1));
     const float *dxbase = a.d + m0 * nb;
     const uint32_t dxoffg = (uint32_t)(((tid & (TM - 1)) < mrow_cap ? (tid & (TM - 1)) : mrow_cap) * (int)nb);
 
-    v4i sql[4], sqh[2], ssc, areg[PA], bsreg;
+    v4i sql[4], sqh[2], ssc, areg[PA];
     float dxreg;
     uint32_t dcur = 0, dnext = 0;   // fp16 d of the lane's row: current super-block, next
     auto load_next = [&](int64_t sb) {   // activations first: they are wanted at the end of this trip already
 #pragma unroll
         for (int p = 0; p < PA; ++p) areg[p] = *reinterpret_cast<const v4i *>(abase + sb * 256 + aoffg[p]);
-        bsreg = *reinterpret_cast<const v4i *>(bsbase + sb * 32 + bsoffg);
         dxreg = dxbase[sb + dxoffg];
 #pragma unroll
         for (int c = 0; c < 4; ++c) sql[c] = *reinterpret_cast<const v4i *>(qlbase + sb * 128 + qloff[c]);
@@ -132,107 +158,42 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
     int8_t *psc = sm.sc[wave];
     auto store_next = [&](int buf) {
 #pragma unroll
-        for (int p = 0; p < PA; ++p) {
-            *reinterpret_cast<v2i *>(sm.a[buf] + aoffl[p]) = areg[p].xy;
-            *reinterpret_cast<v2i *>(sm.a[buf] + aoffl[p] + 128) = areg[p].zw;
-        }
-        // threads beyond the first 2*TM / TM repeat a store of the same value: no branch, no load sunk into one
-        *reinterpret_cast<v4i *>(reinterpret_cast<uint8_t *>(sm.bs[buf]) + 16 * (tid & (2 * TM - 1))) = bsreg;
+        for (int p = 0; p < PA; ++p) *reinterpret_cast<v4i *>(sm.a[buf] + aoffl[p]) = areg[p];
+        // threads beyond the first TM repeat a store of the same value: no branch, no load sunk into one
         sm.dx[buf][tid & (TM - 1)] = dxreg;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            *reinterpret_cast<v2i *>(pql + qlpark[c]) = sql[c].xy;
-            *reinterpret_cast<v2i *>(pql + qlpark[c] + 8) = sql[c].zw;
-        }
+        for (int c = 0; c < 4; ++c) *reinterpret_cast<v4i *>(pql + qlpark[c]) = sql[c];
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            *reinterpret_cast<v2i *>(pqh + qhpark[c]) = sqh[c].xy;
-            *reinterpret_cast<v2i *>(pqh + qhpark[c] + 8) = sqh[c].zw;
-        }
+        for (int c = 0; c < 2; ++c) *reinterpret_cast<v4i *>(pqh + qhpark[c]) = sqh[c];
         *reinterpret_cast<v4i *>(psc + l32 * 16) = ssc;
         dcur = dnext;
     };
 
     const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     auto superblock = [&](int buf, uint32_t dbits) {
-        const v4i scv = *reinterpret_cast<const v4i *>(psc + l32 * 16);   // the 16 scales of the lane's row
-        const int8_t *ap = sm.a[buf] + l32 * LA + 128 * lh;
-        v16i isum[JT];
-        // ---- -32 * sum_s sc_s * bsum_s: block sums as 64*hi + lo against the scales of k-half l/32
-        {
-            const long bsc = lh ? as_i64((uint32_t)scv[2], (uint32_t)scv[3]) : as_i64((uint32_t)scv[0], (uint32_t)scv[1]);
+        const v2i scq = *reinterpret_cast<const v2i *>(psc + l32 * 16 + 8 * lh);   // the eight scales of the half
+        v4i cl[8], ch[8];
 #pragma unroll
-            for (int j = 0; j < JT; ++j) {
-                const v4i b = *reinterpret_cast<const v4i *>(reinterpret_cast<const uint8_t *>(sm.bs[buf]) +
-                                                           (j * 32 + l32) * 32 + 16 * lh);
-                uint32_t lo[4], hi[4];
+        for (int e = 0; e < 2; ++e) {
+            const v4i hq = *reinterpret_cast<const v4i *>(pqh + l32 * SQH + 32 * lh + 16 * e);
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    lo[c] = (uint32_t)b[c] & 0x003f003fu;
-                    hi[c] = ((uint32_t)b[c] >> 6) & 0x00ff00ffu;   // bits 6..13 of each half: the low byte of (sum >> 6)
-                }
-                // bytes 0 and 2 of two dwords -> four bytes (v_perm_b32: selectors 0..3 second operand, 4..7 first)
-                const long alo = as_i64(__builtin_amdgcn_perm(lo[1], lo[0], 0x06040200u), __builtin_amdgcn_perm(lo[3], lo[2], 0x06040200u));
-                const long ahi = as_i64(__builtin_amdgcn_perm(hi[1], hi[0], 0x06040200u), __builtin_amdgcn_perm(hi[3], hi[2], 0x06040200u));
-                const v16i tl = __builtin_amdgcn_mfma_i32_32x32x16_i8(alo, bsc, zi, 0, 0, 0);
-                const v16i th = __builtin_amdgcn_mfma_i32_32x32x16_i8(ahi, bsc, zi, 0, 0, 0);
-#pragma unroll
-                for (int v = 0; v < 16; ++v) isum[j][v] = __mul24(th[v], -2048) + __mul24(tl[v], -32);
-            }
-        }
-        // ---- the 16 sub-blocks: j = 8f + 2k + p holds weights 128f + 32k + 16p + (0..15)
-#pragma unroll
-        for (int f = 0; f < 2; ++f) {
-            uint32_t wl[2][4], wh[2][4];
-#pragma unroll
-            for (int p = 0; p < 2; ++p) {
-                // bytes shared by the four sub-blocks k = 0..3 of (f, p): the lane's eight of each
-                const v2i qa = *reinterpret_cast<const v2i *>(pql + l32 * SQL + 64 * f + 16 * p + 8 * lh);
-                const v2i qb = *reinterpret_cast<const v2i *>(pql + l32 * SQL + 64 * f + 32 + 16 * p + 8 * lh);
-                const v2i qh = *reinterpret_cast<const v2i *>(pqh + l32 * SQH + 32 * f + 16 * p + 8 * lh);
-                const uint32_t ax = (uint32_t)qa.x, ay = (uint32_t)qa.y, bx = (uint32_t)qb.x, by = (uint32_t)qb.y;
-                const uint32_t hx = (uint32_t)qh.x, hy = (uint32_t)qh.y;
-                wl[p][0] = (ax & 0x0f0f0f0fu) | ((hx << 4) & 0x30303030u);
-                wh[p][0] = (ay & 0x0f0f0f0fu) | ((hy << 4) & 0x30303030u);
-                wl[p][1] = (bx & 0x0f0f0f0fu) | ((hx << 2) & 0x30303030u);
-                wh[p][1] = (by & 0x0f0f0f0fu) | ((hy << 2) & 0x30303030u);
-                wl[p][2] = ((ax >> 4) & 0x0f0f0f0fu) | (hx & 0x30303030u);
-                wh[p][2] = ((ay >> 4) & 0x0f0f0f0fu) | (hy & 0x30303030u);
-                wl[p][3] = ((bx >> 4) & 0x0f0f0f0fu) | ((hx >> 2) & 0x30303030u);
-                wh[p][3] = ((by >> 4) & 0x0f0f0f0fu) | ((hy >> 2) & 0x30303030u);
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int sb0 = 8 * f + 2 * k;   // sub-blocks sb0 (p = 0) and sb0 + 1 (p = 1) lie side by side in the tile
-                int s0 = (int)(int8_t)((uint32_t)scv[sb0 >> 2] >> (8 * (sb0 & 3)));
-                int s1 = (int)(int8_t)((uint32_t)scv[(sb0 + 1) >> 2] >> (8 * ((sb0 + 1) & 3)));
-                // The scales are made opaque registers on purpose: left to itself the compiler reads the byte
-                // straight out of the packed word with a sub-dword operand select, which only exists for the
-                // two-operand multiply, and then needs separate additions (1.5 instructions per product
-                // instead of one multiply-add).
-                asm volatile("" : "+v"(s0), "+v"(s1));
-#pragma unroll
-                for (int j = 0; j < JT; ++j) {
-                    const v4i av = *reinterpret_cast<const v4i *>(ap + j * 32 * LA + 8 * sb0);
-                    const v16i i0 = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64((uint32_t)av[0], (uint32_t)av[1]),
-                                                                          as_i64(wl[0][k], wh[0][k]), zi, 0, 0, 0);
-                    const v16i i1 = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64((uint32_t)av[2], (uint32_t)av[3]),
-                                                                          as_i64(wl[1][k], wh[1][k]), zi, 0, 0, 0);
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        int t = __mul24(i0[v], s0) + isum[j][v];
-                        asm("" : "+v"(t));   // keeps the multiply-adds apart (see above: otherwise mul, mul, add3)
-                        t = __mul24(i1[v], s1) + t;
-                        asm("" : "+v"(t));
-                        isum[j][v] = t;
-                    }
-                }
+            for (int gl = 0; gl < 2; ++gl) {
+                const v4i lq = *reinterpret_cast<const v4i *>(pql + l32 * SQL + 64 * lh + 32 * gl + 16 * e);
+                convert_pieces(lq, hq, scq, gl, e, cl, ch);
             }
         }
         const float dn = h2f(dbits);
+        const int8_t *ap = sm.a[buf] + l32 * LA + 128 * lh;
         const float *dxs = sm.dx[buf];
 #pragma unroll
         for (int j = 0; j < JT; ++j) {
+            v16i ilo = zi, ihi = zi;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const v4i af = *reinterpret_cast<const v4i *>(ap + j * 32 * LA + 16 * t);
+                ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, cl[t], ilo, 0, 0, 0);
+                ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, ch[t], ihi, 0, 0, 0);
+            }
             float dxv[16];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -240,7 +201,7 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
                 dxv[4 * i] = d4.x; dxv[4 * i + 1] = d4.y; dxv[4 * i + 2] = d4.z; dxv[4 * i + 3] = d4.w;
             }
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][v] = fmaf((float)isum[j][v], dxv[v] * dn, acc[j][v]);
+            for (int v = 0; v < 16; ++v) acc[j][v] = fmaf((float)((ihi[v] << 8) + ilo[v]), dxv[v] * dn, acc[j][v]);
         }
     };
 
@@ -275,6 +236,172 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q6k_q8k_kernel(const WeightVi
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------
+// The same product for large grids: 128 tokens x 256 weight rows per workgroup (eight waves, one workgroup per
+// compute unit), so a wave converts its weights once per 128 tokens.  Nothing is staged through registers:
+// activations, activation scales and the raw planes of the wave's 32 rows go from global memory straight into LDS
+// (16 bytes a lane, a wave writes a contiguous kilobyte per request).  Such a load cannot pad LDS rows, so the
+// 16-byte segments of a row are XOR-swizzled by the row index instead -- the loading lane simply asks global memory
+// for the segment that belongs in its slot: activations [token][16 slots], slot s holds segment s ^ (token % 16);
+// ql [row][8 slots], slot s holds piece s ^ (row % 8); qh [row][4 slots], slot s holds piece s ^ ((row / 2) % 4);
+// the 16 scales of a row lie as they are.
+struct Q6WideSmem {
+    int8_t a[2][128 * 256];
+    float dx[2][128];
+    uint8_t ql[8][32 * 128];
+    uint8_t qh[8][32 * 64];
+    int8_t sc[8][64 * 16];   // 32 rows; the upper half takes the duplicate pieces of lanes 32..63
+};
+
+__global__ __launch_bounds__(512, 1) void gemm_q6k_q8k_wide_kernel(const WeightView w, const ActView a, int64_t M,
+                                                                 float *__restrict__ y, float *__restrict__ part) {
+    constexpr int NW = 8, TM = 128, TN = 256, JT = 4, PA = 4;
+    extern __shared__ __align__(16) uint8_t smem_raw[];
+    Q6WideSmem &sm = *reinterpret_cast<Q6WideSmem *>(smem_raw);
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int64_t N = w.N, K = w.K, nb = w.nb;
+    int tile_n, tile_m;
+    tile_of_workgroup((int)((N + TN - 1) / TN), (int)((M + TM - 1) / TM), tile_n, tile_m);
+    const int64_t n0 = (int64_t)tile_n * TN, m0 = (int64_t)tile_m * TM;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    v16f acc[JT];
+#pragma unroll
+    for (int j = 0; j < JT; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+
+    // ---- global -> LDS requests: wave-uniform bases plus 32-bit lane offsets; rows past the edge of the matrix
+    // repeat its last valid row (computed, never stored)
+    const int64_t wave_row0 = n0 + wave * 32 < N ? n0 + wave * 32 : N - 1;
+    const int wrow_cap = (int)(N - 1 - wave_row0 < 31 ? N - 1 - wave_row0 : 31);
+    const uint8_t *qlbase = scalar_pointer(w.q6_ql + wave_row0 * nb * 128);
+    const uint8_t *qhbase = scalar_pointer(w.q6_qh + wave_row0 * nb * 64);
+    const uint8_t *scbase = scalar_pointer(reinterpret_cast<const uint8_t *>(w.q6_sc) + wave_row0 * nb * 16);
+    const uint16_t *dbase = scalar_pointer(w.q6_d + wave_row0 * nb);
+    uint32_t qloff[4], qhoff[2];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {   // slot p = lane + 64*c of the wave's 256: row p / 8, slot p % 8
+        const int p = lane + 64 * c, row = p >> 3, r = row < wrow_cap ? row : wrow_cap;
+        qloff[c] = (uint32_t)(r * (int)nb * 128 + 16 * ((p & 7) ^ (row & 7)));
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {   // slot p of 128: row p / 4, slot p % 4
+        const int p = lane + 64 * c, row = p >> 2, r = row < wrow_cap ? row : wrow_cap;
+        qhoff[c] = (uint32_t)(r * (int)nb * 64 + 16 * ((p & 3) ^ ((row >> 1) & 3)));
+    }
+    const int myrow = l32 < wrow_cap ? l32 : wrow_cap;
+    const uint32_t scoff = (uint32_t)(myrow * (int)nb * 16);
+    const uint32_t doff = (uint32_t)(myrow * (int)nb);
+    const int mrow_cap = (int)(M - 1 - m0 < TM - 1 ? M - 1 - m0 : TM - 1);
+    const int8_t *abase = scalar_pointer(a.qs + m0 * K);
+    uint32_t aoffg[PA];   // chunk wave + NW*p = tokens 4*chunk .. +3; lane -> token lane/16, slot lane%16
+#pragma unroll
+    for (int p = 0; p < PA; ++p) {
+        const int row = 4 * (wave + NW * p) + (lane >> 4), seg = (lane & 15) ^ (row & 15);
+        aoffg[p] = (uint32_t)((row < mrow_cap ? row : mrow_cap) * (int)K + 16 * seg);
+    }
+    const float *dxbase = scalar_pointer(a.d + m0 * nb);
+    const int dxtok = tid & 127;
+    const uint32_t dxoffg = (uint32_t)((dxtok < mrow_cap ? dxtok : mrow_cap) * (int)nb);
+    uint8_t *pql = sm.ql[wave], *pqh = sm.qh[wave];
+    int8_t *psc = sm.sc[wave];
+
+    auto request_strip = [&](uint32_t sb) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) global_to_lds16(qlbase + (qloff[c] + sb * 128u), pql + 1024 * c);
+#pragma unroll
+        for (int c = 0; c < 2; ++c) global_to_lds16(qhbase + (qhoff[c] + sb * 64u), pqh + 1024 * c);
+        global_to_lds16(scbase + (scoff + sb * 16u), psc);
+    };
+    auto request_act = [&](uint32_t sb, int buf, int p) {
+        global_to_lds16(abase + (aoffg[p] + sb * 256u), sm.a[buf] + (wave + NW * p) * 1024);
+    };
+    // the lane's reads: ql piece q8 = 4f + 2gl + e of row l%32 sits in slot q8 ^ (l%8); qh piece 2f + e in slot
+    // (2f + e) ^ ((l%32 / 2) % 4); activation segment 8f + t of token l%32 (+32j) in slot (8f + t) ^ (l%16)
+    const int qlrow = l32 * 128, qhrow = l32 * 64;
+    const int qlx = l32 & 7, qhx = (l32 >> 1) & 3;
+    const int aoffl = l32 * 256 + 16 * ((8 * lh) ^ (l32 & 15));
+    const v16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+
+    // a grid with gridDim.y > 1 cuts K: this workgroup does the super-blocks [sb_begin, sb_end) and writes a
+    // partial tile; the partial tiles are added in order afterwards
+    const int64_t sb_begin = nb * blockIdx.y / gridDim.y, sb_end = nb * (blockIdx.y + 1) / gridDim.y;
+    // ---- prologue: requests of the first super-block
+    request_strip((uint32_t)sb_begin);
+#pragma unroll
+    for (int p = 0; p < PA; ++p) request_act((uint32_t)sb_begin, 0, p);
+    sm.dx[0][dxtok] = dxbase[dxoffg + (uint32_t)sb_begin];
+    uint32_t dcur = dbase[doff + (uint32_t)sb_begin];
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    for (int64_t sb = sb_begin; sb < sb_end; ++sb) {
+        const int buf = (int)((sb - sb_begin) & 1);
+        const uint32_t sb_next = (uint32_t)(sb + 1 < sb_end ? sb + 1 : sb_end - 1);   // past the end: requested again, never used
+        // ---- the lane's 128 weights into both int8 operands, out of the strip
+        v4i cl[8], ch[8];
+        {
+            const v2i scq = *reinterpret_cast<const v2i *>(psc + l32 * 16 + 8 * lh);
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const v4i hq = *reinterpret_cast<const v4i *>(pqh + qhrow + 16 * ((2 * lh + e) ^ qhx));
+#pragma unroll
+                for (int gl = 0; gl < 2; ++gl) {
+                    const v4i lq = *reinterpret_cast<const v4i *>(pql + qlrow + 16 * ((4 * lh + 2 * gl + e) ^ qlx));
+                    convert_pieces(lq, hq, scq, gl, e, cl, ch);
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the strip has been read: it may be overwritten
+        __builtin_amdgcn_sched_barrier(0);
+        request_strip(sb_next);
+        const float dn = h2f(dcur);
+        const uint32_t dnext = dbase[doff + sb_next];
+        const float dxreg = dxbase[dxoffg + sb_next];
+        const int8_t *ab = sm.a[buf];
+        const float *dxs = sm.dx[buf];
+#pragma unroll
+        for (int j = 0; j < JT; ++j) {
+            v16i ilo = zi, ihi = zi;
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                const v4i af = *reinterpret_cast<const v4i *>(ab + j * 32 * 256 + (aoffl ^ (16 * t)));
+                ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, cl[t], ilo, 0, 0, 0);
+                ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, ch[t], ihi, 0, 0, 0);
+            }
+            if (j == 1) {   // the next super-block's activations, once the strip requests are under way
+#pragma unroll
+                for (int p = 0; p < PA; ++p) request_act(sb_next, buf ^ 1, p);
+            }
+            float dxv[16];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float4 d4 = *reinterpret_cast<const float4 *>(dxs + j * 32 + 8 * i + 4 * lh);
+                dxv[4 * i] = d4.x; dxv[4 * i + 1] = d4.y; dxv[4 * i + 2] = d4.z; dxv[4 * i + 3] = d4.w;
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][v] = fmaf((float)((ihi[v] << 8) + ilo[v]), dxv[v] * dn, acc[j][v]);
+        }
+        sm.dx[buf ^ 1][dxtok] = dxreg;   // every thread stores (a repeated value past 128): no branch
+        dcur = dnext;
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
+
+    // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
+    const int64_t n = n0 + wave * 32 + l32;
+    float *out = gridDim.y > 1 ? part + (size_t)blockIdx.y * M * N : y;
+#pragma unroll
+    for (int j = 0; j < JT; ++j) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (m < M && n < N) out[m * N + n] = acc[j][v];
+        }
+    }
+}
 }  // namespace
 
 namespace {
@@ -293,16 +420,50 @@ hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y
 }
 }  // namespace
 
+// Which kernel and how many stretches of K.  The 128-token kernel (256 weight rows a workgroup, one workgroup per
+// compute unit) wants about 192 workgroups or more: a grid of 96..191 such tiles is doubled by cutting K in two, one of
+// 48..95 quadrupled, never under twelve super-blocks a stretch.  Smaller grids take 64-token tiles (128 rows, two
+// workgroups per compute unit) with the stretches of q8k_tile_splits, or 32-token tiles where K is too short for that.
+namespace {
+struct Q6Plan {
+    bool wide;
+    int n_split;
+};
+Q6Plan q6k_plan(int64_t K, int64_t M, int64_t N, bool have_scratch) {
+    const int64_t wide_tiles = ((N + 255) / 256) * ((M + 127) / 128);
+    if (wide_tiles >= 192) return {true, 1};
+    if (have_scratch && (M * N) % 4 == 0 && wide_tiles >= 48) {
+        int n = wide_tiles >= 96 ? 2 : 4;
+        while (n > 1 && K / 256 < 12 * n) n >>= 1;
+        if (n > 1) return {true, n};
+    }
+    return {false, have_scratch ? q8k_tile_splits(K, M, N) : 1};
+}
+}  // namespace
+
+size_t q6k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N) {
+    const Q6Plan p = q6k_plan(K, M, N, true);
+    return p.n_split > 1 ? (size_t)p.n_split * M * N * 4 : 0;
+}
+
 // ggml-format activations (Q8_K planes in `a`), Q6_K weights, any M
 hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s) {
-    if (w.type != kTypeQ6_K || a.kind != kActKindQ8_K || !a.bsums || M <= 0) return hipErrorInvalidValue;
-    if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 64 token rows of K bytes, 32 weight rows of K/2
-    // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit.  A grid of such tiles that
-    // would leave compute units idle is filled by cutting K into stretches (partial tiles added afterwards);
-    // where K is too short for that, 32-token tiles double the number of workgroups instead.
-    const int n_split = scratch.p ? q8k_tile_splits(w.K, M, w.N) : 1;
-    if (n_split > 1 && (size_t)n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
-    if (n_split > 1 || ((w.N + 127) / 128) * ((M + 63) / 64) >= 384) return launch_q6k<4, 2>(w, a, M, y, scratch.p, n_split, s);
+    if (w.type != kTypeQ6_K || a.kind != kActKindQ8_K || M <= 0) return hipErrorInvalidValue;
+    if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 128 token rows of K bytes, 32 weight rows of K/2
+    const Q6Plan p = q6k_plan(w.K, M, w.N, scratch.p != nullptr);
+    if (p.n_split > 1 && (size_t)p.n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
+    if (p.wide) {
+        if (dry_run()) return hipSuccess;
+        static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q6k_q8k_wide_kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Q6WideSmem));
+        if (attr != hipSuccess) return attr;
+        const int64_t wide_tiles = ((w.N + 255) / 256) * ((M + 127) / 128);
+        hipLaunchKernelGGL(gemm_q6k_q8k_wide_kernel, dim3((unsigned)wide_tiles, (unsigned)p.n_split), dim3(512), sizeof(Q6WideSmem),
+                           s, w, a, M, y, scratch.p);
+        if (p.n_split > 1) return launch_sum_parts(scratch.p, p.n_split, (size_t)M * w.N, y, s);
+        return hipGetLastError();
+    }
+    if (p.n_split > 1 || ((w.N + 127) / 128) * ((M + 63) / 64) >= 384) return launch_q6k<4, 2>(w, a, M, y, scratch.p, p.n_split, s);
     return launch_q6k<4, 1>(w, a, M, y, nullptr, 1, s);
 }
 

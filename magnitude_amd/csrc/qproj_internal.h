@@ -155,6 +155,7 @@ hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, flo
 hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, int64_t M, float *const *y,
                                  const Scratch &scratch, hipStream_t s);
 hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s);
+size_t q6k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N);   // what launch_gemm_q6k_q8k asks of its scratch
 hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s);
 
 }  // namespace qproj
