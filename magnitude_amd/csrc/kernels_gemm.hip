@@ -590,7 +590,7 @@ struct WideSmem {
 
 template <int NW>
 __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const WeightView w, const ActView a, int64_t M,
-                                                                      float *__restrict__ y) {
+                                                                      float *__restrict__ y, float *__restrict__ part) {
     static_assert(NW == 8, "the loading roles below are laid out for eight waves");
     constexpr int TM = 128, TN = 32 * NW, JT = TM / 32;
     constexpr int PA = (TM * 16) / (64 * NW);   // 1-KB activation chunks (4 tokens) a wave requests per super-block
@@ -682,13 +682,16 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
         }
     };
 
-    // ---- prologue: requests of super-block 0
+    // a grid with gridDim.y > 1 cuts K: this workgroup does the super-blocks [sb_begin, sb_end) and writes a
+    // partial tile that sum_parts_kernel adds to the others in order
+    const int64_t sb_begin = nb * blockIdx.y / gridDim.y, sb_end = nb * (blockIdx.y + 1) / gridDim.y;
+    // ---- prologue: requests of the first super-block
 #pragma unroll
-    for (int c = 0; c < 5; ++c) request_strip(0, c);
+    for (int c = 0; c < 5; ++c) request_strip((uint32_t)sb_begin, c);
 #pragma unroll
-    for (int p = 0; p < PA; ++p) request_act(0, 0, p);
-    request_ms(0, 0);
-    sm.dx[0][tid & 127] = dxbase_s[dxoffg];
+    for (int p = 0; p < PA; ++p) request_act((uint32_t)sb_begin, 0, p);
+    request_ms((uint32_t)sb_begin, 0);
+    sm.dx[0][tid & 127] = dxbase_s[dxoffg + (uint32_t)sb_begin];
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
@@ -707,15 +710,15 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
     // the memory pipeline.
     auto run = [&](auto late_tag) {
         constexpr bool LATE = decltype(late_tag)::value;
-        if (LATE) {   // weights of super-block 0, with nothing to overlap
+        if (LATE) {   // weights of the first super-block, with nothing to overlap
             read_header();
 #pragma unroll
             for (int t = 0; t < 8; ++t) convert(t, strip_piece(t));
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the strip is about to be overwritten
         }
-        for (int64_t sb = 0; sb < nb; ++sb) {
-            const int buf = (int)(sb & 1);
-            const uint32_t sb_next = (uint32_t)(sb + 1 < nb ? sb + 1 : nb - 1);   // past the end: requested again, never used
+        for (int64_t sb = sb_begin; sb < sb_end; ++sb) {
+            const int buf = (int)((sb - sb_begin) & 1);
+            const uint32_t sb_next = (uint32_t)(sb + 1 < sb_end ? sb + 1 : sb_end - 1);   // past the end: requested again, never used
             v4i raw[4];
             if (!LATE) {   // out of the strip: header of row l%32, then the lane's 64 nibble bytes
                 read_header();
@@ -804,12 +807,13 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
     const int64_t n = n0 + wave * 32 + l32;
     const float inv = 1.0f / kMinPrescale;
+    float *out = gridDim.y > 1 ? part + (size_t)blockIdx.y * M * N : y;
 #pragma unroll
     for (int j = 0; j < JT; ++j) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < M && n < N) y[m * N + n] = acc[j][v] * inv;
+            if (m < M && n < N) out[m * N + n] = acc[j][v] * inv;
         }
     }
 }
@@ -902,38 +906,63 @@ hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, fl
     return launch_per32<kTypeQ8_0>(w, a, M, y, scratch, s);
 }
 
+// Which Q4_K kernel and how many stretches of K (one rule for the launcher and for the scratch sizing).  The
+// 128-token kernel (256 weight rows a workgroup, one workgroup per compute unit) wants about 192 workgroups or more:
+// a grid of 96..191 such tiles is doubled by cutting K in two, one of 48..95 quadrupled, never under twelve
+// super-blocks a stretch.  Everything else takes 64-token tiles with the stretches of q8k_tile_splits.
+namespace {
+struct Q4Plan {
+    bool wide;
+    int n_split;
+};
+Q4Plan q4k_plan(int64_t K, int64_t M, int64_t N, bool have_scratch) {
+    static const int wide_env = tuning_int("QPROJ_Q8K_WIDE", -1);
+    const int64_t wide_tiles = ((N + 255) / 256) * ((M + 127) / 128);
+    if (wide_env >= 0 ? wide_env != 0 : wide_tiles >= 192) return {true, 1};
+    if (wide_env < 0 && have_scratch && (M * N) % 4 == 0 && wide_tiles >= 48) {
+        int n = wide_tiles >= 96 ? 2 : 4;
+        while (n > 1 && K / 256 < 12 * n) n >>= 1;
+        if (n > 1) return {true, n};
+    }
+    return {false, have_scratch ? q8k_tile_splits(K, M, N) : 1};
+}
+}  // namespace
+
+size_t q4k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N) {
+    const Q4Plan p = q4k_plan(K, M, N, true);
+    return p.n_split > 1 ? (size_t)p.n_split * M * N * 4 : 0;
+}
+
 // ggml-format activations (Q8_K planes in `a`, including the min-term plane), Q4_K weights, any M
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s) {
     if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || !a.msum || M <= 0) return hipErrorInvalidValue;
-    if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 64 token rows of K bytes, 32 weight rows of K*144/256
-    // large batches: 128 tokens x 256 weight rows per workgroup, one workgroup per compute unit
-    static const int wide_env = tuning_int("QPROJ_Q8K_WIDE", -1);
-    const int64_t wide_tiles = ((w.N + 255) / 256) * ((M + 127) / 128);
-    if (wide_env >= 0 ? wide_env != 0 : wide_tiles >= 192) {
-        if (dry_run()) return hipSuccess;
+    if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 128 token rows of K bytes, 32 weight rows of K*144/256
+    const Q4Plan p = q4k_plan(w.K, M, w.N, scratch.p != nullptr);
+    if (p.n_split > 1 && (size_t)p.n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
+    if (dry_run()) return hipSuccess;
+    if (p.wide) {   // 128 tokens x 256 weight rows per workgroup, one workgroup per compute unit
         using Smem = WideSmem<8>;
         const auto kern = &gemm_q4k_q8k_wide_kernel<8>;
         static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
         if (attr != hipSuccess) return attr;
-        hipLaunchKernelGGL(kern, dim3((unsigned)wide_tiles), dim3(512), sizeof(Smem), s, w, a, M, y);
+        const int64_t wide_tiles = ((w.N + 255) / 256) * ((M + 127) / 128);
+        hipLaunchKernelGGL(kern, dim3((unsigned)wide_tiles, (unsigned)p.n_split), dim3(512), sizeof(Smem), s, w, a, M, y, scratch.p);
+        if (p.n_split > 1) return launch_sum_parts(scratch.p, p.n_split, (size_t)M * w.N, y, s);
         return hipGetLastError();
     }
     constexpr int NW = 4;   // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit
     using Smem = DirectSmem<NW>;
-    const int n_split = scratch.p ? q8k_tile_splits(w.K, M, w.N) : 1;
-    if (n_split > 1 && (size_t)n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
-    if (dry_run()) return hipSuccess;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_direct_kernel<NW>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
     if (attr != hipSuccess) return attr;
-    const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64)), (unsigned)n_split);
+    const dim3 grid((unsigned)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64)), (unsigned)p.n_split);
     DirectTargets tg{};
     tg.n = 1;
     tg.w[0] = w;
     tg.y[0] = y;
     hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, tg, a, M, scratch.p);
-    if (n_split > 1) return launch_sum_parts(scratch.p, n_split, (size_t)M * w.N, y, s);
+    if (p.n_split > 1) return launch_sum_parts(scratch.p, p.n_split, (size_t)M * w.N, y, s);
     return hipGetLastError();
 }
 
@@ -949,10 +978,9 @@ hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, i
     const bool can = !off && n >= 2 && n <= 3 && wide_env < 0 && a.kind == kActKindQ8_K && a.msum && M > 0;
     int joined[3], n_joined = 0;
     for (int i = 0; i < n; ++i) {
-        const int64_t wide_tiles = ((w[i].N + 255) / 256) * ((M + 127) / 128);
-        const bool fits = can && w[i].type == kTypeQ4_K && w[i].K == w[0].K && w[i].K <= (1 << 24) && wide_tiles < 192 &&
-                          (!scratch.p || q8k_tile_splits(w[i].K, M, w[i].N) == 1 ||
-                           ((w[i].N + 127) / 128) * ((M + 63) / 64) < 96);   // small ones are better off together than cut
+        const Q4Plan p = q4k_plan(w[i].K, M, w[i].N, scratch.p != nullptr);
+        const bool fits = can && w[i].type == kTypeQ4_K && w[i].K == w[0].K && w[i].K <= (1 << 24) && !p.wide &&
+                          (p.n_split == 1 || ((w[i].N + 127) / 128) * ((M + 63) / 64) < 96);   // small ones are better off together than cut
         if (fits) joined[n_joined++] = i;
     }
     if (n_joined < 2) n_joined = 0;

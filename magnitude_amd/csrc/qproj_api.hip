@@ -356,7 +356,7 @@ size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
     if (M > 16 && w[0]->type != kTypeQ8_0)   // tiled Q4_K / Q6_K products with K cut into stretches
         for (int i = 0; i < n; ++i)
             need = std::max(need, w[0]->type == kTypeQ6_K ? q6k_tile_scratch_bytes(w[i]->K, M, w[i]->N)
-                                                          : q8k_tile_scratch_bytes(w[i]->K, M, w[i]->N));
+                                                          : q4k_tile_scratch_bytes(w[i]->K, M, w[i]->N));
     if (!use_mfma_kernel(w[0]->type, M, w[0]->K)) return need;
     int64_t sum_n = 0, rgs = 0;
     for (int i = 0; i < n; ++i) {

@@ -151,6 +151,7 @@ hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, f
 int q8k_tile_splits(int64_t K, int64_t M, int64_t N);
 size_t q8k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N);
 hipError_t launch_sum_parts(const float *part, int n_split, size_t n, float *y, hipStream_t s);
+size_t q4k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N);   // what launch_gemm_q8k asks of its scratch
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s);
 hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, int64_t M, float *const *y,
                                  const Scratch &scratch, hipStream_t s);

@@ -841,6 +841,60 @@ def test_full_size_prefill_gemm_against_device_fp64(ctx):
     err = ((y.double() - ref).abs() / ref.abs().clamp(min=1.0)).max().item()
     assert err <= 5e-5, err
 
+@pytest.mark.parametrize("m", [64, 130, 512])
+def test_q6k_prefill_extreme_codes_and_scales(ctx, orc, m):
+    """The Q6_K prefill kernels carry sc * (q - 32) as two int8 operands, 256 * hi + lo with hi in [-16, 16] and lo
+    a signed byte, and add each over a whole super-block in int32: |I_lo| <= 256 * 128 * 127 < 2^23,
+    |I_hi| <= 256 * 16 * 127 < 2^20, (I_hi << 8) + I_lo < 2^28 -- the exact integer ggml's vec_dot forms, no
+    rounding anywhere before the one fp32 scaling per super-block.  Rows built to sit on those bounds: every code
+    0 or 63 (q - 32 = -32 or 31), every scale -128 or 127 or a mix with small ones, activations that quantize to
+    +-127 throughout, beside ordinary rows; d = 1 so nothing hides behind a small scale.  Against the oracle, both
+    the 64-token and the 128-token kernel (M = 512 takes the latter with K cut in stretches)."""
+    from magnitude_amd import ACT_GGML
+    rng = np.random.default_rng(600 + m)
+    k, n = 3072, 160
+    nb = k // 256
+    blocks = encode(Q6_K, (rng.standard_normal((n, k)) * 0.02).astype(np.float32)).reshape(n, nb, 210).copy()
+    one = np.frombuffer(np.float16(1.0).tobytes(), np.uint8)
+    pat = [(0x00, 0x00, 0x80), (0xff, 0xff, 0x7f), (0x00, 0x00, 0x7f), (0xff, 0xff, 0x80), (0xff, 0x00, 0x80), (0x0f, 0xff, 0x7f)]
+    for r in range(96):
+        ql, qh, sc = pat[r % len(pat)]
+        blocks[r, :, 0:128] = ql
+        blocks[r, :, 128:192] = qh
+        blocks[r, :, 192:208] = sc
+        if r % 12 >= 6:     # alternating extreme scales inside a super-block, and small ones between
+            blocks[r, :, 192:208] = np.array([0x80, 0x7f, 0x01, 0xff] * 4, np.uint8)
+        blocks[r, :, 208:210] = one
+    blocks = blocks.reshape(n, -1)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    x[0] = 1.0                                  # every code -127
+    x[1] = -3.0                                 # every code -127 with d > 0 ... and its mirror image
+    x[2] = np.where(np.arange(k) % 2 == 0, 2.0, -2.0)
+    x[3, :] = 0.0
+    x[3, 5::256] = 9.0                          # one non-zero code per super-block
+    w = ctx.upload(Q6_K, k, n, blocks)
+    got = ctx.mul_mat(w, dev(x), ACT_GGML).cpu().numpy()
+    want = orc.mul_mat(Q6_K, blocks, k, x, orc.ACT_GGML)
+    assert np.abs(want[:4, :96]).max() > 1e7    # the extreme rows do reach the large sums
+    close(got[:, 96:], want[:, 96:], 2e-5)      # ordinary rows: the usual bar against the oracle
+    # Extreme rows: with d = 1 the dequantized weights are the integers sc * (q - 32), so the exact result is
+    # sum_sb dx[m, sb] * I[m, n, sb] with I an exact integer.  Random activations make those twelve terms of ~1e5
+    # cancel to a few tens, so "relative to the result" measures the fp32 order of summation (the oracle's eight
+    # interleaved lanes against one sum per super-block here), not the arithmetic.  The bar is relative to the
+    # mass of the terms instead: (float)I, the scale product and one fma per super-block each round once.
+    wi = orc.dequantize(Q6_K, blocks[:96], k).astype(np.float64)
+    assert np.array_equal(wi, np.rint(wi)) and np.abs(wi).max() == 4096
+    raw = orc.quantize_q8_K(x).reshape(m, nb, 292)
+    dx = raw[:, :, 0:4].copy().view(np.float32)[:, :, 0].astype(np.float64)
+    qa = raw[:, :, 4:260].view(np.int8).astype(np.float64)
+    ints = np.einsum("msk,nsk->mns", qa, wi.reshape(96, nb, 256))          # exact: |I| < 2^28
+    exact = (ints * dx[:, None, :]).sum(-1)
+    mass = np.abs(ints * dx[:, None, :]).sum(-1)
+    assert np.all(np.abs(got[:, :96] - exact) <= 1e-6 * mass + 1e-30)
+    assert np.all(np.abs(want[:, :96] - exact) <= 1e-6 * mass + 1e-30)     # the oracle meets the same bar
+    w.free()
+
+
 BENCHED_PREFILL = (   # every (mode, type, K, N) x M the benchmark's prefill leg times (config 4 and the layer's other formats)
     [("q8x32", Q4_K, k, n) for (k, n) in ((4096, 14336), (14336, 4096), (4096, 4096))] +
     [("ggml", Q4_K, k, n) for (k, n) in ((4096, 14336), (14336, 4096), (4096, 4096))] +
