@@ -142,6 +142,14 @@ int qproj_rms_norm_ffn_gate_up(qproj_ctx *ctx, const qproj_weight *gate, const q
                                const float *x_dev, const float *gamma_dev, float eps, int64_t M, float *h_dev,
                                int act);
 
+/* The whole dense feed-forward of llama.cpp's build_ffn (LLM_FFN_SILU, LLM_FFN_PAR), optionally behind the block's
+ * RMS norm (use_norm != 0; gamma_dev may be null):
+ *     y_dev[M][N] = down . ( silu(gate . x') * (up . x') ),   x' = rms_norm(x) * gamma or x.
+ * gate and up are [K -> d_ff], down is [d_ff -> N].  Runs qproj_(rms_norm_)ffn_gate_up into scratch of the context and
+ * qproj_mul_mat on the result: two launches for M <= 2, and bit-identical to those two calls. */
+int qproj_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, const qproj_weight *down,
+              const float *x_dev, const float *gamma_dev, float eps, int use_norm, int64_t M, float *y_dev, int act);
+
 /* GGML_OP_MUL_MAT: y_dev[M][N] = x_dev[M][K] . W^T.  Picks the decode (M=1), small-batch
  * (M<=16) or prefill kernel from M.  W must have n_expert == 1. */
 int qproj_mul_mat(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, int64_t M, float *y_dev,

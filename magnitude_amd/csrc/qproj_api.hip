@@ -963,6 +963,27 @@ int qproj_rms_norm_ffn_gate_up(qproj_ctx *ctx, const qproj_weight *gate, const q
     return ffn_gate_up_impl(ctx, gate, up, x_dev, M, h_dev, act, &norm);
 }
 
+int qproj_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, const qproj_weight *down, const float *x_dev,
+              const float *gamma_dev, float eps, int use_norm, int64_t M, float *y_dev, int act) {
+    if (!ctx) return QPROJ_ERR_INVALID_ARG;
+    if (!gate || !up || !down || !x_dev || !y_dev) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_ffn: null argument");
+    if (gate->E != 1 || up->E != 1 || down->E != 1 || gate->K != up->K || gate->N != up->N || gate->type != up->type ||
+        down->K != gate->N)
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_ffn: gate/up/down shapes do not agree");
+    if (M < 0) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_ffn: negative M");
+    if (M == 0) return QPROJ_OK;
+    QP_HIP(ctx, hipSetDevice(ctx->device));
+    const int64_t K = gate->K, d_ff = gate->N;
+    const NormSpec norm{gamma_dev, eps};
+    // the scratch row(s) h between the halves, kept apart from the workspace the projections themselves use
+    int rc = ensure_ws2(ctx, (size_t)3 * M * d_ff * 4);
+    if (rc) return rc;
+    float *h = reinterpret_cast<float *>(ctx->ws2) + (size_t)2 * M * d_ff;
+    rc = ffn_gate_up_impl(ctx, gate, up, x_dev, M, h, act, use_norm ? &norm : nullptr);
+    if (rc) return rc;
+    return qproj_mul_mat(ctx, down, h, M, y_dev, act);
+}
+
 int qproj_mul_mat_quantized(qproj_ctx *ctx, int n, const qproj_weight *const *w, const void *act_dev, int kind,
                             int64_t M, float *const *y_dev) {
     if (!ctx) return QPROJ_ERR_INVALID_ARG;

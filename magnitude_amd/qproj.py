@@ -52,6 +52,7 @@ SYMBOLS = {
     "qproj_rms_norm_ffn_gate_up": (_i32, [_vp, _vp, _vp, _vp, _vp, C.c_float, _i64, _vp, _i32]),
     "qproj_rms_norm_mul_mat": (_i32, [_vp, _i32, _vp, _vp, _vp, C.c_float, _i64, _vp, _i32]),
     "qproj_rms_norm_quantize": (_i32, [_vp, _i32, _i32, _vp, _vp, C.c_float, _i64, _i64, _vp]),
+    "qproj_ffn": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, C.c_float, _i32, _i64, _vp, _i32]),
     "qproj_mul_mat": (_i32, [_vp, _vp, _vp, _i64, _vp, _i32]),
     "qproj_mul_mat_multi": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i64, C.POINTER(_vp), _i32]),
     "qproj_mul_mat_multi_noalloc": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i64, C.POINTER(_vp), _i32]),
@@ -413,6 +414,22 @@ class Context:
         if sync:
             self.sync()
         return outs
+
+    def ffn(self, gate: Weight, up: Weight, down: Weight, x: torch.Tensor, act: int = ACT_GGML,
+            gamma: Optional[torch.Tensor] = None, eps: Optional[float] = None, out: Optional[torch.Tensor] = None,
+            sync: bool = True) -> torch.Tensor:
+        """down . (silu(gate . x') * (up . x')), x' = rms_norm(x) * gamma when eps is given: the dense feed-forward."""
+        x = x.contiguous()
+        m = x.shape[0]
+        y = out if out is not None else torch.empty((m, down.N), dtype=torch.float32, device=x.device)
+        if sync:
+            torch.cuda.current_stream().synchronize()
+        self._check(self.lib.qproj_ffn(self.handle, gate.handle, up.handle, down.handle, _ptr(x),
+                                       0 if gamma is None else _ptr(gamma.contiguous()),
+                                       C.c_float(0.0 if eps is None else eps), 0 if eps is None else 1, m, _ptr(y), act))
+        if sync:
+            self.sync()
+        return y
 
     def mul_mat_id(self, w: Weight, x: torch.Tensor, ids: torch.Tensor, act: int = ACT_GGML,
                    sync: bool = True) -> torch.Tensor:

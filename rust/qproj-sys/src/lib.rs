@@ -66,6 +66,9 @@ extern "C" {
     pub fn qproj_rms_norm_ffn_gate_up(ctx: *mut qproj_ctx, gate: *const qproj_weight,
                                       up: *const qproj_weight, x_dev: *const f32, gamma_dev: *const f32,
                                       eps: f32, m: i64, h_dev: *mut f32, act: c_int) -> c_int;
+    pub fn qproj_ffn(ctx: *mut qproj_ctx, gate: *const qproj_weight, up: *const qproj_weight,
+                     down: *const qproj_weight, x_dev: *const f32, gamma_dev: *const f32, eps: f32,
+                     use_norm: c_int, m: i64, y_dev: *mut f32, act: c_int) -> c_int;
     pub fn qproj_mul_mat(ctx: *mut qproj_ctx, w: *const qproj_weight, x_dev: *const f32, m: i64,
                          y_dev: *mut f32, act: c_int) -> c_int;
     pub fn qproj_mul_mat_multi(ctx: *mut qproj_ctx, n: c_int, w: *const *const qproj_weight,

@@ -894,6 +894,41 @@ def test_q6k_prefill_extreme_codes_and_scales(ctx, orc, m):
     assert np.all(np.abs(want[:, :96] - exact) <= 1e-6 * mass + 1e-30)     # the oracle meets the same bar
     w.free()
 
+@pytest.mark.parametrize("down_type", [Q4_K, Q6_K])
+@pytest.mark.parametrize("m", [1, 2, 5])
+def test_ffn_equals_the_chain_and_the_oracle(ctx, orc, down_type, m):
+    """qproj_ffn = norm -> gate/up -> swiglu -> down: bit for bit what qproj_(rms_norm_)ffn_gate_up followed by
+    qproj_mul_mat gives, with and without the norm, on calls in a row; against the CPU restatement at the
+    re-quantized-intermediate bar of the MoE feed-forward (2e-4)."""
+    from magnitude_amd import ACT_GGML
+    for d_model, d_ff in ((512, 768), (4096, 2048)):
+        rng = np.random.default_rng(7000 + d_model + d_ff + m + down_type)
+        gate_b = make_weight(orc, Q4_K, d_ff, d_model, seed=7100 + d_ff)
+        up_b = make_weight(orc, Q4_K, d_ff, d_model, seed=7200 + d_ff)
+        down_b = make_weight(orc, down_type, d_model, d_ff, seed=7300 + d_ff + down_type)
+        wg, wu, wd = ctx.upload(Q4_K, d_model, d_ff, gate_b), ctx.upload(Q4_K, d_model, d_ff, up_b), ctx.upload(down_type, d_ff, d_model, down_b)
+        gam = dev((1.0 + 0.1 * rng.standard_normal(d_model)).astype(np.float32))
+        xs = [dev(rng.standard_normal((m, d_model)).astype(np.float32)) for _ in range(3)]
+        for norm in (False, True):
+            kw = dict(gamma=gam, eps=1e-5) if norm else {}
+            outs = [torch.full((m, d_model), float("nan"), device="cuda") for _ in xs]
+            for x, y in zip(xs, outs):
+                ctx.ffn(wg, wu, wd, x, ACT_GGML, out=y, sync=False, **kw)
+            ctx.sync()
+            for x, y in zip(xs, outs):
+                h = ctx.ffn_gate_up(wg, wu, x, ACT_GGML, **kw)
+                want = ctx.mul_mat(wd, h, ACT_GGML)
+                assert torch.equal(y.view(torch.int32), want.view(torch.int32)), f"norm={norm}"
+        xh = xs[0].cpu().numpy()
+        go, uo = orc.mul_mat(Q4_K, gate_b, d_model, xh, orc.ACT_GGML), orc.mul_mat(Q4_K, up_b, d_model, xh, orc.ACT_GGML)
+        hh = (go / (1.0 + np.exp(-go.astype(np.float64)))).astype(np.float32) * uo
+        ref = orc.mul_mat(down_type, down_b, d_ff, hh, orc.ACT_GGML)
+        got = ctx.ffn(wg, wu, wd, xs[0], ACT_GGML).cpu().numpy()
+        close(got, ref, 2e-4)
+        gate(got, ref)
+        for w in (wg, wu, wd):
+            w.free()
+
 
 BENCHED_PREFILL = (   # every (mode, type, K, N) x M the benchmark's prefill leg times (config 4 and the layer's other formats)
     [("q8x32", Q4_K, k, n) for (k, n) in ((4096, 14336), (14336, 4096), (4096, 4096))] +
