@@ -346,24 +346,36 @@ size_t per32_scratch_max(int n, const qproj_weight *const *w, int64_t M) {   // 
     return need;
 }
 
-// Q8_0 takes the tiled product from 64 rows on, K a multiple of 128.  One predicate for the dispatch and for the
-// scratch sizing: the partial tiles of a K cut into stretches go to scratch that only this rule provides.
-bool q8_0_tiled(const qproj_weight *t, int64_t M) { return t->type == kTypeQ8_0 && t->K % 128 == 0 && M >= 64; }
+// Which batches take the tiled matrix-core products (weights reused across a tile of tokens, K cut into stretches
+// where the grid would leave the chip idle) instead of passes of the 16-row small-batch kernel.  ONE predicate for
+// the dispatch and for the scratch sizing: the partial tiles of a K cut into stretches go to scratch that only this
+// rule provides.  Q8_0 from 64 rows on with K a multiple of 128; Q4_K and Q6_K from the row counts below.
+int tiled_min_m(int type) {
+    static const int q4 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q4K", 17));
+    static const int q6 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q6K", 32));
+    return type == kTypeQ4_K ? q4 : type == kTypeQ6_K ? q6 : 64;
+}
+bool takes_tiled(const qproj_weight *t, int64_t M) {
+    if (M < tiled_min_m(t->type)) return false;
+    return t->type != kTypeQ8_0 || t->K % 128 == 0;
+}
 
 size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
-    if (q8_0_tiled(w[0], M)) return per32_scratch_max(n, w, M);
-    size_t need = 0;
-    if (M > 16 && w[0]->type != kTypeQ8_0)   // tiled Q4_K / Q6_K products with K cut into stretches
+    if (takes_tiled(w[0], M)) {
+        if (w[0]->type == kTypeQ8_0) return per32_scratch_max(n, w, M);
+        size_t need = 0;
         for (int i = 0; i < n; ++i)
             need = std::max(need, w[0]->type == kTypeQ6_K ? q6k_tile_scratch_bytes(w[i]->K, M, w[i]->N)
                                                           : q4k_tile_scratch_bytes(w[i]->K, M, w[i]->N));
-    if (!use_mfma_kernel(w[0]->type, M, w[0]->K)) return need;
+        return need;
+    }
+    if (!use_mfma_kernel(w[0]->type, M, w[0]->K)) return 0;
     int64_t sum_n = 0, rgs = 0;
     for (int i = 0; i < n; ++i) {
         sum_n += w[i]->N;
         rgs += (w[i]->N + 31) / 32;
     }
-    need = std::max(need, mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, std::min<int64_t>(M, 16), sum_n, rgs));
+    size_t need = mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, std::min<int64_t>(M, 16), sum_n, rgs);
     if (M > 16 && M % 16) need = std::max(need, mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, M % 16, sum_n, rgs));
     return need;
 }
@@ -380,18 +392,10 @@ bool dense_fuses_quantizer(const qproj_weight *w, int64_t M) {
 // x_f32: non-null when `a` carries no planes and the kernel quantizes these rows itself (small batches only)
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
                     float *const *y, const Scratch &sc, const float *x_f32 = nullptr) {
-    // (never under 17: the scratch for K cut into stretches is sized for more than 16 rows only)
-    static const int gemm_min_m = std::max(17, tuning_int("QPROJ_GEMM_MIN_M", 17));
-    // Beyond the 16 rows one pass of the small-batch kernel takes: the tiled product, weights reused across 64
+    // Beyond the rows one pass of the small-batch kernel takes: the tiled product, weights reused across a tile of
     // tokens, K cut into stretches where the grid would leave the chip idle.  (Measured, 8B shapes: Q4_K 17..47
-    // rows 19-72 us in steps of 16 against 15-31 us tiled; Q6_K, whose workgroups are slow -- a vector
-    // multiply-add per output and sub-block --, pays from 32 rows on: 62-206 us in steps against 58-63 tiled.)
-    const auto tiled = [&](const qproj_weight *t) {
-        if (M < gemm_min_m) return false;
-        if (t->type == kTypeQ4_K) return true;
-        if (t->type == kTypeQ8_0) return q8_0_tiled(t, M);
-        return t->type == kTypeQ6_K && M >= 32;
-    };
+    // rows 19-72 us in steps of 16 against 15-31 us tiled; Q6_K pays from 32 rows on.)
+    const auto tiled = [&](const qproj_weight *t) { return takes_tiled(t, M); };
     if (tiled(w[0])) {
         if (w[0]->type == kTypeQ4_K && n >= 2 && n <= 3) {   // q/k/v, gate/up: one launch where the tiles allow it
             WeightView views[3];
