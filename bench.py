@@ -644,23 +644,34 @@ def main():
         nl = min(4, L)
         host = [[(qt, n, k, ctx.download(layers[l][name])) for name, qt, n, k in LAYER_TENSORS] for l in range(nl)]
         xs = {D_MODEL: x_attn.cpu().numpy(), D_FF: x_down.cpu().numpy()}
+        # every thread of the box's CPU share (16 for one GPU); the reference's own policy is one thread per physical
+        # core (inference/parity/profiles/pr.toml:41).  AVX2 dot products in the shape of ggml's x86 path when the
+        # oracle was built with them, the generic C loops otherwise.
         threads = min(orc.max_threads(), 16)
+        avx2 = orc.has_avx2()
+        run_cpu = (lambda qt, blocks, k, th: orc.time_mul_mat_avx2(qt, blocks, k, xs[k], th, 1)) if avx2 else \
+                  (lambda qt, blocks, k, th: orc.time_mul_mat(qt, blocks, k, xs[k], orc.ACT_GGML, th, 1))
         t_end = time.time() + args.cpu_seconds
         passes, spent = 0, 0.0
         while passes < 2 or time.time() < t_end:
             for lw in host:
                 for qt, n, k, blocks in lw:
-                    spent += orc.time_mul_mat(qt, blocks, k, xs[k], orc.ACT_GGML, threads, 1)
+                    spent += run_cpu(qt, blocks, k, threads)
             passes += 1
         cpu_gbs = passes * nl * LAYER_BYTES / spent / 1e9
-        one = 0.0                                  # one thread, one layer: the scalar figure beside the threaded one
+        one = 0.0                                  # one thread, one layer
         for qt, n, k, blocks in host[0]:
-            one += orc.time_mul_mat(qt, blocks, k, xs[k], orc.ACT_GGML, 1, 1)
+            one += run_cpu(qt, blocks, k, 1)
+        scalar_one = 0.0                           # the same with the generic C loops the parity tests use
+        for qt, n, k, blocks in host[0]:
+            scalar_one += orc.time_mul_mat(qt, blocks, k, xs[k], orc.ACT_GGML, 1, 1)
         out["cpu_baseline"] = {"value": cpu_gbs, "unit": "GB/s", "cores": threads, "kind": "port",
                                "sample": f"{passes} passes over {nl} of the same layers (7 projections each, M=1, "
-                                         f"ggml activation mode), {spent:.1f} s of OpenMP C on the host",
+                                         f"ggml activation mode), {spent:.1f} s on the host",
+                               "isa": "AVX2 maddubs/madd dot products, OpenMP over rows" if avx2 else "generic C, OpenMP over rows",
                                "host_cpus": os.cpu_count(),
-                               "one_thread_GBps": LAYER_BYTES / one / 1e9}
+                               "one_thread_GBps": LAYER_BYTES / one / 1e9,
+                               "one_thread_generic_c_GBps": LAYER_BYTES / scalar_one / 1e9}
         log(f"[bench] cpu baseline: {cpu_gbs:.2f} GB/s on {threads} threads")
 
     # ------------------------------------------------------------------ llama-bench style leg

@@ -80,6 +80,11 @@ def lib() -> C.CDLL:
         L.orc_rms_norm.restype = None
         L.orc_time_mul_mat.argtypes = [i32, vp, i64, i64, f32p, i64, f32p, i32, i32, i32]
         L.orc_max_threads.restype = i32
+        L.orc_has_avx2.restype = i32
+        L.orc_mul_mat_avx2.restype = i32
+        L.orc_mul_mat_avx2.argtypes = [i32, vp, i64, i64, f32p, i64, f32p, i32]
+        L.orc_time_mul_mat_avx2.restype = C.c_double
+        L.orc_time_mul_mat_avx2.argtypes = [i32, vp, i64, i64, f32p, i64, f32p, i32, i32]
         _lib = L
     return _lib
 
@@ -214,6 +219,35 @@ def time_mul_mat(qtype: int, w: np.ndarray, k: int, x: np.ndarray, act: int, nth
     m = x.shape[0]
     y = np.empty((m, n), dtype=np.float32)
     return float(lib().orc_time_mul_mat(qtype, _p(w), k, n, _p(x), m, _p(y), act, nthreads, reps))
+
+
+def has_avx2() -> bool:
+    return bool(lib().orc_has_avx2())
+
+
+def mul_mat_avx2(qtype: int, w: np.ndarray, k: int, x: np.ndarray, nthreads: int = 8) -> np.ndarray:
+    """mul_mat in the ggml activation mode through the AVX2 dot products (the CPU-baseline code path)."""
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, k)
+    n = w.size // row_bytes(qtype, k)
+    m = x.shape[0]
+    y = np.empty((m, n), dtype=np.float32)
+    rc = lib().orc_mul_mat_avx2(qtype, _p(w), k, n, _p(x), m, _p(y), nthreads)
+    if rc:
+        raise RuntimeError(f"orc_mul_mat_avx2 failed rc={rc}")
+    return y
+
+
+def time_mul_mat_avx2(qtype: int, w: np.ndarray, k: int, x: np.ndarray, nthreads: int, reps: int) -> float:
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, k)
+    n = w.size // row_bytes(qtype, k)
+    m = x.shape[0]
+    y = np.empty((m, n), dtype=np.float32)
+    t = float(lib().orc_time_mul_mat_avx2(qtype, _p(w), k, n, _p(x), m, _p(y), nthreads, reps))
+    if t < 0:
+        raise RuntimeError("the oracle was built without AVX2")
+    return t
 
 
 def rms_norm(x: np.ndarray, gamma, eps: float) -> np.ndarray:

@@ -22,7 +22,7 @@
 #ifdef _OPENMP
 #include <omp.h>
 #endif
-#if defined(__F16C__)
+#if defined(__F16C__) || defined(__AVX2__)
 #include <immintrin.h>
 #endif
 
@@ -629,6 +629,167 @@ int orc_max_threads(void) {
 #else
     return 1;
 #endif
+}
+
+/* ---------------------------------------------------------------- AVX2 dot products (CPU baseline timing)
+ *
+ * ggml's CPU backend does not run the generic C loops above on x86: its ggml-cpu/arch/x86/quants.c holds AVX2
+ * forms of the same dot products (unsigned x signed byte products with maddubs, 16-bit pair sums with madd, one
+ * float multiply-add per block).  These follow that shape so that the CPU baseline timed beside the GPU is the
+ * kind of code the reference's CPU path runs, not scalar C.  Same integers as the generic functions, another
+ * order of the float additions; tests hold them to the generic ones within 1e-5.  Never used as the parity
+ * reference. */
+#if defined(__AVX2__)
+static inline float hsum8(__m256 v) {
+    __m128 r = _mm_add_ps(_mm256_castps256_ps128(v), _mm256_extractf128_ps(v, 1));
+    r = _mm_add_ps(r, _mm_movehl_ps(r, r));
+    r = _mm_add_ss(r, _mm_movehdup_ps(r));
+    return _mm_cvtss_f32(r);
+}
+
+float orc_vec_dot_q8_0_q8_0_avx2(int64_t k, const orc_block_q8_0 *w, const orc_block_q8_0 *a) {
+    const int64_t nb = k / ORC_QK8_0;
+    __m256 acc = _mm256_setzero_ps();
+    const __m256i ones = _mm256_set1_epi16(1);
+    for (int64_t ib = 0; ib < nb; ++ib) {
+        const __m256 d = _mm256_set1_ps(orc_fp16_to_fp32_f16c(w[ib].d) * orc_fp16_to_fp32_f16c(a[ib].d));
+        const __m256i qw = _mm256_loadu_si256((const __m256i *)w[ib].qs);
+        const __m256i qa = _mm256_loadu_si256((const __m256i *)a[ib].qs);
+        /* |w| * sign(w)(a): unsigned x signed bytes */
+        const __m256i p16 = _mm256_maddubs_epi16(_mm256_sign_epi8(qw, qw), _mm256_sign_epi8(qa, qw));
+        const __m256i p32 = _mm256_madd_epi16(p16, ones);
+        acc = _mm256_fmadd_ps(d, _mm256_cvtepi32_ps(p32), acc);
+    }
+    return hsum8(acc);
+}
+
+float orc_vec_dot_q4_K_q8_K_avx2(int64_t k, const orc_block_q4_K *w, const orc_block_q8_K *a) {
+    const int64_t nb = k / ORC_QK_K;
+    const __m256i m4 = _mm256_set1_epi8(0xF);
+    __m256 acc = _mm256_setzero_ps();
+    float acc_m = 0.f;
+    for (int64_t i = 0; i < nb; ++i) {
+        const float d = a[i].d * orc_fp16_to_fp32_f16c(w[i].d);
+        const float dmin = a[i].d * orc_fp16_to_fp32_f16c(w[i].dmin);
+        uint8_t sc[8], mn[8];
+        for (int j = 0; j < 8; ++j) orc_get_scale_min_k4(j, w[i].scales, &sc[j], &mn[j]);
+        int summ = 0;
+        for (int j = 0; j < 8; ++j) summ += mn[j] * (a[i].bsums[2 * j] + a[i].bsums[2 * j + 1]);
+        acc_m += dmin * (float)summ;
+        const uint8_t *q4 = w[i].qs;
+        const int8_t *q8 = a[i].qs;
+        __m256i sumi = _mm256_setzero_si256();
+        for (int j = 0; j < ORC_QK_K / 64; ++j) {
+            const __m256i s_l = _mm256_set1_epi16(sc[2 * j]), s_h = _mm256_set1_epi16(sc[2 * j + 1]);
+            const __m256i q4b = _mm256_loadu_si256((const __m256i *)q4);
+            q4 += 32;
+            const __m256i q4l = _mm256_and_si256(q4b, m4);
+            const __m256i q4h = _mm256_and_si256(_mm256_srli_epi16(q4b, 4), m4);
+            const __m256i q8l = _mm256_loadu_si256((const __m256i *)q8);
+            q8 += 32;
+            const __m256i q8h = _mm256_loadu_si256((const __m256i *)q8);
+            q8 += 32;
+            const __m256i p16l = _mm256_madd_epi16(s_l, _mm256_maddubs_epi16(q4l, q8l));
+            const __m256i p16h = _mm256_madd_epi16(s_h, _mm256_maddubs_epi16(q4h, q8h));
+            sumi = _mm256_add_epi32(sumi, _mm256_add_epi32(p16l, p16h));
+        }
+        acc = _mm256_fmadd_ps(_mm256_set1_ps(d), _mm256_cvtepi32_ps(sumi), acc);
+    }
+    return hsum8(acc) - acc_m;
+}
+
+float orc_vec_dot_q6_K_q8_K_avx2(int64_t k, const orc_block_q6_K *w, const orc_block_q8_K *a) {
+    const int64_t nb = k / ORC_QK_K;
+    const __m256i m4 = _mm256_set1_epi8(0xF), m2 = _mm256_set1_epi8(3), m32s = _mm256_set1_epi8(32);
+    __m256 acc = _mm256_setzero_ps();
+    for (int64_t i = 0; i < nb; ++i) {
+        const float d = a[i].d * orc_fp16_to_fp32_f16c(w[i].d);
+        const uint8_t *q4 = w[i].ql, *qh = w[i].qh;
+        const int8_t *q8 = a[i].qs;
+        __m256i sumi = _mm256_setzero_si256();
+        for (int j = 0; j < ORC_QK_K / 128; ++j) {
+            const __m256i q4b1 = _mm256_loadu_si256((const __m256i *)q4);
+            const __m256i q4b2 = _mm256_loadu_si256((const __m256i *)(q4 + 32));
+            q4 += 64;
+            const __m256i q4bh = _mm256_loadu_si256((const __m256i *)qh);
+            qh += 32;
+            const __m256i h0 = _mm256_slli_epi16(_mm256_and_si256(q4bh, m2), 4);
+            const __m256i h1 = _mm256_slli_epi16(_mm256_and_si256(_mm256_srli_epi16(q4bh, 2), m2), 4);
+            const __m256i h2 = _mm256_slli_epi16(_mm256_and_si256(_mm256_srli_epi16(q4bh, 4), m2), 4);
+            const __m256i h3 = _mm256_slli_epi16(_mm256_and_si256(_mm256_srli_epi16(q4bh, 6), m2), 4);
+            const __m256i q0 = _mm256_or_si256(_mm256_and_si256(q4b1, m4), h0);
+            const __m256i q1 = _mm256_or_si256(_mm256_and_si256(q4b2, m4), h1);
+            const __m256i q2 = _mm256_or_si256(_mm256_and_si256(_mm256_srli_epi16(q4b1, 4), m4), h2);
+            const __m256i q3 = _mm256_or_si256(_mm256_and_si256(_mm256_srli_epi16(q4b2, 4), m4), h3);
+            const __m256i qs[4] = {q0, q1, q2, q3};
+            for (int g = 0; g < 4; ++g) {
+                const __m256i q8v = _mm256_loadu_si256((const __m256i *)q8);
+                q8 += 32;
+                /* (q - 32) * a = q * a - 32 * a, both as unsigned x signed byte products */
+                __m256i p16 = _mm256_sub_epi16(_mm256_maddubs_epi16(qs[g], q8v), _mm256_maddubs_epi16(m32s, q8v));
+                /* two sub-blocks of 16 in the 32 bytes: scale is[0] for the low lane, is[1] for the high lane */
+                const int is = 8 * j + 2 * g;
+                const __m256i sc = _mm256_set_m128i(_mm_set1_epi16(w[i].scales[is + 1]), _mm_set1_epi16(w[i].scales[is]));
+                sumi = _mm256_add_epi32(sumi, _mm256_madd_epi16(sc, p16));
+            }
+        }
+        acc = _mm256_fmadd_ps(_mm256_set1_ps(d), _mm256_cvtepi32_ps(sumi), acc);
+    }
+    return hsum8(acc);
+}
+
+static float dot_quantized_avx2(int type, int64_t K, const void *wrow, const void *arow) {
+    switch (type) {
+    case ORC_TYPE_Q8_0:
+        return orc_vec_dot_q8_0_q8_0_avx2(K, (const orc_block_q8_0 *)wrow, (const orc_block_q8_0 *)arow);
+    case ORC_TYPE_Q4_K:
+        return orc_vec_dot_q4_K_q8_K_avx2(K, (const orc_block_q4_K *)wrow, (const orc_block_q8_K *)arow);
+    default:
+        return orc_vec_dot_q6_K_q8_K_avx2(K, (const orc_block_q6_K *)wrow, (const orc_block_q8_K *)arow);
+    }
+}
+#endif
+
+int orc_has_avx2(void) {
+#if defined(__AVX2__)
+    return 1;
+#else
+    return 0;
+#endif
+}
+
+/* orc_mul_mat in the ggml activation mode with the AVX2 dot products (timing and its cross-check only) */
+int orc_mul_mat_avx2(int type, const void *w, int64_t K, int64_t N, const float *x, int64_t M, float *y, int nthreads) {
+#if defined(__AVX2__)
+    const size_t rb = orc_row_bytes(type, K);
+    if (rb == 0) return -1;
+    if (nthreads < 1) nthreads = 1;
+    const size_t ab = act_row_bytes(type, ORC_ACT_GGML, K);
+    char *aq = (char *)malloc(ab * (size_t)M);
+    if (!aq) return -2;
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+    for (int64_t m = 0; m < M; ++m) quantize_act_row(type, ORC_ACT_GGML, x + m * K, aq + (size_t)m * ab, K);
+#pragma omp parallel for num_threads(nthreads) schedule(static)
+    for (int64_t n = 0; n < N; ++n) {
+        const void *wrow = (const char *)w + (size_t)n * rb;
+        for (int64_t m = 0; m < M; ++m) y[m * N + n] = dot_quantized_avx2(type, K, wrow, aq + (size_t)m * ab);
+    }
+    free(aq);
+    return 0;
+#else
+    (void)type; (void)w; (void)K; (void)N; (void)x; (void)M; (void)y; (void)nthreads;
+    return -3;
+#endif
+}
+
+double orc_time_mul_mat_avx2(int type, const void *w, int64_t K, int64_t N, const float *x, int64_t M, float *y,
+                             int nthreads, int reps) {
+    struct timespec t0, t1;
+    clock_gettime(CLOCK_MONOTONIC, &t0);
+    for (int r = 0; r < reps; ++r)
+        if (orc_mul_mat_avx2(type, w, K, N, x, M, y, nthreads) != 0) return -1.0;
+    clock_gettime(CLOCK_MONOTONIC, &t1);
+    return (double)(t1.tv_sec - t0.tv_sec) + 1e-9 * (double)(t1.tv_nsec - t0.tv_nsec);
 }
 
 double orc_time_mul_mat(int type, const void *w, int64_t K, int64_t N, const float *x, int64_t M,

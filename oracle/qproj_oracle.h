@@ -113,6 +113,14 @@ float orc_vec_dot_q4_K_q8_K(int64_t k, const orc_block_q4_K *w, const orc_block_
 float orc_vec_dot_q6_K_q8_K(int64_t k, const orc_block_q6_K *w, const orc_block_q8_K *a);
 float orc_vec_dot_q8x32(int type, int64_t k, const void *w, const orc_block_q8x32 *a);
 
+/* AVX2 forms of the three dot products in the shape of ggml's x86 path (CPU-baseline timing only; same integers,
+ * another order of the float additions) and the mul_mat / timer built on them; orc_has_avx2() tells whether the
+ * library was built with them (orc_mul_mat_avx2 returns -3 otherwise). */
+int orc_has_avx2(void);
+int orc_mul_mat_avx2(int type, const void *w, int64_t K, int64_t N, const float *x, int64_t M, float *y, int nthreads);
+double orc_time_mul_mat_avx2(int type, const void *w, int64_t K, int64_t N, const float *x, int64_t M, float *y,
+                             int nthreads, int reps);
+
 /* y[m*N + n] = sum_k W[n,k] * x[m*K + k];  W = N rows of K quantized weights. */
 int orc_mul_mat(int type, const void *w, int64_t K, int64_t N, const float *x, int64_t M,
                 float *y, int act, int nthreads);

@@ -615,3 +615,35 @@ def test_rms_norm_against_fp64_and_scale_invariance(orc):
         assert np.array_equal(orc.rms_norm(x * np.float32(8.0), g, 0.0), y0)
         assert np.array_equal(orc.rms_norm(x, None, 0.0) * g, y0)
 
+
+@pytest.mark.parametrize("qtype,k", [(Q8_0, 4096), (Q4_K, 4096), (Q6_K, 14336), (Q4_K, 256), (Q6_K, 512), (Q8_0, 96)])
+def test_avx2_baseline_dots_agree_with_the_generic_ones(orc, qtype, k):
+    """The CPU baseline is timed on AVX2 forms of the dot products (the shape of ggml's x86 path).  They form the
+    same integers as the generic functions the parity tests use and add the floats in another order."""
+    if not orc.has_avx2():
+        pytest.skip("oracle built without AVX2")
+    rng = np.random.default_rng(k + qtype)
+    w = (rng.standard_normal((37, k)) * 0.02).astype(np.float32)
+    x = rng.standard_normal((3, k)).astype(np.float32)
+    x[1] *= 30.0
+    blocks = encode(qtype, w)
+    want = orc.mul_mat(qtype, blocks, k, x, orc.ACT_GGML)
+    got = orc.mul_mat_avx2(qtype, blocks, k, x)
+    assert np.max(np.abs(got - want) / np.maximum(1.0, np.abs(want))) <= 1e-5
+    # random byte patterns (every scale / min / code value), finite fp16 scales kept small
+    nblk = k // (32 if qtype == Q8_0 else 256)
+    size = {Q8_0: 34, Q4_K: 144, Q6_K: 210}[qtype]
+    raw = rng.integers(0, 256, (5 * nblk, size), dtype=np.uint8)
+    one = np.frombuffer(np.float16(0.01).tobytes(), np.uint8)
+    if qtype == Q8_0:
+        raw[:, 0:2] = one
+    elif qtype == Q4_K:
+        raw[:, 0:2] = one
+        raw[:, 2:4] = one
+    else:
+        raw[:, 208:210] = one
+    raw = raw.reshape(5, -1)
+    want = orc.mul_mat(qtype, raw, k, x, orc.ACT_GGML)
+    got = orc.mul_mat_avx2(qtype, raw, k, x)
+    # random codes and scales: terms far larger than their sum, so the order of the float additions shows more
+    assert np.max(np.abs(got - want) / np.maximum(1.0, np.abs(want))) <= 5e-5
