@@ -629,7 +629,7 @@ def test_avx2_baseline_dots_agree_with_the_generic_ones(orc, qtype, k):
     blocks = encode(qtype, w)
     want = orc.mul_mat(qtype, blocks, k, x, orc.ACT_GGML)
     got = orc.mul_mat_avx2(qtype, blocks, k, x)
-    assert np.max(np.abs(got - want) / np.maximum(1.0, np.abs(want))) <= 1e-5
+    assert np.max(np.abs(got - want) / np.maximum(1.0, np.abs(want))) <= 5e-5   # eight float lanes against one running sum
     # random byte patterns (every scale / min / code value), finite fp16 scales kept small
     nblk = k // (32 if qtype == Q8_0 else 256)
     size = {Q8_0: 34, Q4_K: 144, Q6_K: 210}[qtype]
