@@ -99,13 +99,18 @@ int qproj_dequantize(qproj_ctx *ctx, const qproj_weight *w, float *out_dev);
  * prefill format, for M rows of K floats.  `kind` = QPROJ_ACT_GGML with `wtype` selecting Q8_0 vs
  * Q8_K, or QPROJ_ACT_Q8X32.  Output planes in `out_dev` (size from qproj_act_bytes):
  *   Q8_0  : int8 qs[M][K] | f32 d[M][K/32]   (d already rounded through fp16)
- *   Q8_K  : int8 qs[M][K] | f32 d[M][K/256] | int16 bsums[M][K/16] | f16 msum[M][K/256][16]
- *           (msum: d * (sum of the 32 codes of a sub-block) / 16 as an fp16 pair, the 8 high parts of
- *           a super-block, then the 8 low parts; operand of the prefill kernel's min term)
- *   Q8X32 : int8 qs[M][K] | f32 d[M][K/32]  | int32 isum[M][K/32] | f16 msum[M][K/256][16] (as above)
+ *   Q8_K  : int8 qs[M][K] | f32 d[M][K/256] | int16 bsums[M][K/16] | f16 msum[M][K/256][16] | f32 rs[M]
+ *           (rs[m]: the largest power of two not above the row's largest |d|, 1 for an all-zero row;
+ *           msum: (d / rs[m]) * (sum of the 32 codes of a sub-block) / 16 as an fp16 pair, the 8 high parts of a
+ *           super-block, then the 8 low parts: the operand of the tiled kernels' min term, normalised by the row so
+ *           that it keeps its 22 bits whatever the size of the activations)
+ *   Q8X32 : int8 qs[M][K] | f32 d[M][K/32]  | int32 isum[M][K/32] | f16 msum[M][K/256][16] | f32 rs[M] (as above,
+ *           with the per-32 scales and sums)
  * each plane starting at a 256-byte aligned offset, in that order.  K must be a multiple of 32 for Q8_0 and of
  * 256 for Q8_K and Q8X32 (both carry one msum record per 256 weights of a row); qproj_act_bytes returns 0 and
- * qproj_quantize_activations QPROJ_ERR_INVALID_ARG otherwise. */
+ * qproj_quantize_activations QPROJ_ERR_INVALID_ARG otherwise.  Activations may have any finite size; the weight
+ * side of the same term is carried as fp16 pairs of dmin * min, which wants dmin * 63 < 65504 (GGUF files are
+ * orders of magnitude inside that). */
 size_t qproj_act_bytes(int kind, int wtype, int64_t M, int64_t K);
 int qproj_quantize_activations(qproj_ctx *ctx, int kind, int wtype, const float *x_dev, int64_t M,
                                int64_t K, void *out_dev);

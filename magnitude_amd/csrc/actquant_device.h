@@ -97,34 +97,25 @@ __device__ __forceinline__ uint32_t wave_quantize_q8_32(const float4 v, int &isu
 
 
 // One wave quantizes 256 consecutive floats (lane l holds elements 4l..4l+3 in `v`) as ggml's block_q8_K and
-// writes super-block `sb` of the planes, including d * (sum over each 32-wide sub-block) split into two fp16
-// parts in the order the prefill kernel feeds them to the fp16 matrix instruction.
+// writes super-block `sb` of the planes qs, d, bsums (the min-term plane is made afterwards, row by row:
+// minterm_rows_kernel)
 __device__ __forceinline__ void wave_store_q8k(const float4 &v, int lane, int64_t sb, int8_t *__restrict__ qs,
-                                               float *__restrict__ d, int16_t *__restrict__ bsums,
-                                               uint16_t *__restrict__ msum) {
+                                               float *__restrict__ d, int16_t *__restrict__ bsums) {
     int bsum;
     float dd;
     const uint32_t packed = wave_quantize_q8k(v, lane, bsum, dd);
     reinterpret_cast<uint32_t *>(qs + sb * 256)[lane] = packed;
     if ((lane & 3) == 0) bsums[sb * 16 + (lane >> 2)] = (int16_t)bsum;
     if (lane == 0) d[sb] = dd;
-    const int pair = bsum + __shfl_xor(bsum, 4);
-    if ((lane & 7) == 0) {
-        const float t = dd * (float)pair * kMinPrescale;
-        const _Float16 hi = (_Float16)t, lo = (_Float16)(t - (float)hi);
-        msum[sb * 16 + (lane >> 3)] = __builtin_bit_cast(uint16_t, hi);
-        msum[sb * 16 + 8 + (lane >> 3)] = __builtin_bit_cast(uint16_t, lo);
-    }
 }
 
 // The per-32 formats: lane l's four floats belong to block (e0 >> 5) of the flattened input, e0 = the lane's
-// first element; `ch` = e0 / 256 indexes the msum plane.  FP16_SCALE: ggml Q8_0 blocks (scale rounded through
-// fp16); otherwise fp32 scale, the integer sum of the block and its msum entry.  Every lane of the wave must
-// call this (shuffles inside); `live` = the lane's elements exist.
+// first element.  FP16_SCALE: ggml Q8_0 blocks (scale rounded through fp16); otherwise fp32 scale and the integer
+// sum of the block.  Every lane of the wave must call this (shuffles inside); `live` = the lane's elements exist.
 template <bool FP16_SCALE>
-__device__ __forceinline__ void wave_store_q8_32(const float4 &v, int lane, int64_t e0, int64_t ch, bool live,
+__device__ __forceinline__ void wave_store_q8_32(const float4 &v, int lane, int64_t e0, bool live,
                                                  int8_t *__restrict__ qs, float *__restrict__ d,
-                                                 int32_t *__restrict__ isum, uint16_t *__restrict__ msum) {
+                                                 int32_t *__restrict__ isum) {
     int s;
     float dd;
     const uint32_t packed = wave_quantize_q8_32(v, s, dd);
@@ -133,16 +124,15 @@ __device__ __forceinline__ void wave_store_q8_32(const float4 &v, int lane, int6
     if ((lane & 7) == 0) {
         const int64_t b = e0 >> 5;
         d[b] = FP16_SCALE ? h2f(f2h(dd)) : dd;
-        if (!FP16_SCALE) {
-            isum[b] = s;
-            const float t = dd * (float)s * kMinPrescale;
-            const _Float16 hi = (_Float16)t, lo = (_Float16)(t - (float)hi);
-            msum[ch * 16 + (lane >> 3)] = __builtin_bit_cast(uint16_t, hi);
-            msum[ch * 16 + 8 + (lane >> 3)] = __builtin_bit_cast(uint16_t, lo);
-        }
+        if (!FP16_SCALE) isum[b] = s;
     }
 }
 
+// The largest power of two not above v (v > 0 and normal), 1 for v = 0 or a subnormal.
+__device__ __forceinline__ float pow2_floor(float v) {
+    const uint32_t e = __float_as_uint(v) & 0x7f800000u;
+    return e ? __uint_as_float(e) : 1.0f;
+}
 
 // Sum of squares of a row spread over a workgroup of 16 waves in ggml's precision (float products summed in
 // double).  The order is fixed - lane's own pieces, butterfly over the wave, waves 0..15 - so that every

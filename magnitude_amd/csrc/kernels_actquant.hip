@@ -8,12 +8,12 @@ namespace qproj {
 
 __global__ __launch_bounds__(256) void quant_q8k_kernel(const float *__restrict__ x, int64_t n_super,
                                                         int8_t *__restrict__ qs, float *__restrict__ d,
-                                                        int16_t *__restrict__ bsums, uint16_t *__restrict__ msum) {
+                                                        int16_t *__restrict__ bsums) {
     const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (sb >= n_super) return;  // whole wave leaves together
     const float4 v = reinterpret_cast<const float4 *>(x + sb * 256)[lane];
-    wave_store_q8k(v, lane, sb, qs, d, bsums, msum);
+    wave_store_q8k(v, lane, sb, qs, d, bsums);
 }
 
 // FP16_SCALE: ggml Q8_0 blocks (scale rounded through fp16).  Otherwise the prefill format:
@@ -21,8 +21,7 @@ __global__ __launch_bounds__(256) void quant_q8k_kernel(const float *__restrict_
 template <bool FP16_SCALE>
 __global__ __launch_bounds__(256) void quant_q8_32_kernel(const float *__restrict__ x, int64_t n_chunks256,
                                                           int64_t n_elems, int8_t *__restrict__ qs,
-                                                          float *__restrict__ d, int32_t *__restrict__ isum,
-                                                          uint16_t *__restrict__ msum) {
+                                                          float *__restrict__ d, int32_t *__restrict__ isum) {
     const int64_t ch = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (ch >= n_chunks256) return;
@@ -30,26 +29,95 @@ __global__ __launch_bounds__(256) void quant_q8_32_kernel(const float *__restric
     const bool live = e0 < n_elems;  // rows are multiples of 32, so a block is all in or all out
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (live) v = *reinterpret_cast<const float4 *>(x + e0);
-    wave_store_q8_32<FP16_SCALE>(v, lane, e0, ch, live, qs, d, isum, msum);
+    wave_store_q8_32<FP16_SCALE>(v, lane, e0, live, qs, d, isum);
 }
 
+// The min-term operand of the tiled Q4_K kernels, one wave per activation row, after the row's blocks are quantized.
+// For every 32-wide sub-block the kernels want d * (sum of its 32 codes) as an fp16 high / low pair (22 bits).  fp16
+// has a narrow range, so the values are normalised by the row: rs[m] = the largest power of two not above the
+// row's largest block scale, and the pair holds (d / rs[m]) * sum / 16 -- at most 2 * 4064 / 16 whatever the size of
+// the activations; a block far below the row's largest loses bits only where they no longer matter to the row.
+// The kernels scale the activation scales by 1 / rs[m] and the result by 16 * rs[m], both exact.
+// Per super-block: eight high parts, then eight low parts (the order the fp16 matrix instruction is fed).
+// PER32: scales and sums per 32-block (d [K/32], isum [K/32]); otherwise per 256 (d [K/256], bsums [K/16]).
+template <bool PER32>
+__global__ __launch_bounds__(256) void minterm_rows_kernel(const float *__restrict__ d, const int16_t *__restrict__ bsums,
+                                                           const int32_t *__restrict__ isum, int64_t M, int nb,
+                                                           uint16_t *__restrict__ msum, float *__restrict__ rs) {
+    const int64_t m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (m >= M) return;   // whole wave leaves together
+    const int nd = PER32 ? nb * 8 : nb;   // scales of the row
+    const float *dr = d + m * nd;
+    float dmax = 0.f;
+    for (int i = lane; i < nd; i += 64) dmax = fmaxf(dmax, fabsf(dr[i]));   // a Q8_K scale carries a sign
+    dmax = wave_max(dmax);
+    const float r = pow2_floor(dmax), inv = 1.0f / r;   // exact: a power of two
+    if (lane == 0) rs[m] = r;
+    for (int sb = lane; sb < nb; sb += 64) {
+        uint32_t hi[4], lo[4];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            float dd;
+            int sum;
+            if (PER32) {
+                dd = dr[sb * 8 + t];
+                sum = isum[(m * nb + sb) * 8 + t];
+            } else {
+                dd = dr[sb];
+                const int16_t *b = bsums + (m * nb + sb) * 16 + 2 * t;
+                sum = (int)b[0] + (int)b[1];
+            }
+            const float v = (dd * inv) * (float)sum * kMinPrescale;
+            const _Float16 h = (_Float16)v, l = (_Float16)(v - (float)h);
+            const uint32_t hb = __builtin_bit_cast(uint16_t, h), lb = __builtin_bit_cast(uint16_t, l);
+            if (t & 1) {
+                hi[t >> 1] |= hb << 16;
+                lo[t >> 1] |= lb << 16;
+            } else {
+                hi[t >> 1] = hb;
+                lo[t >> 1] = lb;
+            }
+        }
+        uint4 *dst = reinterpret_cast<uint4 *>(msum + (m * nb + sb) * 16);
+        dst[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        dst[1] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    }
+}
+
+hipError_t launch_minterm_rows(int kind, const float *d, const int16_t *bsums, const int32_t *isum, int64_t M, int64_t K,
+                               uint16_t *msum, float *rs, hipStream_t s) {
+    if (M == 0) return hipSuccess;
+    if (K % 256 != 0 || !msum || !rs || (kind != kActKindQ8_K && kind != kActKindQ8X32)) return hipErrorInvalidValue;
+    if (dry_run()) return hipSuccess;
+    const dim3 grid((unsigned)((M + 3) / 4)), block(256);
+    if (kind == kActKindQ8_K)
+        hipLaunchKernelGGL(minterm_rows_kernel<false>, grid, block, 0, s, d, bsums, isum, M, (int)(K / 256), msum, rs);
+    else
+        hipLaunchKernelGGL(minterm_rows_kernel<true>, grid, block, 0, s, d, bsums, isum, M, (int)(K / 256), msum, rs);
+    return hipGetLastError();
+}
+
+// msum / rs null: the min-term plane is not wanted (the decode, small-batch and expert-grouped kernels take the block
+// sums themselves)
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
-                               int16_t *bsums, uint16_t *msum, int32_t *isum, hipStream_t s) {
+                               int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s) {
     const int64_t n = M * K;
     if (n == 0) return hipSuccess;
-    if (dry_run()) return kind == kActKindQ8_K || kind == kActKindQ8_0 || kind == kActKindQ8X32 ? hipSuccess : hipErrorInvalidValue;
+    if (kind != kActKindQ8_K && kind != kActKindQ8_0 && kind != kActKindQ8X32) return hipErrorInvalidValue;
+    if (dry_run()) return hipSuccess;
     const int64_t chunks = (n + 255) / 256;
     const dim3 grid((unsigned)((chunks + 3) / 4)), block(256);
     if (kind == kActKindQ8_K) {
-        hipLaunchKernelGGL(quant_q8k_kernel, grid, block, 0, s, x, n / 256, qs, d, bsums, msum);
+        hipLaunchKernelGGL(quant_q8k_kernel, grid, block, 0, s, x, n / 256, qs, d, bsums);
     } else if (kind == kActKindQ8_0) {
-        hipLaunchKernelGGL(quant_q8_32_kernel<true>, grid, block, 0, s, x, chunks, n, qs, d, isum, msum);
-    } else if (kind == kActKindQ8X32) {
-        hipLaunchKernelGGL(quant_q8_32_kernel<false>, grid, block, 0, s, x, chunks, n, qs, d, isum, msum);
+        hipLaunchKernelGGL(quant_q8_32_kernel<true>, grid, block, 0, s, x, chunks, n, qs, d, isum);
     } else {
-        return hipErrorInvalidValue;
+        hipLaunchKernelGGL(quant_q8_32_kernel<false>, grid, block, 0, s, x, chunks, n, qs, d, isum);
     }
-    return hipGetLastError();
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || kind == kActKindQ8_0 || !msum) return e;
+    return launch_minterm_rows(kind, d, bsums, isum, M, K, msum, rs, s);
 }
 
 }  // namespace qproj

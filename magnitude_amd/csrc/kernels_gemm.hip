@@ -171,12 +171,20 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const Weigh
                 al = al_n;
             }
         }
-        const float inv = 1.0f / kMinPrescale;
+        // the operand was normalised by the row (rs[m], a power of two) and pre-scaled by 1/16: both undone exactly
+        __syncthreads();   // the planes have been read
+        float *rs_tile = reinterpret_cast<float *>(smem_raw);   // the tile's 128 row normalisers, times 16
+        if (tid < BM) rs_tile[tid] = a.rs[m0 + tid < M ? m0 + tid : M - 1] * (1.0f / kMinPrescale);
+        __syncthreads();
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int g = 0; g < 4; ++g) {
+            const float4 f = *reinterpret_cast<const float4 *>(rs_tile + wm * 32 + 8 * g + 4 * lh);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][v] *= inv;
-        __syncthreads();   // the planes have been read: the main loop may overwrite them
+            for (int j = 0; j < 2; ++j) {
+                acc[j][4 * g] *= f.x; acc[j][4 * g + 1] *= f.y; acc[j][4 * g + 2] *= f.z; acc[j][4 * g + 3] *= f.w;
+            }
+        }
+        __syncthreads();   // the main loop may overwrite the tile
     }
 
     // ---------------------------------------------------------------- main loop, int8 cores
@@ -445,6 +453,10 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const D
     const uint32_t msoffg = (uint32_t)((msrow < mrow_cap ? msrow : mrow_cap) * (int)nb * 32 + 16 * (tid & 1));
     const float *dxbase = a.d + m0 * nb;
     const uint32_t dxoffg = (uint32_t)(((tid & 63) < mrow_cap ? (tid & 63) : mrow_cap) * (int)nb);
+    // the min-term operand is normalised by the row (rs[m], a power of two): the accumulators run in units of
+    // 1 / (16 * rs[m]) until the store, so the activation scales are divided by rs[m] as they are staged (exact)
+    const float rs_mine = a.rs[m0 + ((tid & 63) < mrow_cap ? (tid & 63) : mrow_cap)];
+    const float inv_rs = 1.0f / rs_mine;
 
     v4i stg[5], areg[PA], msreg;
     float dxreg;
@@ -462,7 +474,7 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const D
         for (int p = 0; p < PA; ++p) *reinterpret_cast<v4i *>(sm.a[buf] + aoffl[p]) = areg[p];
         // threads beyond the first 128 / 64 repeat a store of the same value: no branch, no load sunk into one
         *reinterpret_cast<v4i *>(reinterpret_cast<uint8_t *>(sm.ms[buf]) + 16 * (tid & 127)) = msreg;
-        sm.dx[buf][tid & 63] = dxreg;
+        sm.dx[buf][tid & 63] = dxreg * inv_rs;   // (here, not at the load: nothing waits for the load before it must)
 #pragma unroll
         for (int c = 0; c < 5; ++c) *reinterpret_cast<v4i *>(park + wpark[c]) = stg[c];
     };
@@ -551,14 +563,21 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const D
 
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
     const int64_t n = n0 + wave * 32 + l32;
-    const float inv = 1.0f / kMinPrescale;
+    // the rows' factors (normaliser / 16) go through the idle scale buffer: four rows per read, no load per store
+    sm.dx[0][tid & 63] = rs_mine * (1.0f / kMinPrescale);
+    __syncthreads();
     float *out = gridDim.y > 1 ? part + (size_t)blockIdx.y * M * N : y;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < M && n < N) out[m * N + n] = acc[j][v] * inv;
+        for (int g = 0; g < 4; ++g) {
+            const float4 f4 = *reinterpret_cast<const float4 *>(&sm.dx[0][j * 32 + 8 * g + 4 * lh]);
+            const float f[4] = {f4.x, f4.y, f4.z, f4.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t m = m0 + j * 32 + 8 * g + 4 * lh + r;
+                if (m < M && n < N) out[m * N + n] = acc[j][4 * g + r] * f[r];
+            }
         }
     }
 }
@@ -635,6 +654,10 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
     const uint32_t msoffg = (uint32_t)((mstok < mrow_cap ? mstok : mrow_cap) * (int)nb * 32 + 16 * (lane & 1));
     const float *dxbase = a.d + m0 * nb;
     const uint32_t dxoffg = (uint32_t)((dxtok < mrow_cap ? dxtok : mrow_cap) * (int)nb);
+    // the min-term operand is normalised by the row (rs[m], a power of two): the accumulators run in units of
+    // 1 / (16 * rs[m]) until the store, so the activation scales are divided by rs[m] as they are staged (exact)
+    const float rs_mine = a.rs[m0 + (dxtok < mrow_cap ? dxtok : mrow_cap)];
+    const float inv_rs = 1.0f / rs_mine;
     uint8_t *park = sm.park[wave];
 
     // Addresses are a scalar base that never moves plus a 32-bit lane offset to which the super-block's
@@ -691,7 +714,7 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
 #pragma unroll
     for (int p = 0; p < PA; ++p) request_act((uint32_t)sb_begin, 0, p);
     request_ms((uint32_t)sb_begin, 0);
-    sm.dx[0][tid & 127] = dxbase_s[dxoffg + (uint32_t)sb_begin];
+    sm.dx[0][tid & 127] = dxbase_s[dxoffg + (uint32_t)sb_begin] * inv_rs;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
@@ -796,7 +819,7 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
 #pragma unroll
                 for (int t = 0; t < 8; ++t) convert(t, strip_piece(t));
             }
-            sm.dx[buf ^ 1][tid & 127] = dxreg;   // every thread stores (a repeated value past 128): no branch
+            sm.dx[buf ^ 1][tid & 127] = dxreg * inv_rs;   // every thread stores (a repeated value past 128): no branch
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             __syncthreads();
         }
@@ -806,14 +829,21 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
 
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
     const int64_t n = n0 + wave * 32 + l32;
-    const float inv = 1.0f / kMinPrescale;
+    // the rows' factors (normaliser / 16) go through the idle scale buffer: four rows per read, no load per store
+    sm.dx[0][tid & 127] = rs_mine * (1.0f / kMinPrescale);
+    __syncthreads();
     float *out = gridDim.y > 1 ? part + (size_t)blockIdx.y * M * N : y;
 #pragma unroll
     for (int j = 0; j < JT; ++j) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < M && n < N) out[m * N + n] = acc[j][v] * inv;
+        for (int g = 0; g < 4; ++g) {
+            const float4 f4 = *reinterpret_cast<const float4 *>(&sm.dx[0][j * 32 + 8 * g + 4 * lh]);
+            const float f[4] = {f4.x, f4.y, f4.z, f4.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t m = m0 + j * 32 + 8 * g + 4 * lh + r;
+                if (m < M && n < N) out[m * N + n] = acc[j][4 * g + r] * f[r];
+            }
         }
     }
 }
@@ -896,7 +926,7 @@ size_t per32_scratch_bytes(int64_t K, int64_t M, int64_t N) {
 }
 
 hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s) {
-    if (w.type != kTypeQ4_K || w.K % 256 != 0 || M <= 0 || !a.msum) return hipErrorInvalidValue;
+    if (w.type != kTypeQ4_K || w.K % 256 != 0 || M <= 0 || !a.msum || !a.rs) return hipErrorInvalidValue;
     return launch_per32<kTypeQ4_K>(w, a, M, y, scratch, s);
 }
 
@@ -935,7 +965,7 @@ size_t q4k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N) {
 
 // ggml-format activations (Q8_K planes in `a`, including the min-term plane), Q4_K weights, any M
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s) {
-    if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || !a.msum || M <= 0) return hipErrorInvalidValue;
+    if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || !a.msum || !a.rs || M <= 0) return hipErrorInvalidValue;
     if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 128 token rows of K bytes, 32 weight rows of K*144/256
     const Q4Plan p = q4k_plan(w.K, M, w.N, scratch.p != nullptr);
     if (p.n_split > 1 && (size_t)p.n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
@@ -975,7 +1005,7 @@ hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, i
     static const bool off = tuning_int("QPROJ_Q8K_NO_MULTI", 0) != 0;
     // the matrices that would take the 64-token kernel with K in one stretch go together; the others (128-token
     // tiles, K cut into stretches) get their own launches first
-    const bool can = !off && n >= 2 && n <= 3 && wide_env < 0 && a.kind == kActKindQ8_K && a.msum && M > 0;
+    const bool can = !off && n >= 2 && n <= 3 && wide_env < 0 && a.kind == kActKindQ8_K && a.msum && a.rs && M > 0;
     int joined[3], n_joined = 0;
     for (int i = 0; i < n; ++i) {
         const Q4Plan p = q4k_plan(w[i].K, M, w[i].N, scratch.p != nullptr);

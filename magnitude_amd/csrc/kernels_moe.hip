@@ -157,7 +157,7 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
         if (sb < job.n_super) {   // whole wave decides together
             const int lane = threadIdx.x & 63;
             const float4 v = reinterpret_cast<const float4 *>(job.x + sb * 256)[lane];
-            wave_store_q8k(v, lane, sb, job.qs, job.d, job.bsums, job.msum);
+            wave_store_q8k(v, lane, sb, job.qs, job.d, job.bsums);
         }
         return;
     }

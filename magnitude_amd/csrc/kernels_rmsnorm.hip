@@ -26,8 +26,7 @@ template <int MODE>
 __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                                 float eps, int64_t K, float *__restrict__ y,
                                                                 int8_t *__restrict__ qs, float *__restrict__ d,
-                                                                int16_t *__restrict__ bsums, uint16_t *__restrict__ msum,
-                                                                int32_t *__restrict__ isum) {
+                                                                int16_t *__restrict__ bsums, int32_t *__restrict__ isum) {
     __shared__ double partial[kNormWaves];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t row = blockIdx.x;
@@ -73,38 +72,32 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const float *__r
         if (MODE == 0) {
             if (live) *reinterpret_cast<float4 *>(y + row * K + e0) = v;
         } else if (MODE == 1) {   // K is a multiple of 256 here: every piece is whole
-            wave_store_q8k(v, lane, row * (K / 256) + p, qs, d, bsums, msum);
+            wave_store_q8k(v, lane, row * (K / 256) + p, qs, d, bsums);
         } else {
-            // the planes are indexed by the flattened element: row * K is a multiple of 32, and of 256 whenever
-            // the msum plane exists (MODE 3 needs K % 256 == 0)
-            wave_store_q8_32<MODE == 2>(v, lane, row * K + e0, (row * K + e0) >> 8, live, qs, d, isum, msum);
+            // the planes are indexed by the flattened element: row * K is a multiple of 32
+            wave_store_q8_32<MODE == 2>(v, lane, row * K + e0, live, qs, d, isum);
         }
     }
 }
 
 }  // namespace
 
-// y (fp32) when kind < 0, otherwise the activation planes of `kind`
+// y (fp32) when kind < 0, otherwise the activation planes of `kind` (msum / rs null: no min-term plane wanted)
 hipError_t launch_rms_norm(int kind, const float *x, const float *gamma, float eps, int64_t M, int64_t K, float *y,
-                           int8_t *qs, float *d, int16_t *bsums, uint16_t *msum, int32_t *isum, hipStream_t s) {
+                           int8_t *qs, float *d, int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s) {
     if (M == 0) return hipSuccess;
     if (K <= 0 || K % 32 != 0) return hipErrorInvalidValue;
+    if ((kind == kActKindQ8_K || kind == kActKindQ8X32) && K % 256 != 0) return hipErrorInvalidValue;
+    if (kind >= 0 && kind != kActKindQ8_K && kind != kActKindQ8_0 && kind != kActKindQ8X32) return hipErrorInvalidValue;
     if (dry_run()) return hipSuccess;
     const dim3 grid((unsigned)M), block(kNormThreads);
-    if (kind < 0) {
-        hipLaunchKernelGGL(rms_norm_kernel<0>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, msum, isum);
-    } else if (kind == kActKindQ8_K) {
-        if (K % 256 != 0) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(rms_norm_kernel<1>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, msum, isum);
-    } else if (kind == kActKindQ8_0) {
-        hipLaunchKernelGGL(rms_norm_kernel<2>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, msum, isum);
-    } else if (kind == kActKindQ8X32) {
-        if (K % 256 != 0) return hipErrorInvalidValue;
-        hipLaunchKernelGGL(rms_norm_kernel<3>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, msum, isum);
-    } else {
-        return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
+    if (kind < 0) hipLaunchKernelGGL(rms_norm_kernel<0>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum);
+    else if (kind == kActKindQ8_K) hipLaunchKernelGGL(rms_norm_kernel<1>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum);
+    else if (kind == kActKindQ8_0) hipLaunchKernelGGL(rms_norm_kernel<2>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum);
+    else hipLaunchKernelGGL(rms_norm_kernel<3>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess || kind < 0 || kind == kActKindQ8_0 || !msum) return e;
+    return launch_minterm_rows(kind, d, bsums, isum, M, K, msum, rs, s);
 }
 
 }  // namespace qproj

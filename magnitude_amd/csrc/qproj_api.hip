@@ -155,7 +155,7 @@ int ensure_ws2(qproj_ctx *ctx, size_t bytes) {
 
 // planes of a quantized-activation buffer, in the order the header documents
 struct ActPlanes {
-    size_t off_qs = 0, off_d = 0, off_aux = 0, off_msum = 0, total = 0;
+    size_t off_qs = 0, off_d = 0, off_aux = 0, off_msum = 0, off_rs = 0, total = 0;
     int kind = 0;
 };
 
@@ -175,7 +175,9 @@ ActPlanes act_planes(int kind, int64_t M, int64_t K) {
     if (kind == kActKindQ8_K) aux = (size_t)(M * (K / 16)) * 2;
     if (kind == kActKindQ8X32) aux = (size_t)(M * (K / 32)) * 4;
     p.off_msum = p.off_aux + align_up(aux);
-    p.total = p.off_msum + (kind == kActKindQ8_K || kind == kActKindQ8X32 ? align_up((size_t)(M * (K / 256)) * 32) : 0);
+    const bool minterm = kind == kActKindQ8_K || kind == kActKindQ8X32;
+    p.off_rs = p.off_msum + (minterm ? align_up((size_t)(M * (K / 256)) * 32) : 0);
+    p.total = p.off_rs + (minterm ? align_up((size_t)M * 4) : 0);
     return p;
 }
 
@@ -188,6 +190,7 @@ ActView act_view(const ActPlanes &p, uint8_t *base, int64_t K) {
     a.bsums = p.kind == kActKindQ8_K ? reinterpret_cast<const int16_t *>(base + p.off_aux) : nullptr;
     a.msum = p.kind == kActKindQ8_K || p.kind == kActKindQ8X32 ? reinterpret_cast<const uint16_t *>(base + p.off_msum) : nullptr;
     a.isum = p.kind == kActKindQ8X32 ? reinterpret_cast<const int32_t *>(base + p.off_aux) : nullptr;
+    a.rs = a.msum ? reinterpret_cast<const float *>(base + p.off_rs) : nullptr;
     return a;
 }
 
@@ -199,16 +202,19 @@ RowQuantJob quantize_job(const ActPlanes &p, uint8_t *base, const float *x, int6
     j.qs = reinterpret_cast<int8_t *>(base + p.off_qs);
     j.d = reinterpret_cast<float *>(base + p.off_d);
     j.bsums = reinterpret_cast<int16_t *>(base + p.off_aux);
-    j.msum = reinterpret_cast<uint16_t *>(base + p.off_msum);
     return j;
 }
 
-hipError_t run_quantize(qproj_ctx *ctx, const ActPlanes &p, uint8_t *base, const float *x, int64_t M, int64_t K) {
+// minterm: also the min-term plane and the row normalisers that only the tiled Q4_K kernels read (a second, small launch)
+hipError_t run_quantize(qproj_ctx *ctx, const ActPlanes &p, uint8_t *base, const float *x, int64_t M, int64_t K,
+                        bool minterm = true) {
+    const bool mt = minterm && (p.kind == kActKindQ8_K || p.kind == kActKindQ8X32);
     return launch_quantize_act(p.kind, x, M, K, reinterpret_cast<int8_t *>(base + p.off_qs),
                                reinterpret_cast<float *>(base + p.off_d),
                                reinterpret_cast<int16_t *>(base + p.off_aux),
-                               reinterpret_cast<uint16_t *>(base + p.off_msum),
-                               reinterpret_cast<int32_t *>(base + p.off_aux), ctx->stream);
+                               mt ? reinterpret_cast<uint16_t *>(base + p.off_msum) : nullptr,
+                               reinterpret_cast<int32_t *>(base + p.off_aux),
+                               mt ? reinterpret_cast<float *>(base + p.off_rs) : nullptr, ctx->stream);
 }
 
 ActView act_rows(const ActView &a, int64_t m0) {
@@ -218,6 +224,7 @@ ActView act_rows(const ActView &a, int64_t m0) {
     r.d = a.d + m0 * (a.K / dblk);
     if (a.bsums) r.bsums = a.bsums + m0 * (a.K / 16);
     if (a.msum) r.msum = a.msum + m0 * (a.K / 16);
+    if (a.rs) r.rs = a.rs + m0;
     if (a.isum) r.isum = a.isum + m0 * (a.K / 32);
     return r;
 }
@@ -728,7 +735,7 @@ int qproj_rms_norm(qproj_ctx *ctx, const float *x_dev, const float *gamma_dev, f
     if (!x_dev || !y_dev) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_rms_norm: null argument");
     if (M < 0 || K <= 0 || K % 32 != 0) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_rms_norm: K must be a positive multiple of 32");
     QP_HIP(ctx, hipSetDevice(ctx->device));
-    QP_HIP(ctx, launch_rms_norm(-1, x_dev, gamma_dev, eps, M, K, y_dev, nullptr, nullptr, nullptr, nullptr, nullptr, ctx->stream));
+    QP_HIP(ctx, launch_rms_norm(-1, x_dev, gamma_dev, eps, M, K, y_dev, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, ctx->stream));
     return QPROJ_OK;
 }
 
@@ -744,10 +751,12 @@ int qproj_rms_norm_quantize(qproj_ctx *ctx, int kind, int wtype, const float *x_
     QP_HIP(ctx, hipSetDevice(ctx->device));
     const ActPlanes p = act_planes(k, M, K);
     uint8_t *base = static_cast<uint8_t *>(out_dev);
+    const bool mt = k == kActKindQ8_K || k == kActKindQ8X32;
     QP_HIP(ctx, launch_rms_norm(k, x_dev, gamma_dev, eps, M, K, nullptr, reinterpret_cast<int8_t *>(base + p.off_qs),
                                 reinterpret_cast<float *>(base + p.off_d), reinterpret_cast<int16_t *>(base + p.off_aux),
-                                reinterpret_cast<uint16_t *>(base + p.off_msum),
-                                reinterpret_cast<int32_t *>(base + p.off_aux), ctx->stream));
+                                mt ? reinterpret_cast<uint16_t *>(base + p.off_msum) : nullptr,
+                                reinterpret_cast<int32_t *>(base + p.off_aux),
+                                mt ? reinterpret_cast<float *>(base + p.off_rs) : nullptr, ctx->stream));
     return QPROJ_OK;
 }
 
@@ -808,16 +817,19 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
         int rc = reserve(ctx, wsp, p.total + extra);
         if (rc) return rc;
         uint8_t *ws = wsp.base;
+        // the min-term plane (a second small launch, one wave a row) only where a tiled Q4_K kernel will read it
+        const bool minterm = act == kActQ8X32 || (w[0]->type == kTypeQ4_K && takes_tiled(w[0], M));
         if (norm) {   // norm, weights and quantizer in one launch
             if (p.kind == kActKindQ8X32 && K % 256 != 0)
                 return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_rms_norm_mul_mat: the per-32 format needs K % 256 == 0");
             QP_HIP(ctx, launch_rms_norm(p.kind, x_dev, norm->gamma, norm->eps, M, K, nullptr,
                                         reinterpret_cast<int8_t *>(ws + p.off_qs), reinterpret_cast<float *>(ws + p.off_d),
                                         reinterpret_cast<int16_t *>(ws + p.off_aux),
-                                        reinterpret_cast<uint16_t *>(ws + p.off_msum),
-                                        reinterpret_cast<int32_t *>(ws + p.off_aux), ctx->stream));
+                                        minterm ? reinterpret_cast<uint16_t *>(ws + p.off_msum) : nullptr,
+                                        reinterpret_cast<int32_t *>(ws + p.off_aux),
+                                        minterm ? reinterpret_cast<float *>(ws + p.off_rs) : nullptr, ctx->stream));
         } else {
-            QP_HIP(ctx, run_quantize(ctx, p, ws, x_dev, M, K));
+            QP_HIP(ctx, run_quantize(ctx, p, ws, x_dev, M, K, minterm));
         }
         const ActView a = act_view(p, ws, K);
         // the partial results lie behind the activation planes; `extra` is all a launcher may use of it
@@ -831,7 +843,7 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
             int rc = reserve(ctx, wsp, (size_t)M * K * 4);
             if (rc) return rc;
             QP_HIP(ctx, launch_rms_norm(-1, x_dev, norm->gamma, norm->eps, M, K, reinterpret_cast<float *>(wsp.base), nullptr,
-                                        nullptr, nullptr, nullptr, nullptr, ctx->stream));
+                                        nullptr, nullptr, nullptr, nullptr, nullptr, ctx->stream));
             x_dev = reinterpret_cast<const float *>(wsp.base);
         }
         for (int64_t m0 = 0; m0 < M; m0 += 4) {
@@ -1047,7 +1059,7 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     // the quantizer and the grouping pass read only the call's inputs: one launch carries both
     const bool joined = !fuse && !pair_mode && p.kind == kActKindQ8_K;
     const RowQuantJob job = quantize_job(p, ctx->ws, x_dev, rows, K);
-    if (!fuse && !joined) QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, rows, K));
+    if (!fuse && !joined) QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, rows, K, false));
     if (!pair_mode)
         QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, w->E, order, offsets, active, ctx->flag_dev,
                                      joined ? &job : nullptr, ctx->stream));
@@ -1121,7 +1133,7 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     // the quantizer of x and the grouping pass read only the call's inputs: one launch carries both
     const bool joined = !fuse_x && !pair_mode && px.kind == kActKindQ8_K;
     const RowQuantJob job = quantize_job(px, ws, x_dev, B, d_model);
-    if (!fuse_x && !joined) QP_HIP(ctx, run_quantize(ctx, px, ws, x_dev, B, d_model));
+    if (!fuse_x && !joined) QP_HIP(ctx, run_quantize(ctx, px, ws, x_dev, B, d_model, false));
     if (!pair_mode)
         QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, E, order, offsets, active, ctx->flag_dev,
                                      joined ? &job : nullptr, ctx->stream));
@@ -1146,7 +1158,7 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
         QP_HIP(ctx, launch_gemv_mfma_grouped(g, n_pairs, true, ctx->stream));
     else
         QP_HIP(ctx, launch_moe_swiglu_gemv(g, mt, (int)E, ctx->stream));
-    if (!fuse_h) QP_HIP(ctx, run_quantize(ctx, ph, ws + off_hq, h, n_pairs, d_ff));
+    if (!fuse_h) QP_HIP(ctx, run_quantize(ctx, ph, ws + off_hq, h, n_pairs, d_ff, false));
     GemvArgs gd{};
     if (pair_mode) {
         gd.ids = ids_dev;

@@ -41,11 +41,12 @@ struct ActView {
     const int8_t *qs;      // [rows][K]
     const float *d;        // [rows][K/32] (Q8_0, Q8X32) or [rows][K/256] (Q8_K)
     const int16_t *bsums;  // Q8_K: [rows][K/16]
-    const uint16_t *msum;  // Q8_K, Q8X32: [rows][K/256][16] fp16: d * (sum of 32 codes) * kMinPrescale for the 8
+    const uint16_t *msum;  // Q8_K, Q8X32: [rows][K/256][16] fp16: (d / rs[row]) * (sum of 32 codes) * kMinPrescale for the 8
                            //       sub-blocks, high parts, then the 8 low parts (v - high); prefill min term
     const int32_t *isum;   // Q8X32: [rows][K/32]
+    const float *rs;       // Q8_K, Q8X32: [rows] the power of two the row's msum entries are normalised by
 };
-constexpr float kMinPrescale = 0.0625f;  // keeps d * sum inside fp16 range for |x| up to ~1e5
+constexpr float kMinPrescale = 0.0625f;  // (d / rs) * sum / 16 <= 2 * 4064 / 16: well inside fp16 whatever the activations
 constexpr int kActKindQ8_0 = 0;
 constexpr int kActKindQ8_K = 1;
 constexpr int kActKindQ8X32 = 2;
@@ -107,10 +108,14 @@ hipError_t launch_repack_to_planes(int type, const uint8_t *gguf, uint8_t *plane
                                    int64_t n_blocks, hipStream_t s);
 hipError_t launch_repack_to_gguf(int type, const WeightView &w, uint8_t *gguf, int64_t n_blocks, hipStream_t s);
 // RMS_NORM + MUL by the norm weights (gamma may be null); kind < 0: fp32 rows to y, otherwise the planes of `kind`
+// (msum and rs may be null together: the min-term plane of the tiled Q4_K kernels is then not made)
 hipError_t launch_rms_norm(int kind, const float *x, const float *gamma, float eps, int64_t M, int64_t K, float *y,
-                           int8_t *qs, float *d, int16_t *bsums, uint16_t *msum, int32_t *isum, hipStream_t s);
+                           int8_t *qs, float *d, int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s);
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
-                               int16_t *bsums, uint16_t *msum, int32_t *isum, hipStream_t s);
+                               int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s);
+// the min-term plane and the row normalisers from planes already quantized (one wave per row)
+hipError_t launch_minterm_rows(int kind, const float *d, const int16_t *bsums, const int32_t *isum, int64_t M, int64_t K,
+                               uint16_t *msum, float *rs, hipStream_t s);
 hipError_t launch_gemv_q8act(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
 // persistent decode kernel (mt <= 4 rows); fuse_quantize: args.x holds fp32 rows, else args.a
 bool decode_kernel_fits(int type, int mt, int64_t K);
@@ -134,7 +139,6 @@ struct RowQuantJob {
     int8_t *qs;
     float *d;
     int16_t *bsums;
-    uint16_t *msum;
 };
 hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_expert, int32_t *order,
                             int32_t *offsets, int32_t *active, int32_t *error_flag, const RowQuantJob *quantize,

@@ -274,10 +274,14 @@ class Context:
             out["bsums"] = buf[off_aux:off_aux + m * (k // 16) * 2].view(torch.int16).view(m, k // 16)
             off_ms = off_aux + al(m * (k // 16) * 2)
             out["msum"] = buf[off_ms:off_ms + m * (k // 256) * 32].view(torch.float16).view(m, k // 256, 2, 8)
+            off_rs = off_ms + al(m * (k // 256) * 32)
+            out["rs"] = buf[off_rs:off_rs + m * 4].view(torch.float32)
         elif kind == ACT_Q8X32:
             out["isum"] = buf[off_aux:off_aux + m * (k // 32) * 4].view(torch.int32).view(m, k // 32)
             off_ms = off_aux + al(m * (k // 32) * 4)
             out["msum"] = buf[off_ms:off_ms + m * (k // 256) * 32].view(torch.float16).view(m, k // 256, 2, 8)
+            off_rs = off_ms + al(m * (k // 256) * 32)
+            out["rs"] = buf[off_rs:off_rs + m * 4].view(torch.float32)
         return out
 
     # ---- operators -----------------------------------------------------------------------

@@ -36,9 +36,9 @@ def test_version_and_sizes(lib):
     assert lib.qproj_row_bytes(12, 4100) == 0
     assert lib.qproj_row_bytes(2, 4096) == 0      # Q4_0 is not a type this path carries
     # activation buffer sizes: planes are 256-byte aligned
-    assert lib.qproj_act_bytes(0, 12, 1, 4096) == 4096 + 256 + 512 + 512   # qs | d | bsums | fp16 min-term plane
+    assert lib.qproj_act_bytes(0, 12, 1, 4096) == 4096 + 256 + 512 + 512 + 256   # qs | d | bsums | fp16 min-term plane | row normalisers
     assert lib.qproj_act_bytes(0, 8, 1, 4096) == 4096 + 512
-    assert lib.qproj_act_bytes(2, 12, 2, 4096) == 8192 + 1024 + 1024 + 1024   # qs | d | isum | fp16 min-term plane
+    assert lib.qproj_act_bytes(2, 12, 2, 4096) == 8192 + 1024 + 1024 + 1024 + 256   # qs | d | isum | fp16 min-term plane | row normalisers
     assert lib.qproj_act_bytes(0, 12, 1, 4000) == 0
     assert lib.qproj_act_bytes(1, 12, 1, 4096) == 0  # fp32 activations are not quantized
     # the per-32 format keeps one min-term record per 256 weights of a row: K must be whole super-blocks, or the

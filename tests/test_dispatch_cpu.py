@@ -49,7 +49,7 @@ def test_per32_and_fp32_modes():
 
 def test_known_sizes():
     al = lambda v: (v + 255) // 256 * 256
-    planes = lambda m, k: al(m * k) + al(m * (k // 256) * 4) + al(m * (k // 16) * 2) + al(m * (k // 256) * 32)
+    planes = lambda m, k: al(m * k) + al(m * (k // 256) * 4) + al(m * (k // 16) * 2) + al(m * (k // 256) * 32) + al(m * 4)
     # down projection of the 8B layer at 512 tokens: 64 tiles of 128 tokens x 256 rows for 256 compute units, K is cut in four
     assert qproj.workspace_bytes(Q6_K, 14336, (4096,), 512, GGML) == planes(512, 14336) + 4 * 512 * 4096 * 4
     # gate/up at 4096 tokens: the grid is full, nothing beyond the activation planes

@@ -161,9 +161,13 @@ def test_quantize_q8_K_bit_exact(ctx, orc):
     assert np.array_equal(got["qs"].cpu().numpy(), want_q)
     assert np.array_equal(got["d"].cpu().numpy().view(np.uint32), want_d.view(np.uint32))
     assert np.array_equal(got["bsums"].cpu().numpy(), want_b)
-    # the prefill kernel's extra plane: d * (sum of each 32 codes) / 16, as an fp16 high part and
-    # the fp16 of what the high part leaves (numpy's float16 rounds to nearest even like the device)
-    v = want_d[:, :, None] * want_b.reshape(m, k // 256, 8, 2).sum(-1).astype(np.float32) * np.float32(0.0625)
+    # the tiled kernels' extra planes: rs = the largest power of two not above the row's largest d (1 for a zero
+    # row), and (d / rs) * (sum of each 32 codes) / 16 as an fp16 high part and the fp16 of what the high part leaves
+    # (numpy's float16 rounds to nearest even like the device)
+    dmax = np.abs(want_d).max(axis=1)       # a Q8_K scale carries a sign
+    rs = np.where(dmax > 0, np.float32(2.0) ** np.floor(np.log2(np.maximum(dmax, np.float32(1e-37)))), np.float32(1.0)).astype(np.float32)
+    assert np.array_equal(got["rs"].cpu().numpy().view(np.uint32), rs.view(np.uint32))
+    v = (want_d / rs[:, None])[:, :, None] * want_b.reshape(m, k // 256, 8, 2).sum(-1).astype(np.float32) * np.float32(0.0625)
     hi = v.astype(np.float16)
     lo = (v - hi.astype(np.float32)).astype(np.float16)
     ms = got["msum"].cpu().numpy()
@@ -194,9 +198,13 @@ def test_quantize_q8x32_bit_exact(ctx, orc):
     assert np.array_equal(got["qs"].cpu().numpy(), raw[:, :, 8:].view(np.int8).reshape(m, k))
     assert np.array_equal(got["d"].cpu().numpy().view(np.uint32), raw[:, :, 0:4].copy().view(np.uint32)[:, :, 0])
     assert np.array_equal(got["isum"].cpu().numpy(), raw[:, :, 4:8].copy().view(np.int32)[:, :, 0])
-    # the prefill kernel's extra plane: d * isum / 16 as an fp16 high part and the fp16 of the rest
+    # the prefill kernel's extra planes: rs (power of two under the row's largest d) and (d / rs) * isum / 16 as an
+    # fp16 high part and the fp16 of the rest
     d32 = raw[:, :, 0:4].copy().view(np.float32)[:, :, 0]
-    v = d32 * raw[:, :, 4:8].copy().view(np.int32)[:, :, 0].astype(np.float32) * np.float32(0.0625)
+    dmax = d32.max(axis=1)
+    rs = np.where(dmax > 0, np.float32(2.0) ** np.floor(np.log2(np.maximum(dmax, np.float32(1e-37)))), np.float32(1.0)).astype(np.float32)
+    assert np.array_equal(got["rs"].cpu().numpy().view(np.uint32), rs.view(np.uint32))
+    v = (d32 / rs[:, None]) * raw[:, :, 4:8].copy().view(np.int32)[:, :, 0].astype(np.float32) * np.float32(0.0625)
     hi = v.astype(np.float16)
     lo = (v - hi.astype(np.float32)).astype(np.float16)
     ms = got["msum"].cpu().numpy()
@@ -928,6 +936,31 @@ def test_ffn_equals_the_chain_and_the_oracle(ctx, orc, down_type, m):
         gate(got, ref)
         for w in (wg, wu, wd):
             w.free()
+
+@pytest.mark.parametrize("act_name", ["ggml", "q8x32"])
+@pytest.mark.parametrize("m", [64, 200])
+def test_tiled_q4k_products_over_a_wide_range_of_activation_scales(ctx, orc, m, act_name):
+    """The tiled Q4_K kernels carry the min term as fp16 high / low pairs of d * (block sum) / 16 and of dmin * min.
+    The pairs are normalised by the row (a power of two under the row's largest block scale), so whole rows scaled by
+    powers of two from 2^-40 to 2^40 must come out like the oracle's, which is exactly scale-invariant for powers of
+    two (the decode and small-batch kernels are too): no precision lost to fp16 subnormals at the small end, no
+    overflow at the large end.  One row carries a block 2^20 below the row's largest."""
+    from magnitude_amd import ACT_GGML, ACT_Q8X32
+    act, oact = (ACT_GGML, orc.ACT_GGML) if act_name == "ggml" else (ACT_Q8X32, orc.ACT_Q8X32)
+    k, n = 2048, 192
+    rng = np.random.default_rng(900 + m)
+    blocks = make_weight(orc, Q4_K, n, k, seed=9100)
+    w = ctx.upload(Q4_K, k, n, blocks)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    exps = [-40, -24, -12, -4, 0, 8, 16, 24, 40]
+    x[5, 256:512] *= np.float32(2.0 ** -20)     # a block far below the row's largest: its bits no longer matter to the row
+    for i in range(m):
+        x[i] *= np.float32(2.0 ** exps[i % len(exps)])
+    got = ctx.mul_mat(w, dev(x), act).cpu().numpy()
+    want = orc.mul_mat(Q4_K, blocks, k, x, oact)
+    scale = np.float32(2.0) ** np.array([exps[i % len(exps)] for i in range(m)], np.float32)[:, None]
+    close(got / scale, want / scale, 5e-5)      # compared at the scale of an N(0, 1) row
+    w.free()
 
 
 BENCHED_PREFILL = (   # every (mode, type, K, N) x M the benchmark's prefill leg times (config 4 and the layer's other formats)
