@@ -84,14 +84,6 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const Weigh
     const int64_t u_begin = min((int64_t)blockIdx.y * per, n_units), u_end = min(u_begin + per, n_units);
     if (gridDim.y > 1) y = part + (size_t)blockIdx.y * M * N;
 
-    // the lane's two output columns (clamped for loads; stores are guarded)
-    int64_t ncol[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        int64_t n = n0 + wn * 64 + j * 32 + l32;
-        ncol[j] = n < N ? n : N - 1;
-    }
-
     v16f acc[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j)
@@ -188,40 +180,55 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const Weigh
     }
 
     // ---------------------------------------------------------------- main loop, int8 cores
+    // Addresses: a scalar base per operand plus a 32-bit lane offset that never changes; the K position is added
+    // to the scalar side.  (64-bit pointers per lane cost the registers this kernel does not have.)  Rows past the
+    // end of a tile read the last valid row: their results are never stored.
+    const int mrow_cap = (int)(M - 1 - m0 < BM - 1 ? M - 1 - m0 : BM - 1);
+    const int nrow_cap = (int)(N - 1 - n0 < BN - 1 ? N - 1 - n0 : BN - 1);
+    const global_ptr<int8_t> abase_s = scalar_global(a.qs + m0 * K);
+    const global_ptr<float> adbase_s = scalar_global(a.d + m0 * kb32);
+    uint32_t aoffg[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int idx = tid + kGemmThreads * i, row = idx >> 3, seg = idx & 7;
+        aoffg[i] = (uint32_t)(row < mrow_cap ? row : mrow_cap) * (uint32_t)K + 16u * seg;
+    }
+    const uint32_t wrow = (uint32_t)((tid >> 2) < nrow_cap ? (tid >> 2) : nrow_cap);
+    const uint32_t hrow = (uint32_t)(tid - BM < 0 ? 0 : (tid - BM < nrow_cap ? tid - BM : nrow_cap));
+    const uint32_t adoffg = (uint32_t)(tid < mrow_cap ? tid : mrow_cap) * (uint32_t)kb32;
+    global_ptr<uint8_t> wbase_s = nullptr;
+    global_ptr<int8_t> w8base_s = nullptr;
+    global_ptr<uint16_t> w8d_s = nullptr;
+    uint32_t woffg, hoffg;
+    if constexpr (kQ4) {
+        wbase_s = scalar_global(w.q4k + n0 * w.nb * 144);
+        woffg = wrow * (uint32_t)w.nb * 144u + 16u + 16u * (tid & 3);
+        hoffg = hrow * (uint32_t)w.nb * 144u;
+    } else {
+        w8base_s = scalar_global(w.q8_qs + n0 * K);
+        w8d_s = scalar_global(w.q8_d + n0 * w.nb);
+        woffg = wrow * (uint32_t)K + 32u * (tid & 3);
+        hoffg = hrow * (uint32_t)w.nb;
+    }
     auto load_stage = [&](StageRegs &r, int64_t k0) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {  // activations: 128 rows x 128 B
-            const int idx = tid + kGemmThreads * i;
-            const int row = idx >> 3, seg = idx & 7;
-            int64_t m = m0 + row;
-            r.act[i] = make_uint4(0, 0, 0, 0);
-            if (m < M) r.act[i] = *reinterpret_cast<const uint4 *>(a.qs + m * K + k0 + 16 * seg);
-        }
+        for (int i = 0; i < 2; ++i)   // activations: 128 rows x 128 B
+            r.act[i] = load_global<uint4>(abase_s + k0, aoffg[i]);
         if constexpr (kQ4) {  // weights: 128 rows x 64 packed bytes (two 64-weight chunks of the super-block)
-            const int row = tid >> 2, part = tid & 3;
-            int64_t n = n0 + row;
-            if (n >= N) n = N - 1;
             const int c2 = (int)((k0 & 255) >> 5);  // 32-byte chunk pair index * 2
-            const uint8_t *blk = w.q4k + (n * w.nb + (k0 >> 8)) * 144 + 16 + 16 * c2 + 16 * part;
-            r.wq = *reinterpret_cast<const uint4 *>(blk);
+            r.wq = load_global<uint4>(wbase_s + ((k0 >> 8) * 144 + 16 * c2), woffg);
         } else {              // weights: 128 rows x 128 int8
-            const int row = tid >> 2, part = tid & 3;
-            int64_t n = n0 + row;
-            if (n >= N) n = N - 1;
-            const int8_t *src = w.q8_qs + n * K + k0 + 32 * part;
-            r.wq = *reinterpret_cast<const uint4 *>(src);
-            r.wq2 = *reinterpret_cast<const uint4 *>(src + 16);
+            r.wq = load_global<uint4>(w8base_s + k0, woffg);
+            r.wq2 = load_global<uint4>(w8base_s + k0 + 16, woffg);
         }
         r.ad = make_float4(0.f, 0.f, 0.f, 0.f);
         if (tid < BM) {
-            if (m0 + tid < M) r.ad = *reinterpret_cast<const float4 *>(a.d + (m0 + tid) * kb32 + (k0 >> 5));
+            r.ad = load_global<float4>(adbase_s + (k0 >> 5), 4u * adoffg);
         } else if (tid < BM + BN && (!kQ4 || (k0 & 255) == 0)) {
-            int64_t n = n0 + (tid - BM);
-            if (n >= N) n = N - 1;
             if constexpr (kQ4) {   // a new super-block starts: its header
-                r.ad = *reinterpret_cast<const float4 *>(w.q4k + (n * w.nb + (k0 >> 8)) * 144);
+                r.ad = load_global<float4>(wbase_s + (k0 >> 8) * 144, hoffg);
             } else {               // the four fp16 scales of this K-step
-                const uint2 d4 = *reinterpret_cast<const uint2 *>(w.q8_d + n * w.nb + (k0 >> 5));
+                const uint2 d4 = load_global<uint2>(w8d_s + (k0 >> 5), 2u * hoffg);
                 r.ad.x = __uint_as_float(d4.x);
                 r.ad.y = __uint_as_float(d4.y);
             }
@@ -312,12 +319,17 @@ __global__ __launch_bounds__(kGemmThreads, 4) void gemm_per32_kernel(const Weigh
     }
 
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
+    // (the lane's coordinates are worked out again from the thread index, made opaque so that nothing of the
+    // address arithmetic is carried through the main loop in registers the loop needs)
+    int tid_s = tid;
+    asm volatile("" : "+v"(tid_s));
+    const int l32_s = tid_s & 31, lh_s = (tid_s >> 5) & 1, wm_s = tid_s >> 7, wn_s = (tid_s >> 6) & 1;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const int64_t n = n0 + wn * 64 + j * 32 + l32;
+        const int64_t n = n0 + wn_s * 64 + j * 32 + l32_s;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const int64_t m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            const int64_t m = m0 + wm_s * 32 + 8 * (v >> 2) + 4 * lh_s + (v & 3);
             if (m < M && n < N) y[m * N + n] = acc[j][v];
         }
     }
@@ -665,7 +677,7 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
     const uint8_t *wbase_s = scalar_pointer(wbase);
     const int8_t *abase_s = scalar_pointer(abase);
     const uint8_t *msbase_s = scalar_pointer(msbase);
-    const float *dxbase_s = scalar_pointer(dxbase);
+    const global_ptr<float> dxbase_s = scalar_global(dxbase);
     auto request_strip = [&](uint32_t sb, int c) {
         global_to_lds16(wbase_s + (woff[c] + sb * 144u), park + 1024 * c);
     };
@@ -866,6 +878,7 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(const float *__restrict_
 
 template <int QT>
 hipError_t launch_per32(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &sc, hipStream_t s) {
+    if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 128 rows of K bytes
     const int n_split = sc.p ? per32_splits(w.K, M, w.N) : 1;
     if (n_split > 1 && (size_t)n_split * M * w.N * 4 > sc.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
     if (dry_run()) return hipSuccess;

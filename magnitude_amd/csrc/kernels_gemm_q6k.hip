@@ -279,7 +279,7 @@ __global__ __launch_bounds__(512, 1) void gemm_q6k_q8k_wide_kernel(const WeightV
     const uint8_t *qlbase = scalar_pointer(w.q6_ql + wave_row0 * nb * 128);
     const uint8_t *qhbase = scalar_pointer(w.q6_qh + wave_row0 * nb * 64);
     const uint8_t *scbase = scalar_pointer(reinterpret_cast<const uint8_t *>(w.q6_sc) + wave_row0 * nb * 16);
-    const uint16_t *dbase = scalar_pointer(w.q6_d + wave_row0 * nb);
+    const global_ptr<uint16_t> dbase = scalar_global(w.q6_d + wave_row0 * nb);
     uint32_t qloff[4], qhoff[2];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {   // slot p = lane + 64*c of the wave's 256: row p / 8, slot p % 8
@@ -302,7 +302,7 @@ __global__ __launch_bounds__(512, 1) void gemm_q6k_q8k_wide_kernel(const WeightV
         const int row = 4 * (wave + NW * p) + (lane >> 4), seg = (lane & 15) ^ (row & 15);
         aoffg[p] = (uint32_t)((row < mrow_cap ? row : mrow_cap) * (int)K + 16 * seg);
     }
-    const float *dxbase = scalar_pointer(a.d + m0 * nb);
+    const global_ptr<float> dxbase = scalar_global(a.d + m0 * nb);
     const int dxtok = tid & 127;
     const uint32_t dxoffg = (uint32_t)((dxtok < mrow_cap ? dxtok : mrow_cap) * (int)nb);
     uint8_t *pql = sm.ql[wave], *pqh = sm.qh[wave];

@@ -22,4 +22,25 @@ __device__ __forceinline__ const T *scalar_pointer(const T *p) {
     return reinterpret_cast<const T *>(((uint64_t)hi << 32) | lo);
 }
 
+// The same, typed as a pointer into global memory: a pointer rebuilt from integers has lost its address space,
+// and loads through it would be flat loads, which count against the LDS wait counter as well as the vector
+// memory one (a wait for an LDS read would then also wait for them).
+template <typename T>
+using global_ptr = const T __attribute__((address_space(1))) *;
+
+template <typename T>
+__device__ __forceinline__ global_ptr<T> scalar_global(const T *p) {
+    return (global_ptr<T>)scalar_pointer(p);
+}
+
+// 16 / 8 / 4 bytes at byte offset `off` from a global base
+template <typename V, typename T>
+__device__ __forceinline__ V load_global(global_ptr<T> base, uint32_t off) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *(global_ptr<V>)((global_ptr<uint8_t>)base + off);
+#else
+    return V{};   // device-only; the host pass just has to parse it
+#endif
+}
+
 }  // namespace qproj

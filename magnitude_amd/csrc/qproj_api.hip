@@ -989,7 +989,7 @@ int qproj_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, 
     if (M < 0) return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_ffn: negative M");
     if (M == 0) return QPROJ_OK;
     QP_HIP(ctx, hipSetDevice(ctx->device));
-    const int64_t K = gate->K, d_ff = gate->N;
+    const int64_t d_ff = gate->N;
     const NormSpec norm{gamma_dev, eps};
     // the scratch row(s) h between the halves, kept apart from the workspace the projections themselves use
     int rc = ensure_ws2(ctx, (size_t)3 * M * d_ff * 4);
