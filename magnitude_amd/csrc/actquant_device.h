@@ -134,6 +134,80 @@ __device__ __forceinline__ float pow2_floor(float v) {
     return e ? __uint_as_float(e) : 1.0f;
 }
 
+// ---- quantizer and min-term operand in one launch: a 16-wave workgroup owns an activation row.
+// The waves quantize the row's super-blocks as above and also leave the row's scales (`ld`: nb, or 8 nb for the
+// per-32 format) and sums of 32 codes (`ls`: [nb][8]) in LDS; row_minterm_finish then finds the row's normaliser
+// and writes the min-term plane with the arithmetic of minterm_rows_kernel (the same bits as that launch).
+constexpr int kRowWaves = 16, kRowThreads = 64 * kRowWaves;
+__host__ __device__ constexpr size_t row_minterm_lds_bytes(bool per32, int nb) { return (size_t)nb * (per32 ? 16 : 9) * 4; }
+
+__device__ __forceinline__ void wave_store_q8k_row(const float4 &v, int lane, int64_t g, int sb, int8_t *__restrict__ qs,
+                                                   float *__restrict__ d, int16_t *__restrict__ bsums, float *ld, int *ls) {
+    int bsum;
+    float dd;
+    const uint32_t packed = wave_quantize_q8k(v, lane, bsum, dd);
+    reinterpret_cast<uint32_t *>(qs + g * 256)[lane] = packed;
+    if ((lane & 3) == 0) bsums[g * 16 + (lane >> 2)] = (int16_t)bsum;
+    const int pair = bsum + __shfl_down(bsum, 4);   // two neighbouring groups of 16
+    if ((lane & 7) == 0) ls[sb * 8 + (lane >> 3)] = pair;
+    if (lane == 0) {
+        d[g] = dd;
+        ld[sb] = dd;
+    }
+}
+
+__device__ __forceinline__ void wave_store_q8x32_row(const float4 &v, int lane, int64_t g, int sb, int8_t *__restrict__ qs,
+                                                     float *__restrict__ d, int32_t *__restrict__ isum, float *ld, int *ls) {
+    int sum;
+    float dd;
+    const uint32_t packed = wave_quantize_q8_32(v, sum, dd);
+    reinterpret_cast<uint32_t *>(qs + g * 256)[lane] = packed;
+    if ((lane & 7) == 0) {
+        d[g * 8 + (lane >> 3)] = dd;
+        isum[g * 8 + (lane >> 3)] = sum;
+        ld[sb * 8 + (lane >> 3)] = dd;
+        ls[sb * 8 + (lane >> 3)] = sum;
+    }
+}
+
+// called by all kRowThreads threads of the workgroup after their stores into ld / ls; `wmax`: kRowWaves floats of LDS
+template <bool PER32>
+__device__ __forceinline__ void row_minterm_finish(const float *ld, const int *ls, int nb, int64_t m,
+                                                   uint16_t *__restrict__ msum, float *__restrict__ rs, float *wmax) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nd = PER32 ? nb * 8 : nb;
+    __syncthreads();
+    float dmax = 0.f;
+    for (int i = tid; i < nd; i += kRowThreads) dmax = fmaxf(dmax, fabsf(ld[i]));   // a Q8_K scale carries a sign
+    dmax = wave_max(dmax);
+    if (lane == 0) wmax[wave] = dmax;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < kRowWaves; ++w) dmax = fmaxf(dmax, wmax[w]);
+    const float r = pow2_floor(dmax), inv = 1.0f / r;   // exact: a power of two
+    if (tid == 0) rs[m] = r;
+    for (int sb = tid; sb < nb; sb += kRowThreads) {
+        uint32_t hi[4], lo[4];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const float dd = PER32 ? ld[sb * 8 + t] : ld[sb];
+            const float v = (dd * inv) * (float)ls[sb * 8 + t] * kMinPrescale;
+            const _Float16 h = (_Float16)v, l = (_Float16)(v - (float)h);
+            const uint32_t hb = __builtin_bit_cast(uint16_t, h), lb = __builtin_bit_cast(uint16_t, l);
+            if (t & 1) {
+                hi[t >> 1] |= hb << 16;
+                lo[t >> 1] |= lb << 16;
+            } else {
+                hi[t >> 1] = hb;
+                lo[t >> 1] = lb;
+            }
+        }
+        uint4 *dst = reinterpret_cast<uint4 *>(msum + (m * nb + sb) * 16);
+        dst[0] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        dst[1] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+    }
+}
+
 // Sum of squares of a row spread over a workgroup of 16 waves in ggml's precision (float products summed in
 // double).  The order is fixed - lane's own pieces, butterfly over the wave, waves 0..15 - so that every
 // kernel that normalises a row gets the same bits.  `partial` is 16 doubles of LDS; contains a barrier.

@@ -22,12 +22,21 @@ constexpr int kNormWaves = 16, kNormThreads = 64 * kNormWaves;
 constexpr int kHeld = 4;   // 256-float pieces a wave keeps in registers: rows up to 16384 floats are read once
 
 // MODE 0: store fp32.  MODE 1: Q8_K planes.  MODE 2: ggml Q8_0 blocks.  MODE 3: per-32 prefill format.
-template <int MODE>
+// MT (modes 1 and 3): also the row normaliser and the min-term plane of the tiled Q4_K kernels, from scales and
+// sums left in dynamic LDS (row_minterm_lds_bytes), so that no second launch goes over the row.
+template <int MODE, bool MT>
 __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                                 float eps, int64_t K, float *__restrict__ y,
                                                                 int8_t *__restrict__ qs, float *__restrict__ d,
-                                                                int16_t *__restrict__ bsums, int32_t *__restrict__ isum) {
+                                                                int16_t *__restrict__ bsums, int32_t *__restrict__ isum,
+                                                                uint16_t *__restrict__ msum, float *__restrict__ rs) {
+    static_assert(kNormThreads == kRowThreads, "the row helpers assume this workgroup");
+    extern __shared__ __align__(16) float row_lds[];
     __shared__ double partial[kNormWaves];
+    __shared__ float wmax[kNormWaves];
+    const int nb = (int)(K / 256);
+    float *ld = row_lds;
+    int *ls = reinterpret_cast<int *>(row_lds + (MODE == 3 ? nb * 8 : nb));
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t row = blockIdx.x;
     const float *xr = x + row * K;
@@ -72,12 +81,16 @@ __global__ __launch_bounds__(kNormThreads) void rms_norm_kernel(const float *__r
         if (MODE == 0) {
             if (live) *reinterpret_cast<float4 *>(y + row * K + e0) = v;
         } else if (MODE == 1) {   // K is a multiple of 256 here: every piece is whole
-            wave_store_q8k(v, lane, row * (K / 256) + p, qs, d, bsums);
+            if constexpr (MT) wave_store_q8k_row(v, lane, row * nb + p, p, qs, d, bsums, ld, ls);
+            else wave_store_q8k(v, lane, row * nb + p, qs, d, bsums);
+        } else if (MODE == 3 && MT) {
+            wave_store_q8x32_row(v, lane, row * nb + p, p, qs, d, isum, ld, ls);
         } else {
             // the planes are indexed by the flattened element: row * K is a multiple of 32
             wave_store_q8_32<MODE == 2>(v, lane, row * K + e0, live, qs, d, isum);
         }
     }
+    if constexpr (MT) row_minterm_finish<MODE == 3>(ld, ls, nb, row, msum, rs, wmax);
 }
 
 }  // namespace
@@ -91,12 +104,17 @@ hipError_t launch_rms_norm(int kind, const float *x, const float *gamma, float e
     if (kind >= 0 && kind != kActKindQ8_K && kind != kActKindQ8_0 && kind != kActKindQ8X32) return hipErrorInvalidValue;
     if (dry_run()) return hipSuccess;
     const dim3 grid((unsigned)M), block(kNormThreads);
-    if (kind < 0) hipLaunchKernelGGL(rms_norm_kernel<0>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum);
-    else if (kind == kActKindQ8_K) hipLaunchKernelGGL(rms_norm_kernel<1>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum);
-    else if (kind == kActKindQ8_0) hipLaunchKernelGGL(rms_norm_kernel<2>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum);
-    else hipLaunchKernelGGL(rms_norm_kernel<3>, grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum);
+    const bool mt = msum && rs && (kind == kActKindQ8_K || kind == kActKindQ8X32) && K / 256 <= 1024;
+    if (kind < 0) hipLaunchKernelGGL((rms_norm_kernel<0, false>), grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum, msum, rs);
+    else if (kind == kActKindQ8_0) hipLaunchKernelGGL((rms_norm_kernel<2, false>), grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum, msum, rs);
+    else if (kind == kActKindQ8_K && mt)
+        hipLaunchKernelGGL((rms_norm_kernel<1, true>), grid, block, row_minterm_lds_bytes(false, (int)(K / 256)), s, x, gamma, eps, K, y, qs, d, bsums, isum, msum, rs);
+    else if (kind == kActKindQ8_K) hipLaunchKernelGGL((rms_norm_kernel<1, false>), grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum, msum, rs);
+    else if (mt)
+        hipLaunchKernelGGL((rms_norm_kernel<3, true>), grid, block, row_minterm_lds_bytes(true, (int)(K / 256)), s, x, gamma, eps, K, y, qs, d, bsums, isum, msum, rs);
+    else hipLaunchKernelGGL((rms_norm_kernel<3, false>), grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum, msum, rs);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess || kind < 0 || kind == kActKindQ8_0 || !msum) return e;
+    if (e != hipSuccess || kind < 0 || kind == kActKindQ8_0 || !msum || mt) return e;
     return launch_minterm_rows(kind, d, bsums, isum, M, K, msum, rs, s);
 }
 
