@@ -494,8 +494,10 @@ constexpr int kDense = 0, kGrouped = 1, kGroupedSwiglu = 2;
 // MODE kDense: y[m][n] for the M rows of `a`.  kGrouped: the workgroup's expert e multiplies its
 // own pairs, y[pair][n].  kGroupedSwiglu: tensors 0 and 1 are gate and up of the same expert and
 // y[pair][n] = silu(gate . x) * (up . x).
-template <int QT, int NI, int W, int MODE>
+// FLAT (expert-grouped launches with K in one part, kw = 1): the wave's row groups as one stream of items.
+template <int QT, int NI, int W, int MODE, bool FLAT = false>
 __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
+    static_assert(!FLAT || MODE != kDense, "the flat item stream is for the expert-grouped modes");
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int MT = 8 * NI, NV = 4 * NI;
     constexpr bool GROUPED = MODE != kDense, SWIGLU = MODE == kGroupedSwiglu;
@@ -580,7 +582,114 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
     uint8_t *region = smem + L.off_w + wave * Cfg<QT>::kRegion;
     int *map = reinterpret_cast<int *>(smem + L.off_map);
 
+    // Expert-grouped launches with K in one part: the wave's row groups are ONE stream of (row group, tensor,
+    // super-block) items, so the loads of the next row group are in flight while the last items of this one are
+    // worked on (with short K a row group is three items: restarting the pipeline for each one left the memory
+    // system idle for a round trip per row group).
+    if constexpr (FLAT) {
+        {
+            const int per = NT * nsb;   // items of a row group
+            int n_rg = 0;               // the wave's row groups that exist (a prefix)
+            for (int rg = 0; rg < g.rg_loop; ++rg) n_rg += ((rs * g.rg_loop + rg) * g.rw + rgl) * 32 < N ? 1 : 0;
+            const int total = n_rg * per;
+            auto row_of = [&](int rg) { return ((rs * g.rg_loop + rg) * g.rw + rgl) * 32; };
+            auto setup = [&](Stager<QT> &st, int rg) {
+                const int r0 = row_of(rg);
+                const int64_t row = (int64_t)expert * N + r0;
+                st.rebase(0, w, row);
+                st.rebase(1, SWIGLU ? g.t[1].w : w, row);
+                st.init(w, min(31, N - 1 - r0), lane);
+            };
+            int rg_a = -1, rg_b = -1;   // the row group each stager's addresses stand at
+            auto issue_at = [&](Stager<QT> &st, int &st_rg, int rg, int i) {
+                if (rg >= n_rg) {   // past the end: the last item again, harmless
+                    rg = n_rg - 1;
+                    i = per - 1;
+                }
+                if (rg != st_rg) {
+                    setup(st, rg);
+                    st_rg = rg;
+                }
+                const int t = SWIGLU && i >= nsb ? 1 : 0;
+                st.issue(t, c0 + i - t * nsb);
+            };
+            for (int m0 = 0; m0 < n_rows; m0 += MT) {
+                const int m_cnt = min(MT, n_rows - m0);
+                // cursors of the two stagers (items 0, 2, 4, .. and 1, 3, 5, ..) and of the consumer; a wave whose row
+                // groups all lie past the end of the matrix (total = 0) only takes part in the staging and the barriers
+                int arg = 0, ai = 0, brg = 0, bi = 1, crg = 0, ci = 0;
+                while (bi >= per) { bi -= per; ++brg; }
+                if (total > 0) {
+                    issue_at(sa, rg_a, arg, ai);
+                    issue_at(sb_, rg_b, brg, bi);
+                }
+                if (m0 > 0) __syncthreads();   // the previous pass is done with the staged rows and the regions
+                if ((int)threadIdx.x < MT)
+                    map[threadIdx.x] = (int)threadIdx.x >= m_cnt ? 0
+                                       : g.ids      ? pair0 + m0 + (int)threadIdx.x
+                                                    : g.order[pair0 + m0 + (int)threadIdx.x];
+                __syncthreads();
+                if (g.x)
+                    stage_quantize<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
+                else
+                    stage_activations<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
+                __syncthreads();
+
+                float out[NT][NV];
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) out[t][v] = 0.f;
+                auto consume = [&]() {
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                    if (SWIGLU && ci >= nsb)
+                        compute<QT, NI>(region, smem, L, ci - nsb, lane, out[NT - 1]);
+                    else
+                        compute<QT, NI>(region, smem, L, ci, lane, out[0]);
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                    if (++ci == per) {   // the row group is complete: store it, start the next one
+                        const int n = row_of(crg) + nl;
+#pragma unroll
+                        for (int v = 0; v < NV; ++v) {
+                            const int m = 8 * (v >> 2) + 4 * h + (v & 3);
+                            float r = out[0][v];
+                            if constexpr (SWIGLU) r = (r / (1.0f + expf(-r))) * out[NT - 1][v];
+                            if (m < m_cnt && n < N) y[(size_t)map[m] * N + n] = r;
+                        }
+#pragma unroll
+                        for (int t = 0; t < NT; ++t)
+#pragma unroll
+                            for (int v = 0; v < NV; ++v) out[t][v] = 0.f;
+                        ci = 0;
+                        ++crg;
+                    }
+                };
+                auto advance2 = [&](int &rg, int &i) {
+                    i += 2;
+                    while (i >= per) { i -= per; ++rg; }
+                };
+                int j = 0;
+                for (; j + 1 < total; j += 2) {
+                    sa.park(region, lane);
+                    advance2(arg, ai);
+                    issue_at(sa, rg_a, arg, ai);
+                    consume();
+                    sb_.park(region, lane);
+                    advance2(brg, bi);
+                    issue_at(sb_, rg_b, brg, bi);
+                    consume();
+                }
+                if (j < total) {
+                    sa.park(region, lane);
+                    consume();
+                }
+            }
+            return;
+        }
+    }
+
     // dense launches stage all (<= MT) rows at once; an expert with more than MT pairs takes several passes
+    if constexpr (!FLAT)
     for (int m0 = 0; m0 < (GROUPED ? n_rows : 1); m0 += MT)
     for (int rg = 0; rg < (GROUPED ? g.rg_loop : 1); ++rg) {   // the rows staged for this pass serve all of the wave's row groups
         const int m_cnt = min(MT, n_rows - m0);
@@ -679,11 +788,16 @@ __global__ __launch_bounds__(256) void sum_chunks_kernel(const MfmaArgs g) {
     }
 }
 
-template <int QT, int NI, int W, int MODE>
+template <int QT, int NI, int W, int MODE, bool FLAT = false>
 hipError_t launch_one(const MfmaArgs &g, hipStream_t s) {
+    // (the 16-row instances of the larger formats would spill registers in the flat form: they keep the loop per row group)
+    if constexpr (MODE != kDense && !FLAT && (QT == kTypeQ4_K || NI == 1)) {
+        static const bool no_flat = tuning_int("QPROJ_MOE_NO_FLAT", 0) != 0;
+        if (g.kw == 1 && !no_flat) return launch_one<QT, NI, W, MODE, true>(g, s);
+    }
     if (dry_run()) return hipSuccess;
     const Layout L = layout<QT, 8 * NI, W>(g.chunk_sb);
-    auto kern = gemv_mfma_kernel<QT, NI, W, MODE>;
+    auto kern = gemv_mfma_kernel<QT, NI, W, MODE, FLAT>;
     static int allowed = 0;
     if (L.total > allowed) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -809,7 +923,11 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
     g.x_div = args.x_div;
     const WeightView &w = args.t[0].w;
     const int type = w.type;
-    const int W = waves_per_wg(type);
+    // Q4_K experts: four waves a workgroup, two workgroups a compute unit - the prologue of one (expert lookup,
+    // row map, staged rows: a chain of dependent loads) hides behind the other's weight stream.  Measured on the
+    // 128-expert FFN against eight waves: 23.2 -> 21.1 us at one token, 121.9 -> 115.5 us at 64.
+    static const int moe_waves = tuning_int("QPROJ_MOE_WAVES", 4);
+    const int W = type == kTypeQ4_K && (moe_waves == 4 || moe_waves == 8) ? moe_waves : waves_per_wg(type);
     const int64_t rg_e = (w.N + 31) / 32;
     const bool small = n_pairs <= 4 * w.E;   // few pairs an expert: 8 staged rows a pass are enough
     Split p = plan(w.K, small ? 8 : 16, std::min<int64_t>(w.E, n_pairs) * rg_e, W);
@@ -827,15 +945,17 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
         g.t[i].y = args.t[i].y;
     }
     // Short K makes a row group a few steps of work against a prologue (row map, staged rows, barriers) of
-    // several microseconds.  A wave can take two row groups in a row and pay the prologue once; measured on
-    // the 128-expert FFN's down projection (K = 768): worth it for a grid of one to three workgroups per
-    // compute unit (416 workgroups: the FFN at B = 8 goes from 61.6 to 55.3 us), neutral above (992
-    // workgroups, B = 64), harmful below (64 workgroups, B = 1: 24 -> 31 us), and four in a row always lose.
-    static const int forced_loop = tuning_int("QPROJ_MOE_RG_LOOP", 0);
+    // several microseconds.  A wave can take two row groups in a row (one stream of items) and pay the prologue
+    // once; measured on the 128-expert FFN (K = 768 down, K = 2048 gate / up): worth it for grids beyond three
+    // workgroups per compute unit (down at 8 and 64 tokens: 62.3 -> 58.8 and 115.5 -> 111.3 us), harmful for small
+    // grids (one token: 21.1 -> 22.9 us; gate / up at 64 tokens, 744 workgroups: 111.3 -> 128 us), and four in a
+    // row always lose.
+    static const int forced_all = tuning_int("QPROJ_MOE_RG_LOOP", 0), forced_down = tuning_int("QPROJ_MOE_RG_LOOP_DOWN", 0);
+    const int forced_loop = !swiglu && forced_down > 0 ? forced_down : forced_all;
     {
         const int64_t wgs1 = (args.ids ? n_pairs : std::min<int64_t>(w.E, n_pairs)) * ((rg_e + g.rw - 1) / g.rw);
         const int64_t cus = 256;
-        int loop = forced_loop > 0 ? forced_loop : (wgs1 > cus && wgs1 <= 3 * cus) ? 2 : 1;
+        int loop = forced_loop > 0 ? forced_loop : wgs1 > 3 * cus ? 2 : 1;
         loop = (int)std::min<int64_t>(loop, std::max<int64_t>(1, rg_e / g.rw));
         while (loop > 1 && rg_e % ((int64_t)g.rw * loop) != 0) --loop;   // no half-empty last workgroup
         g.rg_loop = std::min(loop, 8);
