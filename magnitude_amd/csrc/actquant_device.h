@@ -140,6 +140,7 @@ __device__ __forceinline__ float pow2_floor(float v) {
 // and writes the min-term plane with the arithmetic of minterm_rows_kernel (the same bits as that launch).
 constexpr int kRowWaves = 16, kRowThreads = 64 * kRowWaves;
 __host__ __device__ constexpr size_t row_minterm_lds_bytes(bool per32, int nb) { return (size_t)nb * (per32 ? 16 : 9) * 4; }
+constexpr size_t kRowLdsMax = 48 * 1024;   // rows beyond it (K > 196608 in the per-32 format) take the min-term launch
 
 __device__ __forceinline__ void wave_store_q8k_row(const float4 &v, int lane, int64_t g, int sb, int8_t *__restrict__ qs,
                                                    float *__restrict__ d, int16_t *__restrict__ bsums, float *ld, int *ls) {

@@ -133,7 +133,8 @@ hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, i
     // the min-term launch: 4.6 against 7.1 us at 128 x 4096, 9.3 against 10.6 at 512 x 14336; many short rows are
     // the exception, 22.8 against 18.8 us at 4096 x 4096, where a workgroup has one chunk a wave and two barriers)
     static const int rows_max_short = tuning_int("QPROJ_ROW_QUANT_MAX_M", 1024);
-    if (msum && rs && kind != kActKindQ8_0 && K % 256 == 0 && K / 256 <= 1024 && (K / 256 >= 32 || M <= rows_max_short)) {
+    if (msum && rs && kind != kActKindQ8_0 && K % 256 == 0 && row_minterm_lds_bytes(kind == kActKindQ8X32, (int)(K / 256)) <= kRowLdsMax &&
+        (K / 256 >= 32 || M <= rows_max_short)) {
         const int nb = (int)(K / 256);
         const dim3 rgrid((unsigned)M), rblock(kRowThreads);
         if (kind == kActKindQ8_K)

@@ -104,7 +104,8 @@ hipError_t launch_rms_norm(int kind, const float *x, const float *gamma, float e
     if (kind >= 0 && kind != kActKindQ8_K && kind != kActKindQ8_0 && kind != kActKindQ8X32) return hipErrorInvalidValue;
     if (dry_run()) return hipSuccess;
     const dim3 grid((unsigned)M), block(kNormThreads);
-    const bool mt = msum && rs && (kind == kActKindQ8_K || kind == kActKindQ8X32) && K / 256 <= 1024;
+    const bool mt = msum && rs && (kind == kActKindQ8_K || kind == kActKindQ8X32) &&
+                    row_minterm_lds_bytes(kind == kActKindQ8X32, (int)(K / 256)) <= kRowLdsMax;
     if (kind < 0) hipLaunchKernelGGL((rms_norm_kernel<0, false>), grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum, msum, rs);
     else if (kind == kActKindQ8_0) hipLaunchKernelGGL((rms_norm_kernel<2, false>), grid, block, 0, s, x, gamma, eps, K, y, qs, d, bsums, isum, msum, rs);
     else if (kind == kActKindQ8_K && mt)

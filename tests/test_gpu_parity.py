@@ -190,7 +190,7 @@ def test_quantize_q8_0_activations_bit_exact(ctx, orc):
     assert np.array_equal(got["d"].cpu().numpy().view(np.uint32), want_d.view(np.uint32))
 
 
-@pytest.mark.parametrize("m,k", [(7, 1024), (129, 4608)])
+@pytest.mark.parametrize("m,k", [(7, 1024), (129, 4608), (2, 200704)])   # the last: too long a row for the one-launch route
 def test_quantize_q8x32_bit_exact(ctx, orc, m, k):
     from magnitude_amd import ACT_Q8X32
     rng = np.random.default_rng(52)
