@@ -71,7 +71,9 @@ __device__ __forceinline__ void convert_pieces(const v4i &lq, const v4i &hq, con
             const uint32_t x = nib ? (lw >> 4) & 0x0f0f0f0fu : lw & 0x0f0f0f0fu;
             const uint32_t hs = g == 0 ? hw << 4 : g == 1 ? hw << 2 : g == 2 ? hw : hw >> 2;
             const uint32_t q = (hs & 0x30303030u) | x;                          // four codes 0..63
-            const uint32_t e0 = q & 0x00ff00ffu, e1 = (q >> 8) & 0x00ff00ffu;   // codes 0, 2 and 1, 3 in 16-bit lanes
+            // codes 0, 2 and 1, 3 in 16-bit lanes: byte permutes over zeros (a mask for the first pair made the compiler
+            // build the four codes twice, once for each pair)
+            const uint32_t e0 = __builtin_amdgcn_perm(0u, q, 0x0c020c00u), e1 = __builtin_amdgcn_perm(0u, q, 0x0c030c01u);
             const uint32_t w0 = pk_mad_u16(e0, s16, c16), w1 = pk_mad_u16(e1, s16, c16);   // sc * (q - 32) + 128
             // low bytes (bit 7 flipped: minus 128 modulo 256) and high bytes, back in the order of the codes
             cl[t][c] = (int)(__builtin_amdgcn_perm(w1, w0, 0x06020400u) ^ 0x80808080u);
