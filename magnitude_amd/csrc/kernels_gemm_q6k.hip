@@ -19,6 +19,8 @@
 // rows with consecutive lanes on consecutive 16-byte pieces and parks them in wave-private LDS strips (row
 // strides of 144 and 80 bytes: conflict-free for 16-byte reads by consecutive rows); LDS otherwise holds one
 // super-block of activations, double-buffered: one workgroup barrier per 256 weights.
+#include <type_traits>
+
 #include "qproj_device.h"
 #include "qproj_internal.h"
 #include "gemm_tiles.h"
@@ -339,58 +341,79 @@ __global__ __launch_bounds__(512, 1) void gemm_q6k_q8k_wide_kernel(const WeightV
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
 
-    for (int64_t sb = sb_begin; sb < sb_end; ++sb) {
-        const int buf = (int)((sb - sb_begin) & 1);
-        const uint32_t sb_next = (uint32_t)(sb + 1 < sb_end ? sb + 1 : sb_end - 1);   // past the end: requested again, never used
-        // ---- the lane's 128 weights into both int8 operands, out of the strip
-        v4i cl[8], ch[8];
-        {
-            const v2i scq = *reinterpret_cast<const v2i *>(psc + l32 * 16 + 8 * lh);
+    // The two waves that share a SIMD (w and w + 4) run a super-block in opposite orders, as in the Q4_K kernel of
+    // this shape: EARLY waves (0..3) convert the weights of a super-block at its start, LATE waves (4..7) convert
+    // the weights of the NEXT super-block at the end of the current one, after their last tile - so one of the two
+    // has matrix work while the other has vector work, instead of both wanting the same pipe at the same time.
+    v4i cl[8], ch[8];
+    auto convert_strip = [&]() {   // the lane's 128 weights into both int8 operands, out of the strip
+        const v2i scq = *reinterpret_cast<const v2i *>(psc + l32 * 16 + 8 * lh);
 #pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const v4i hq = *reinterpret_cast<const v4i *>(pqh + qhrow + 16 * ((2 * lh + e) ^ qhx));
+        for (int e = 0; e < 2; ++e) {
+            const v4i hq = *reinterpret_cast<const v4i *>(pqh + qhrow + 16 * ((2 * lh + e) ^ qhx));
 #pragma unroll
-                for (int gl = 0; gl < 2; ++gl) {
-                    const v4i lq = *reinterpret_cast<const v4i *>(pql + qlrow + 16 * ((4 * lh + 2 * gl + e) ^ qlx));
-                    convert_pieces(lq, hq, scq, gl, e, cl, ch);
-                }
+            for (int gl = 0; gl < 2; ++gl) {
+                const v4i lq = *reinterpret_cast<const v4i *>(pql + qlrow + 16 * ((4 * lh + 2 * gl + e) ^ qlx));
+                convert_pieces(lq, hq, scq, gl, e, cl, ch);
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the strip has been read: it may be overwritten
-        __builtin_amdgcn_sched_barrier(0);
-        request_strip(sb_next);
-        const float dn = h2f(dcur);
-        const uint32_t dnext = dbase[doff + sb_next];
-        const float dxreg = dxbase[dxoffg + sb_next];
-        const int8_t *ab = sm.a[buf];
-        const float *dxs = sm.dx[buf];
+    };
+    auto run = [&](auto late_tag) {
+        constexpr bool LATE = decltype(late_tag)::value;
+        if (LATE) convert_strip();   // weights of the first super-block, with nothing to overlap
+        for (int64_t sb = sb_begin; sb < sb_end; ++sb) {
+            const int buf = (int)((sb - sb_begin) & 1);
+            const uint32_t sb_next = (uint32_t)(sb + 1 < sb_end ? sb + 1 : sb_end - 1);   // past the end: requested again, never used
+            if (!LATE) convert_strip();
+            const float dn = h2f(dcur);
+            const uint32_t dnext = dbase[doff + sb_next];
+            const float dxreg = dxbase[dxoffg + sb_next];
+            __builtin_amdgcn_sched_barrier(0);
+            request_strip(sb_next);   // its previous content was read above (early waves) or at the end of the last trip (late waves)
+            __builtin_amdgcn_sched_barrier(0);
+            const int8_t *ab = sm.a[buf];
+            const float *dxs = sm.dx[buf];
 #pragma unroll
-        for (int j = 0; j < JT; ++j) {
-            v16i ilo = zi, ihi = zi;
+            for (int j = 0; j < JT; ++j) {
+                v16i ilo = zi, ihi = zi;
 #pragma unroll
-            for (int t = 0; t < 8; ++t) {
-                const v4i af = *reinterpret_cast<const v4i *>(ab + j * 32 * 256 + (aoffl ^ (16 * t)));
-                ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, cl[t], ilo, 0, 0, 0);
-                ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, ch[t], ihi, 0, 0, 0);
+                for (int t = 0; t < 8; ++t) {
+                    const v4i af = *reinterpret_cast<const v4i *>(ab + j * 32 * 256 + (aoffl ^ (16 * t)));
+                    ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, cl[t], ilo, 0, 0, 0);
+                    ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, ch[t], ihi, 0, 0, 0);
+                }
+                if (j == 1) {   // the next super-block's activations, once the strip requests are under way
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int p = 0; p < PA; ++p) request_act(sb_next, buf ^ 1, p);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                float dxv[16];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float4 d4 = *reinterpret_cast<const float4 *>(dxs + j * 32 + 8 * i + 4 * lh);
+                    dxv[4 * i] = d4.x; dxv[4 * i + 1] = d4.y; dxv[4 * i + 2] = d4.z; dxv[4 * i + 3] = d4.w;
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[j][v] = fmaf((float)((ihi[v] << 8) + ilo[v]), dxv[v] * dn, acc[j][v]);
             }
-            if (j == 1) {   // the next super-block's activations, once the strip requests are under way
-#pragma unroll
-                for (int p = 0; p < PA; ++p) request_act(sb_next, buf ^ 1, p);
+            if (LATE) {
+                // the next super-block's strip was requested at the top of this trip; of the requests made since then
+                // (PA activation chunks) none needs to have landed
+                static_assert(PA == 4, "the wait below counts the activation requests");
+                __builtin_amdgcn_sched_barrier(0);
+                asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+                convert_strip();
             }
-            float dxv[16];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const float4 d4 = *reinterpret_cast<const float4 *>(dxs + j * 32 + 8 * i + 4 * lh);
-                dxv[4 * i] = d4.x; dxv[4 * i + 1] = d4.y; dxv[4 * i + 2] = d4.z; dxv[4 * i + 3] = d4.w;
-            }
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][v] = fmaf((float)((ihi[v] << 8) + ilo[v]), dxv[v] * dn, acc[j][v]);
+            sm.dx[buf ^ 1][dxtok] = dxreg;   // every thread stores (a repeated value past 128): no branch
+            dcur = dnext;
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
         }
-        sm.dx[buf ^ 1][dxtok] = dxreg;   // every thread stores (a repeated value past 128): no branch
-        dcur = dnext;
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        __syncthreads();
-    }
+    };
+    if (wave < 4) run(std::false_type{});
+    else run(std::true_type{});
 
     // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
     const int64_t n = n0 + wave * 32 + l32;
