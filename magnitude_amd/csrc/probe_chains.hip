@@ -21,6 +21,12 @@ __device__ __forceinline__ void filler(uint32_t (&x)[4], uint32_t y) {
 template <int VAR, int FILL>
 __global__ __launch_bounds__(512, 2) void probe(int iters, int sc, int *out) {
     const int lane = threadIdx.x & 63;
+    __shared__ __align__(16) unsigned char lds[32 * 1024];   // one 128-token activation tile: 32 fragments of 1 KB
+    const int lane_off = (lane & 31) * 256 / 8 + 16 * ((lane >> 5) ^ (lane & 1));   // any conflict-free 16-byte pattern
+    if (VAR == 4) {
+        for (int k = threadIdx.x; k < 32 * 1024 / 4; k += blockDim.x) reinterpret_cast<int *>(lds)[k] = k;
+        __syncthreads();
+    }
     v4i a[4], b = {lane * 3, 7, 9, 11}, b2 = {lane, 5, 3, 1};
     for (int t = 0; t < 4; ++t) a[t] = (v4i){lane + t, lane + 1, lane + 2, lane + 3};
     uint32_t x[4] = {1u, 2u, 3u, (uint32_t)lane};
@@ -33,6 +39,28 @@ __global__ __launch_bounds__(512, 2) void probe(int iters, int sc, int *out) {
             for (int t = 0; t < 4; ++t) {
                 acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b, acc[t], 0, 0, 0);
                 hi[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b2, hi[t], 0, 0, 0);
+                filler<FILL / 4>(x, (uint32_t)sc);
+            }
+        } else if (VAR == 2) {   // the same eight matrix instructions on TWO accumulators: each depends on the one two back
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b, acc[0], 0, 0, 0);
+                hi[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b2, hi[0], 0, 0, 0);
+                filler<FILL / 4>(x, (uint32_t)sc);
+            }
+        } else if (VAR == 4) {   // as VAR 2, every pair fed by a fresh 16-byte operand read from LDS four pairs earlier
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b, acc[0], 0, 0, 0);
+                hi[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b2, hi[0], 0, 0, 0);
+                a[t] = *reinterpret_cast<const v4i *>(lds + ((i * 4 + t) & 31) * 1024 + lane_off);
+                filler<FILL / 4>(x, (uint32_t)sc);
+            }
+        } else if (VAR == 3) {   // on FOUR accumulators (two token tiles interleaved)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                acc[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b, acc[t & 1], 0, 0, 0);
+                hi[t & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[t], b2, hi[t & 1], 0, 0, 0);
                 filler<FILL / 4>(x, (uint32_t)sc);
             }
         } else {
@@ -78,6 +106,13 @@ int main() {
     run<0, 40>("two chains + 5 vector instr / matrix instr", cus, out);
     run<0, 60>("two chains + 7.5 (the wide kernel's mix)", cus, out);
     run<0, 80>("two chains + 10", cus, out);
+    run<2, 0>("two chains on TWO accumulators, no other work", cus, out);
+    run<2, 60>("two chains on TWO accumulators + 7.5", cus, out);
+    run<4, 0>("two chains, operands from LDS, no other work", cus, out);
+    run<4, 40>("two chains, operands from LDS + 5", cus, out);
+    run<4, 60>("two chains, operands from LDS + 7.5", cus, out);
+    run<3, 0>("two chains on FOUR accumulators, no other work", cus, out);
+    run<3, 60>("two chains on FOUR accumulators + 7.5", cus, out);
     run<1, 0>("one chain + 16 mad24, nothing else", cus, out);
     run<1, 8>("one chain + 16 mad24 + 2", cus, out);
     run<1, 16>("one chain + 16 mad24 + 4", cus, out);
