@@ -374,14 +374,21 @@ __global__ __launch_bounds__(512, 1) void gemm_q6k_q8k_wide_kernel(const WeightV
             __builtin_amdgcn_sched_barrier(0);
             const int8_t *ab = sm.a[buf];
             const float *dxs = sm.dx[buf];
+            // the tiles as a two-stage pipeline: while tile j is multiplied (two chains of eight matrix instructions into one
+            // of two accumulator pairs), the finished sums of tile j - 1 are flushed from the other pair - independent work
+            // the scheduler can put between the matrix instructions
+            v16i ilo[2], ihi[2];
 #pragma unroll
-            for (int j = 0; j < JT; ++j) {
-                v16i ilo = zi, ihi = zi;
+            for (int j = 0; j <= JT; ++j) {
+                if (j < JT) {
+                    ilo[j & 1] = zi;
+                    ihi[j & 1] = zi;
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const v4i af = *reinterpret_cast<const v4i *>(ab + j * 32 * 256 + (aoffl ^ (16 * t)));
-                    ilo = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, cl[t], ilo, 0, 0, 0);
-                    ihi = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, ch[t], ihi, 0, 0, 0);
+                    for (int t = 0; t < 8; ++t) {
+                        const v4i af = *reinterpret_cast<const v4i *>(ab + j * 32 * 256 + (aoffl ^ (16 * t)));
+                        ilo[j & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, cl[t], ilo[j & 1], 0, 0, 0);
+                        ihi[j & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, ch[t], ihi[j & 1], 0, 0, 0);
+                    }
                 }
                 if (j == 1) {   // the next super-block's activations, once the strip requests are under way
                     __builtin_amdgcn_sched_barrier(0);
@@ -389,14 +396,27 @@ __global__ __launch_bounds__(512, 1) void gemm_q6k_q8k_wide_kernel(const WeightV
                     for (int p = 0; p < PA; ++p) request_act(sb_next, buf ^ 1, p);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                float dxv[16];
+                if (j > 0) {
+                    const int jf = j - 1;
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float4 d4 = *reinterpret_cast<const float4 *>(dxs + j * 32 + 8 * i + 4 * lh);
-                    dxv[4 * i] = d4.x; dxv[4 * i + 1] = d4.y; dxv[4 * i + 2] = d4.z; dxv[4 * i + 3] = d4.w;
+                    for (int i = 0; i < 4; ++i) {
+                        const float4 d4 = *reinterpret_cast<const float4 *>(dxs + jf * 32 + 8 * i + 4 * lh);
+                        const float dxv[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int v = 4 * i + r;
+                            acc[jf][v] = fmaf((float)((ihi[jf & 1][v] << 8) + ilo[jf & 1][v]), dxv[r] * dn, acc[jf][v]);
+                        }
+                    }
                 }
+                if (j > 0 && j < JT) {   // one matrix instruction, its share of the operand reads, four of the flush instructions
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[j][v] = fmaf((float)((ihi[v] << 8) + ilo[v]), dxv[v] * dn, acc[j][v]);
+                    for (int g = 0; g < 16; ++g) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+                    }
+                }
             }
             if (LATE) {
                 // the next super-block's strip was requested at the top of this trip; of the requests made since then
@@ -415,14 +435,22 @@ __global__ __launch_bounds__(512, 1) void gemm_q6k_q8k_wide_kernel(const WeightV
     if (wave < 4) run(std::false_type{});
     else run(std::true_type{});
 
-    // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32
-    const int64_t n = n0 + wave * 32 + l32;
+    // ---- store: accumulator register v of lane l is row 8*(v/4) + 4*(l/32) + v%4, column l%32 (the lane's coordinates
+    // are worked out again from the thread index, made opaque, so that no address arithmetic is carried through the loop)
+    int tid_s = tid, pid_s = (int)blockIdx.x;
+    asm volatile("" : "+v"(tid_s));
+    asm volatile("" : "+s"(pid_s));
+    int tile_n_s, tile_m_s;
+    tile_of_workgroup((int)((N + TN - 1) / TN), (int)((M + TM - 1) / TM), pid_s, tile_n_s, tile_m_s);
+    const int64_t n0_s = (int64_t)tile_n_s * TN, m0_s = (int64_t)tile_m_s * TM;
+    const int l32_s = tid_s & 31, lh_s = (tid_s >> 5) & 1, wave_s = tid_s >> 6;
+    const int64_t n = n0_s + wave_s * 32 + l32_s;
     float *out = gridDim.y > 1 ? part + (size_t)blockIdx.y * M * N : y;
 #pragma unroll
     for (int j = 0; j < JT; ++j) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const int64_t m = m0 + j * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            const int64_t m = m0_s + j * 32 + 8 * (v >> 2) + 4 * lh_s + (v & 3);
             if (m < M && n < N) out[m * N + n] = acc[j][v];
         }
     }
