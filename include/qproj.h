@@ -150,8 +150,9 @@ int qproj_rms_norm_ffn_gate_up(qproj_ctx *ctx, const qproj_weight *gate, const q
 /* The whole dense feed-forward of llama.cpp's build_ffn (LLM_FFN_SILU, LLM_FFN_PAR), optionally behind the block's
  * RMS norm (use_norm != 0; gamma_dev may be null):
  *     y_dev[M][N] = down . ( silu(gate . x') * (up . x') ),   x' = rms_norm(x) * gamma or x.
- * gate and up are [K -> d_ff], down is [d_ff -> N].  Runs qproj_(rms_norm_)ffn_gate_up into scratch of the context and
- * qproj_mul_mat on the result: two launches for M <= 2, and bit-identical to those two calls. */
+ * gate and up are [K -> d_ff], down is [d_ff -> N].  Bit-identical to qproj_(rms_norm_)ffn_gate_up followed by
+ * qproj_mul_mat: two launches for M <= 2; for batches the swiglu is formed inside the quantizer of the down projection
+ * (gate and up go to scratch of the context, the intermediate rows are never written as fp32). */
 int qproj_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, const qproj_weight *down,
               const float *x_dev, const float *gamma_dev, float eps, int use_norm, int64_t M, float *y_dev, int act);
 

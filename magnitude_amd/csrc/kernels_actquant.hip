@@ -6,20 +6,34 @@
 
 namespace qproj {
 
-__global__ __launch_bounds__(256) void quant_q8k_kernel(const float *__restrict__ x, int64_t n_super,
+// Every quantizer below takes an optional second input `u` of the same shape: the rows quantized are then
+// silu(x) * u, the swiglu that joins the gate and up projections of a feed-forward block (the expression of
+// swiglu_kernel, so the planes are the ones that kernel followed by the plain quantizer would write), and the
+// intermediate rows never go to memory as fp32.
+__device__ __forceinline__ float silu_mul(float x, float u) { return (x / (1.0f + expf(-x))) * u; }
+__device__ __forceinline__ float4 load_rows4(const float *__restrict__ x, const float *__restrict__ u, int64_t e0) {
+    float4 v = *reinterpret_cast<const float4 *>(x + e0);
+    if (u) {   // uniform over the launch
+        const float4 w = *reinterpret_cast<const float4 *>(u + e0);
+        v.x = silu_mul(v.x, w.x); v.y = silu_mul(v.y, w.y); v.z = silu_mul(v.z, w.z); v.w = silu_mul(v.w, w.w);
+    }
+    return v;
+}
+
+__global__ __launch_bounds__(256) void quant_q8k_kernel(const float *__restrict__ x, const float *__restrict__ u, int64_t n_super,
                                                         int8_t *__restrict__ qs, float *__restrict__ d,
                                                         int16_t *__restrict__ bsums) {
     const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (sb >= n_super) return;  // whole wave leaves together
-    const float4 v = reinterpret_cast<const float4 *>(x + sb * 256)[lane];
+    const float4 v = load_rows4(x, u, sb * 256 + 4 * lane);
     wave_store_q8k(v, lane, sb, qs, d, bsums);
 }
 
 // FP16_SCALE: ggml Q8_0 blocks (scale rounded through fp16).  Otherwise the prefill format:
 // fp32 scale plus the integer sum of the block.
 template <bool FP16_SCALE>
-__global__ __launch_bounds__(256) void quant_q8_32_kernel(const float *__restrict__ x, int64_t n_chunks256,
+__global__ __launch_bounds__(256) void quant_q8_32_kernel(const float *__restrict__ x, const float *__restrict__ u, int64_t n_chunks256,
                                                           int64_t n_elems, int8_t *__restrict__ qs,
                                                           float *__restrict__ d, int32_t *__restrict__ isum) {
     const int64_t ch = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -28,7 +42,7 @@ __global__ __launch_bounds__(256) void quant_q8_32_kernel(const float *__restric
     const int64_t e0 = ch * 256 + 4 * lane;
     const bool live = e0 < n_elems;  // rows are multiples of 32, so a block is all in or all out
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (live) v = *reinterpret_cast<const float4 *>(x + e0);
+    if (live) v = load_rows4(x, u, e0);
     wave_store_q8_32<FP16_SCALE>(v, lane, e0, live, qs, d, isum);
 }
 
@@ -88,7 +102,7 @@ __global__ __launch_bounds__(256) void minterm_rows_kernel(const float *__restri
 // Quantizer and min-term operand in one launch: one 16-wave workgroup per activation row; a wave quantizes
 // super-blocks wave, wave + 16, ... of the row.  Dynamic LDS: row_minterm_lds_bytes(PER32, nb).
 template <bool PER32>
-__global__ __launch_bounds__(kRowThreads) void quant_rows_minterm_kernel(const float *__restrict__ x, int nb,
+__global__ __launch_bounds__(kRowThreads) void quant_rows_minterm_kernel(const float *__restrict__ x, const float *__restrict__ u, int nb,
                                                                          int8_t *__restrict__ qs, float *__restrict__ d,
                                                                          int16_t *__restrict__ bsums,
                                                                          int32_t *__restrict__ isum,
@@ -101,7 +115,7 @@ __global__ __launch_bounds__(kRowThreads) void quant_rows_minterm_kernel(const f
     const int64_t m = blockIdx.x;
     for (int sb = wave; sb < nb; sb += kRowWaves) {
         const int64_t g = m * nb + sb;
-        const float4 v = reinterpret_cast<const float4 *>(x + g * 256)[lane];
+        const float4 v = load_rows4(x, u, g * 256 + 4 * lane);
         if constexpr (PER32) wave_store_q8x32_row(v, lane, g, sb, qs, d, isum, ld, ls);
         else wave_store_q8k_row(v, lane, g, sb, qs, d, bsums, ld, ls);
     }
@@ -124,7 +138,7 @@ hipError_t launch_minterm_rows(int kind, const float *d, const int16_t *bsums, c
 // msum / rs null: the min-term plane is not wanted (the decode, small-batch and expert-grouped kernels take the block
 // sums themselves)
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
-                               int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s) {
+                               int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s, const float *u) {
     const int64_t n = M * K;
     if (n == 0) return hipSuccess;
     if (kind != kActKindQ8_K && kind != kActKindQ8_0 && kind != kActKindQ8X32) return hipErrorInvalidValue;
@@ -138,19 +152,19 @@ hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, i
         const int nb = (int)(K / 256);
         const dim3 rgrid((unsigned)M), rblock(kRowThreads);
         if (kind == kActKindQ8_K)
-            hipLaunchKernelGGL(quant_rows_minterm_kernel<false>, rgrid, rblock, row_minterm_lds_bytes(false, nb), s, x, nb, qs, d, bsums, isum, msum, rs);
+            hipLaunchKernelGGL(quant_rows_minterm_kernel<false>, rgrid, rblock, row_minterm_lds_bytes(false, nb), s, x, u, nb, qs, d, bsums, isum, msum, rs);
         else
-            hipLaunchKernelGGL(quant_rows_minterm_kernel<true>, rgrid, rblock, row_minterm_lds_bytes(true, nb), s, x, nb, qs, d, bsums, isum, msum, rs);
+            hipLaunchKernelGGL(quant_rows_minterm_kernel<true>, rgrid, rblock, row_minterm_lds_bytes(true, nb), s, x, u, nb, qs, d, bsums, isum, msum, rs);
         return hipGetLastError();
     }
     const int64_t chunks = (n + 255) / 256;
     const dim3 grid((unsigned)((chunks + 3) / 4)), block(256);
     if (kind == kActKindQ8_K) {
-        hipLaunchKernelGGL(quant_q8k_kernel, grid, block, 0, s, x, n / 256, qs, d, bsums);
+        hipLaunchKernelGGL(quant_q8k_kernel, grid, block, 0, s, x, u, n / 256, qs, d, bsums);
     } else if (kind == kActKindQ8_0) {
-        hipLaunchKernelGGL(quant_q8_32_kernel<true>, grid, block, 0, s, x, chunks, n, qs, d, isum);
+        hipLaunchKernelGGL(quant_q8_32_kernel<true>, grid, block, 0, s, x, u, chunks, n, qs, d, isum);
     } else {
-        hipLaunchKernelGGL(quant_q8_32_kernel<false>, grid, block, 0, s, x, chunks, n, qs, d, isum);
+        hipLaunchKernelGGL(quant_q8_32_kernel<false>, grid, block, 0, s, x, u, chunks, n, qs, d, isum);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || kind == kActKindQ8_0 || !msum) return e;

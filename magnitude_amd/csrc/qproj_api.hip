@@ -207,14 +207,14 @@ RowQuantJob quantize_job(const ActPlanes &p, uint8_t *base, const float *x, int6
 
 // minterm: also the min-term plane and the row normalisers that only the tiled Q4_K kernels read (a second, small launch)
 hipError_t run_quantize(qproj_ctx *ctx, const ActPlanes &p, uint8_t *base, const float *x, int64_t M, int64_t K,
-                        bool minterm = true) {
+                        bool minterm = true, const float *swiglu_u = nullptr) {
     const bool mt = minterm && (p.kind == kActKindQ8_K || p.kind == kActKindQ8X32);
     return launch_quantize_act(p.kind, x, M, K, reinterpret_cast<int8_t *>(base + p.off_qs),
                                reinterpret_cast<float *>(base + p.off_d),
                                reinterpret_cast<int16_t *>(base + p.off_aux),
                                mt ? reinterpret_cast<uint16_t *>(base + p.off_msum) : nullptr,
                                reinterpret_cast<int32_t *>(base + p.off_aux),
-                               mt ? reinterpret_cast<float *>(base + p.off_rs) : nullptr, ctx->stream);
+                               mt ? reinterpret_cast<float *>(base + p.off_rs) : nullptr, ctx->stream, swiglu_u);
 }
 
 ActView act_rows(const ActView &a, int64_t m0) {
@@ -767,8 +767,21 @@ struct NormSpec {   // RMS norm (+ weights) applied to the rows before they are 
 };
 }  // namespace
 
+// Can the down projection of a feed-forward block take its rows as silu(gate) * up through the quantizer?  Only the
+// routes that quantize in a launch of their own (not the decode kernel, whose prologue reads fp32 rows, nor the
+// small-batch variant that quantizes inside the projection, nor fp32 activations).
+static bool swiglu_quantizer_serves(const qproj_weight *w, int64_t M, int act) {
+    if (act != kActGGML && act != kActQ8X32) return false;
+    if (act == kActQ8X32) return w->type == kTypeQ4_K && w->K % 256 == 0;
+    if (!use_mfma_kernel(w->type, M, w->K) && use_decode_kernel(w->type, M, w->K)) return false;
+    return !dense_fuses_quantizer(w, M);
+}
+
+// swiglu_u non-null (callers: the quantized routes beyond the decode regime only): the rows multiplied are
+// silu(x_dev) * swiglu_u, formed inside the quantizer
 static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
-                              float *const *y_dev, int act, const NormSpec *norm, Workspace &wsp) {
+                              float *const *y_dev, int act, const NormSpec *norm, Workspace &wsp,
+                              const float *swiglu_u = nullptr) {
     if (!ctx) return QPROJ_ERR_INVALID_ARG;
     if (n <= 0 || n > kMaxTargets || !w || !y_dev || !x_dev)
         return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat: null argument or more than 4 tensors");
@@ -782,6 +795,8 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
     if (M == 0) return QPROJ_OK;
     if (!dry_run()) QP_HIP(ctx, hipSetDevice(ctx->device));
     const int64_t K = w[0]->K;
+    if (swiglu_u && (norm || !swiglu_quantizer_serves(w[0], M, act)))
+        return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj: the fused swiglu needs a quantized route beyond the decode regime");
     if (act == kActGGML && !use_mfma_kernel(w[0]->type, M, K) && use_decode_kernel(w[0]->type, M, K) &&
         (!norm || decode_kernel_norm_fits(pow2_ceil(M), K))) {
         // decode regime: the kernel (normalises and) quantizes the activation rows itself, no scratch needed
@@ -803,7 +818,7 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
     if (act == kActGGML || act == kActQ8X32) {
         if (act == kActQ8X32 && w[0]->type != kTypeQ4_K)
             return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat: the per-32 int8 path is built for Q4_K weights");
-        if (act == kActGGML && !norm && dense_fuses_quantizer(w[0], M)) {
+        if (act == kActGGML && !norm && !swiglu_u && dense_fuses_quantizer(w[0], M)) {
             const size_t extra = dense_scratch_bytes(n, w, M);
             int rc = reserve(ctx, wsp, extra);
             if (rc) return rc;
@@ -829,7 +844,7 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
                                         reinterpret_cast<int32_t *>(ws + p.off_aux),
                                         minterm ? reinterpret_cast<float *>(ws + p.off_rs) : nullptr, ctx->stream));
         } else {
-            QP_HIP(ctx, run_quantize(ctx, p, ws, x_dev, M, K, minterm));
+            QP_HIP(ctx, run_quantize(ctx, p, ws, x_dev, M, K, minterm, swiglu_u));
         }
         const ActView a = act_view(p, ws, K);
         // the partial results lie behind the activation planes; `extra` is all a launcher may use of it
@@ -995,6 +1010,21 @@ int qproj_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, 
     int rc = ensure_ws2(ctx, (size_t)3 * M * d_ff * 4);
     if (rc) return rc;
     float *h = reinterpret_cast<float *>(ctx->ws2) + (size_t)2 * M * d_ff;
+    const bool gate_up_decode = act == kActGGML && M <= 2 && !use_mfma_kernel(gate->type, M, gate->K) &&
+                                use_decode_kernel(gate->type, M, gate->K);
+    if (!gate_up_decode && swiglu_quantizer_serves(down, M, act)) {
+        // batches: gate and up into scratch, then the down projection's quantizer forms silu(gate) * up itself -
+        // the intermediate rows are never written as fp32 (the planes are bit for bit those of the separate calls)
+        float *gu[2] = {reinterpret_cast<float *>(ctx->ws2), reinterpret_cast<float *>(ctx->ws2) + (size_t)M * d_ff};
+        const qproj_weight *ws[2] = {gate, up};
+        Workspace wsp = ctx_workspace(ctx);
+        rc = mul_mat_multi_impl(ctx, 2, ws, x_dev, M, gu, act, use_norm ? &norm : nullptr, wsp);
+        if (rc) return rc;
+        const qproj_weight *wd[1] = {down};
+        float *yd[1] = {y_dev};
+        Workspace wsp2 = ctx_workspace(ctx);
+        return mul_mat_multi_impl(ctx, 1, wd, gu[0], M, yd, act, nullptr, wsp2, gu[1]);
+    }
     rc = ffn_gate_up_impl(ctx, gate, up, x_dev, M, h, act, use_norm ? &norm : nullptr);
     if (rc) return rc;
     return qproj_mul_mat(ctx, down, h, M, y_dev, act);

@@ -111,8 +111,10 @@ hipError_t launch_repack_to_gguf(int type, const WeightView &w, uint8_t *gguf, i
 // (msum and rs may be null together: the min-term plane of the tiled Q4_K kernels is then not made)
 hipError_t launch_rms_norm(int kind, const float *x, const float *gamma, float eps, int64_t M, int64_t K, float *y,
                            int8_t *qs, float *d, int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s);
+// u non-null: the rows quantized are silu(x) * u (the swiglu between gate / up and the down projection)
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
-                               int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s);
+                               int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s,
+                               const float *u = nullptr);
 // the min-term plane and the row normalisers from planes already quantized (one wave per row)
 hipError_t launch_minterm_rows(int kind, const float *d, const int16_t *bsums, const int32_t *isum, int64_t M, int64_t K,
                                uint16_t *msum, float *rs, hipStream_t s);

@@ -904,12 +904,14 @@ def test_q6k_prefill_extreme_codes_and_scales(ctx, orc, m):
     assert np.all(np.abs(want[:, :96] - exact) <= 1e-6 * mass + 1e-30)     # the oracle meets the same bar
     w.free()
 
-@pytest.mark.parametrize("down_type", [Q4_K, Q6_K])
-@pytest.mark.parametrize("m", [1, 2, 5])
+@pytest.mark.parametrize("down_type", [Q4_K, Q6_K, Q8_0])
+@pytest.mark.parametrize("m", [1, 2, 5, 20, 40, 150])
 def test_ffn_equals_the_chain_and_the_oracle(ctx, orc, down_type, m):
     """qproj_ffn = norm -> gate/up -> swiglu -> down: bit for bit what qproj_(rms_norm_)ffn_gate_up followed by
     qproj_mul_mat gives, with and without the norm, on calls in a row; against the CPU restatement at the
-    re-quantized-intermediate bar of the MoE feed-forward (2e-4)."""
+    re-quantized-intermediate bar of the MoE feed-forward (2e-4).  Beyond two rows the swiglu is formed inside the
+    down projection's quantizer (5: small-batch kernel; 20, 40, 150: tiled kernels, with the min-term plane for
+    Q4_K, from the plain quantizer and from the one that takes a workgroup per row)."""
     from magnitude_amd import ACT_GGML
     for d_model, d_ff in ((512, 768), (4096, 2048)):
         rng = np.random.default_rng(7000 + d_model + d_ff + m + down_type)
@@ -934,8 +936,19 @@ def test_ffn_equals_the_chain_and_the_oracle(ctx, orc, down_type, m):
         hh = (go / (1.0 + np.exp(-go.astype(np.float64)))).astype(np.float32) * uo
         ref = orc.mul_mat(down_type, down_b, d_ff, hh, orc.ACT_GGML)
         got = ctx.ffn(wg, wu, wd, xs[0], ACT_GGML).cpu().numpy()
-        close(got, ref, 2e-4)
-        gate(got, ref)
+        # The intermediate rows differ from the oracle's in the last bits (fp32 association of gate / up), so now and then
+        # a code of their re-quantization flips: one step of one code is d_x * w, up to 5e-3 of an output of this size.
+        # A few rows rarely hold one (the 2e-4 bar of the MoE feed-forward); 150 rows x 2048 values hold a few, and a
+        # Q8_0 block (a scale per 32) steps coarser.  There the two halves are held to the oracle one by one instead:
+        # the intermediate rows at 5e-5, and the result against the oracle's down projection of THOSE rows at 5e-5
+        # (the call itself is bitwise the chain, shown above).
+        if m <= 5 and down_type != Q8_0:
+            close(got, ref, 2e-4)
+            gate(got, ref)
+        else:
+            h_gpu = ctx.ffn_gate_up(wg, wu, xs[0], ACT_GGML).cpu().numpy()
+            close(h_gpu, hh, 5e-5)
+            close(got, orc.mul_mat(down_type, down_b, d_ff, h_gpu, orc.ACT_GGML), 5e-5)
         for w in (wg, wu, wd):
             w.free()
 
