@@ -952,6 +952,29 @@ def test_ffn_equals_the_chain_and_the_oracle(ctx, orc, down_type, m):
         for w in (wg, wu, wd):
             w.free()
 
+@pytest.mark.parametrize("m", [1, 3, 40, 150])
+def test_ffn_in_the_per32_format_equals_the_chain(ctx, orc, m):
+    """qproj_ffn with per-32 int8 activations (Q4_K tensors): bit for bit qproj_ffn_gate_up followed by qproj_mul_mat
+    in the same format, with and without the norm - the swiglu inside the quantizer writes the planes the
+    elementwise pass followed by the plain quantizer writes."""
+    from magnitude_amd import ACT_Q8X32
+    d_model, d_ff = 512, 768
+    rng = np.random.default_rng(7700 + m)
+    wg = ctx.upload(Q4_K, d_model, d_ff, make_weight(orc, Q4_K, d_ff, d_model, seed=7701))
+    wu = ctx.upload(Q4_K, d_model, d_ff, make_weight(orc, Q4_K, d_ff, d_model, seed=7702))
+    wd = ctx.upload(Q4_K, d_ff, d_model, make_weight(orc, Q4_K, d_model, d_ff, seed=7703))
+    gam = dev((1.0 + 0.1 * rng.standard_normal(d_model)).astype(np.float32))
+    x = dev(rng.standard_normal((m, d_model)).astype(np.float32))
+    for norm in (False, True):
+        kw = dict(gamma=gam, eps=1e-5) if norm else {}
+        y = ctx.ffn(wg, wu, wd, x, ACT_Q8X32, **kw)
+        want = ctx.mul_mat(wd, ctx.ffn_gate_up(wg, wu, x, ACT_Q8X32, **kw), ACT_Q8X32)
+        assert torch.equal(y.view(torch.int32), want.view(torch.int32)), f"norm={norm}"
+        assert float(y.abs().sum()) > 0
+    for w in (wg, wu, wd):
+        w.free()
+
+
 @pytest.mark.parametrize("act_name", ["ggml", "q8x32"])
 @pytest.mark.parametrize("m", [64, 200])
 def test_tiled_q4k_products_over_a_wide_range_of_activation_scales(ctx, orc, m, act_name):
