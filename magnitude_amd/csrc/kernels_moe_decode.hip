@@ -1,0 +1,277 @@
+// MUL_MAT_ID for one or two decode tokens (at most 16 (token, expert) pairs) on the vector ALU: no grouping
+// pass, no matrix cores, no separate quantizer or combine launch.
+//
+// Every pair has its own expert matrix and, for the down projection, its own activation row, so the launch is
+// a set of independent short GEMVs: a workgroup of 16 waves serves a run of weight rows for a GROUP of pairs
+// (one pair; or the n_used pairs of one token when their results are combined here).  It quantizes the
+// group's activation rows into LDS with the arithmetic of the standalone quantizer, and its waves then walk
+// (pair, row step) units.  Expert rows are short (K = 768 .. 4096), so a step covers S = 64 / (4 K/256) whole
+// rows at once: lane = (row slot, super-block, quarter of the super-block), the row slots' partial dot products
+// are summed over their own lanes only.  Consecutive rows of a matrix are consecutive in memory, so a step's
+// loads cover one contiguous stretch.  With gate and up given, a step walks the same rows of both and stores
+// silu(gate . x) * (up . x); with routing weights given, the workgroup adds its pairs' results in slot order,
+// each product rounded first, which is what the separate combine pass does.
+#include <algorithm>
+
+#include "actquant_device.h"
+#include "gemv_frags.h"
+
+namespace qproj {
+
+namespace {
+
+constexpr int kThreads = 1024, kWaves = kThreads / 64;
+constexpr int kMaxGroup = 16;
+
+struct MoeDecodeArgs {
+    WeightView w0, w1;       // w1: the up tensor when gate / up are paired
+    const float *x;          // fp32 activation rows [.][K]
+    int x_div;               // the activation row of pair p is p / x_div
+    const int32_t *ids;      // expert of pair p
+    int n_pairs, n_expert;
+    int32_t *error_flag;
+    float *y;                // [n_pairs][N]; with routing weights [n_pairs / group][N]
+    const float *cw;         // routing weights [n_pairs], or null
+    int group;               // pairs a workgroup serves
+    int wgs_per_group;       // workgroups that share the rows of a group
+    int rows_per_wg;         // a multiple of the rows a step covers
+};
+
+// sum of v over the `lpr` lanes of each row slot (lpr a multiple of 4); valid in the slot's first lane
+__device__ __forceinline__ float slot_sum(float v, int vlane, int lpr) {
+    v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+#pragma unroll
+    for (int o = 32; o >= 4; o >>= 1) {
+        if (o < lpr) {   // wave-uniform
+            const float t = __shfl_down(v, o);
+            if (vlane + o < lpr) v += t;
+        }
+    }
+    return v;
+}
+
+template <int QT, bool SWIGLU, bool COMBINE>
+__global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArgs g) {
+    extern __shared__ __align__(16) uint8_t smem[];
+    constexpr int NT = SWIGLU ? 2 : 1;
+    const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6);
+    const int K = (int)g.w0.K, nb = (int)g.w0.nb, N = (int)g.w0.N;
+    const int lpr = 4 * nb, S = 64 / lpr;
+    const bool live = lane < S * lpr;
+    const int slot = live ? lane / lpr : 0;
+    const int vlane = live ? lane - slot * lpr : 0;   // idle lanes repeat a valid address and add nothing
+    const int grp = (int)blockIdx.x / g.wgs_per_group, j = (int)blockIdx.x - grp * g.wgs_per_group;
+    const int p0 = grp * g.group, G = g.group;
+    const int r0 = j * g.rows_per_wg;
+    const int r1 = min(N, r0 + g.rows_per_wg);
+    const int steps = r1 > r0 ? (r1 - r0 + S - 1) / S : 0;
+    const int units = G * steps;
+    const int n_u = units > wave ? (units - wave + kWaves - 1) / kWaves : 0;   // this wave's units: wave, wave + 16, ..
+
+    // LDS: the group's quantized activation rows, then the results to combine
+    int8_t *sq = reinterpret_cast<int8_t *>(smem);
+    const int d_bytes = (G * nb * 4 + 15) & ~15;   // the block sums behind it are read eight bytes at a time
+    float *sd = reinterpret_cast<float *>(smem + G * K);
+    int16_t *sb = reinterpret_cast<int16_t *>(smem + G * K + d_bytes);
+    float *res = reinterpret_cast<float *>(smem + G * K + d_bytes + G * (K / 16) * 2);
+    float *cwl = res + G * g.rows_per_wg;
+    XTile xt;
+    xt.qs = sq;
+    xt.d = sd;
+    xt.bs = sb;
+    xt.kt = K;
+
+    // the wave's first piece of the activation rows is requested ahead of its first weights (loads return in order)
+    const int n_chunks = G * nb;
+    constexpr int kAhead = 2;
+    float4 x_first[kAhead];
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) {
+        const int c = wave + kWaves * a;
+        x_first[a] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c < n_chunks) {
+            const int s = c / nb, ch = c - s * nb;
+            x_first[a] = *reinterpret_cast<const float4 *>(g.x + (int64_t)((p0 + s) / g.x_div) * K + ch * 256 + 4 * lane);
+        }
+    }
+    float cw_mine = 0.f;   // routing weights go through LDS: the adding threads would otherwise wait for them at the very end
+    if (COMBINE && tid < G) cw_mine = g.cw[p0 + tid];
+    if (j == 0 && tid < G) {   // one workgroup of the group reports ids that name no expert
+        const int e = g.ids[p0 + tid];
+        if (e < 0 || e >= g.n_expert) atomicOr(g.error_flag, 1);
+    }
+
+    // unit u = (pair s of the group, row step st): experts are read by the wave itself (scalar loads)
+    struct Unit {
+        int s, row, expert;
+        bool ok;
+    };
+    auto unit_of = [&](int i) {
+        Unit u;
+        const int idx = wave + kWaves * i;
+        u.s = idx / steps;
+        u.row = r0 + (idx - u.s * steps) * S;
+        const int e = uniform(g.ids[p0 + u.s]);
+        u.ok = e >= 0 && e < g.n_expert;
+        u.expert = u.ok ? e : 0;   // a pair without an expert is left out; its loads go somewhere valid
+        return u;
+    };
+    auto issue = [&](Raw<QT> (&raw)[NT], int i) {
+        const Unit u = unit_of(i);
+        RowPtr<QT> rp;
+        rp.set(g.w0, (int64_t)u.expert * N + u.row);
+        const uint32_t rel = (uint32_t)min(slot, r1 - 1 - u.row);
+        raw[0].load(rp, (uint32_t)(vlane >> 2), vlane, rel);
+        if constexpr (SWIGLU) {
+            RowPtr<QT> ru;
+            ru.set(g.w1, (int64_t)u.expert * N + u.row);
+            raw[NT - 1].load(ru, (uint32_t)(vlane >> 2), vlane, rel);
+        }
+    };
+    auto consume = [&](const Raw<QT> (&raw)[NT], int i) {
+        const Unit u = unit_of(i);
+        Dot<QT> dx;
+        dx.load_x(xt, u.s, 0, vlane);
+        float acc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            Frag<QT> f;
+            f.unpack(raw[t], vlane);
+            acc[t] = slot_sum(live ? dx.dot(f) : 0.f, vlane, lpr);
+        }
+        const int row = u.row + slot;
+        if (live && vlane == 0 && row < r1) {
+            float r = acc[0];
+            if constexpr (SWIGLU) r = (r / (1.0f + expf(-r))) * acc[NT - 1];
+            if constexpr (COMBINE) res[u.s * g.rows_per_wg + (row - r0)] = u.ok ? r : 0.f;
+            else if (u.ok) g.y[(int64_t)(p0 + u.s) * N + row] = r;
+        }
+    };
+
+    Raw<QT> buf_a[NT], buf_b[NT];
+    if (n_u > 0) issue(buf_a, 0);   // in flight while the activations are quantized
+
+    if (COMBINE && tid < G) cwl[tid] = cw_mine;
+    for (int c = wave, a = 0; c < n_chunks; c += kWaves, ++a) {
+        const int s = c / nb, ch = c - s * nb;
+        float4 v = x_first[kAhead - 1];
+        if (a == 0) v = x_first[0];
+        else if (a >= kAhead) v = *reinterpret_cast<const float4 *>(g.x + (int64_t)((p0 + s) / g.x_div) * K + ch * 256 + 4 * lane);
+        int bsum;
+        float dd;
+        const uint32_t packed = wave_quantize_q8k(v, lane, bsum, dd);
+        *reinterpret_cast<uint32_t *>(sq + s * K + ch * 256 + 4 * lane) = packed;
+        if ((lane & 3) == 0) sb[s * (K / 16) + ch * 16 + (lane >> 2)] = (int16_t)bsum;
+        if (lane == 0) sd[s * nb + ch] = dd;
+    }
+    __syncthreads();
+
+    // two register buffers, the next unit's loads outstanding while this one is multiplied; no load is issued twice
+    int i = 0;
+    for (; i + 2 < n_u; i += 2) {
+        issue(buf_b, i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        consume(buf_a, i);
+        issue(buf_a, i + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        consume(buf_b, i + 1);
+    }
+    if (i + 1 < n_u) {
+        issue(buf_b, i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        consume(buf_a, i);
+        consume(buf_b, i + 1);
+    } else if (i < n_u) {
+        consume(buf_a, i);
+    }
+
+    if constexpr (COMBINE) {
+        __syncthreads();
+        if (tid < r1 - r0) {
+            float s = __fmul_rn(res[tid], cwl[0]);
+            for (int q = 1; q < G; ++q) s = __fadd_rn(s, __fmul_rn(res[q * g.rows_per_wg + tid], cwl[q]));
+            g.y[(int64_t)grp * N + r0 + tid] = s;
+        }
+    }
+}
+
+int cu_count() {
+    static int n = [] {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+        return v;
+    }();
+    return n;
+}
+
+template <int QT, bool SWIGLU, bool COMBINE>
+hipError_t launch_typed(const MoeDecodeArgs &g, unsigned grid, size_t lds, hipStream_t s) {
+    auto kern = &moe_decode_kernel<QT, SWIGLU, COMBINE>;
+    static size_t allowed = 48 * 1024;
+    if (lds > allowed) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        allowed = lds;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), lds, s, g);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool moe_decode_fits(int type, int64_t K, int64_t n_pairs, int64_t group) {
+    return (type == kTypeQ4_K || type == kTypeQ6_K) && K % 256 == 0 && K >= 256 && K <= 4096 && n_pairs >= 1 &&
+           n_pairs <= (1 << 20) && group >= 1 && group <= kMaxGroup && n_pairs % group == 0;
+}
+
+// args: t[0] (and t[1] = up when swiglu) expert stacks, x fp32 rows, x_div, ids, n_pairs, error_flag as for the
+// pair mode of the grouped kernel; n_expert experts a stack.  combine_weights null: t[0].y is [n_pairs][N].
+// Otherwise the pairs of a token (n_used of them, consecutive) are added with their routing weights and
+// t[0].y is [n_pairs / n_used][N].
+hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, const float *combine_weights, int n_used,
+                             hipStream_t s) {
+    const WeightView &w = args.t[0].w;
+    const int group = combine_weights ? n_used : 1;
+    if (!moe_decode_fits(w.type, w.K, args.n_pairs, group) || !args.x || !args.ids || !args.error_flag || args.x_div < 1 ||
+        n_expert < 1 || w.N < 1 || w.N > (1 << 24) || (swiglu && combine_weights))
+        return hipErrorInvalidValue;
+    if (swiglu && (args.n_targets != 2 || args.t[1].w.type != w.type || args.t[1].w.K != w.K || args.t[1].w.N != w.N))
+        return hipErrorInvalidValue;
+    MoeDecodeArgs g{};
+    g.w0 = w;
+    g.w1 = swiglu ? args.t[1].w : w;
+    g.x = args.x;
+    g.x_div = args.x_div;
+    g.ids = args.ids;
+    g.n_pairs = args.n_pairs;
+    g.n_expert = n_expert;
+    g.error_flag = args.error_flag;
+    g.y = args.t[0].y;
+    g.cw = combine_weights;
+    g.group = group;
+    const int nb = (int)w.nb, S = 64 / (4 * nb);
+    const int n_groups = args.n_pairs / group;
+    const int64_t steps_total = (w.N + S - 1) / S;
+    // The launch is latency-bound (all loads of the call are in flight at once): the rows are spread over all
+    // compute units, a unit or two a wave, at least half the waves of a workgroup busy.  The registers of a 16-wave
+    // workgroup leave room for one a compute unit, so the grid stays within one round.
+    const int64_t max_wgs = std::max<int64_t>(1, (int64_t)cu_count() / n_groups);
+    const int64_t steps_per_wg = std::max<int64_t>((steps_total + max_wgs - 1) / max_wgs, std::max<int64_t>(1, kWaves / 2 / group));
+    g.rows_per_wg = (int)(steps_per_wg * S);
+    g.wgs_per_group = (int)((w.N + g.rows_per_wg - 1) / g.rows_per_wg);
+    if (combine_weights && g.rows_per_wg > kThreads) return hipErrorInvalidValue;   // one thread adds one output row
+    const size_t lds = (size_t)group * w.K + (((size_t)group * nb * 4 + 15) & ~(size_t)15) + (size_t)group * (w.K / 16) * 2 +
+                       (combine_weights ? (size_t)group * (g.rows_per_wg + 1) * 4 : 0);
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    if (dry_run()) return hipSuccess;
+    const unsigned grid = (unsigned)(n_groups * g.wgs_per_group);
+    if (w.type == kTypeQ4_K) {
+        if (swiglu) return launch_typed<kTypeQ4_K, true, false>(g, grid, lds, s);
+        return combine_weights ? launch_typed<kTypeQ4_K, false, true>(g, grid, lds, s) : launch_typed<kTypeQ4_K, false, false>(g, grid, lds, s);
+    }
+    if (swiglu) return launch_typed<kTypeQ6_K, true, false>(g, grid, lds, s);
+    return combine_weights ? launch_typed<kTypeQ6_K, false, true>(g, grid, lds, s) : launch_typed<kTypeQ6_K, false, false>(g, grid, lds, s);
+}
+
+}  // namespace qproj

@@ -146,6 +146,13 @@ hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_exper
                             int32_t *offsets, int32_t *active, int32_t *error_flag, const RowQuantJob *quantize,
                             hipStream_t s);
 hipError_t launch_moe_swiglu_gemv(const GemvArgs &gate_up, int mt, int n_experts_grid, hipStream_t s);
+// One or two decode tokens (at most 16 pairs) through expert stacks of Q4_K / Q6_K rows of K <= 4096 on the vector
+// ALU: args as for the pair mode of the grouped kernel (t[0], and t[1] = up when `swiglu`; x fp32 rows, x_div, ids,
+// n_pairs, error_flag).  combine_weights null: t[0].y is [n_pairs][N]; otherwise the n_used consecutive pairs of a
+// token are added with their routing weights in slot order and t[0].y is [n_pairs / n_used][N].
+bool moe_decode_fits(int type, int64_t K, int64_t n_pairs, int64_t group);
+hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, const float *combine_weights, int n_used,
+                             hipStream_t s);
 hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, int64_t n_used, int64_t N,
                               float *y, hipStream_t s);
 // `scratch`: per32_scratch_bytes(K, M, N) bytes (null: K is never split)

@@ -4,7 +4,7 @@ use std::{env, path::PathBuf, process::Command};
 
 const SOURCES: &[&str] = &[
     "qproj_api.hip", "kernels_dequant.hip", "kernels_actquant.hip", "kernels_gemv.hip", "kernels_decode.hip",
-    "kernels_gemv_mfma.hip", "kernels_gemv_f32.hip", "kernels_moe.hip", "kernels_gemm.hip", "kernels_gemm_q6k.hip",
+    "kernels_gemv_mfma.hip", "kernels_gemv_f32.hip", "kernels_moe.hip", "kernels_moe_decode.hip", "kernels_gemm.hip", "kernels_gemm_q6k.hip",
     "kernels_rmsnorm.hip",
 ];
 const HEADERS: &[&str] = &[

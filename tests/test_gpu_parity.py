@@ -521,6 +521,81 @@ def test_moe_ffn_many_experts(ctx, orc, moe, E):
     assert np.median(np.abs(got - want)) <= 1e-6 * np.abs(want).max()
 
 
+@pytest.mark.parametrize("B,E", [(1, 128), (2, 128), (4, 128), (8, 128), (2, 16), (5, 40)])
+def test_moe_ffn_few_tokens_take_an_expert_per_pair(ctx, orc, moe, B, E):
+    """Decode-sized batches (at most 64 pairs and no more pairs than experts, or up to 16 pairs): the route that
+    needs no grouping pass - a set of workgroups per pair reads ids[p] itself, quantizes the pair's activation row,
+    and the down projection adds a token's pairs with their routing weights in slot order.  One unit a wave at one
+    token, several pipelined units a wave at eight."""
+    from magnitude_amd import ACT_GGML
+    d_model, d_ff, top = moe["d_model"], moe["d_ff"], 8
+    rng = np.random.default_rng(700 + 10 * B + E)
+    pick = rng.integers(0, moe["E"], size=E)          # the fixture's 16 experts, repeated
+    gate_b, up_b, down_b = (np.ascontiguousarray(moe[k][pick]) for k in ("gate", "up", "down"))
+    ids, wts = routing(rng, B, top, E)
+    if B > 1:
+        ids[1, :3] = ids[0, :3]                        # experts that come twice are simply read twice
+    x = rng.standard_normal((B, d_model)).astype(np.float32)
+    g = ctx.upload(Q4_K, d_model, d_ff, gate_b, n_expert=E)
+    u = ctx.upload(Q4_K, d_model, d_ff, up_b, n_expert=E)
+    d = ctx.upload(Q4_K, d_ff, d_model, down_b, n_expert=E)
+    got = ctx.moe_ffn(g, u, d, dev(x), dev(ids), dev(wts), ACT_GGML).cpu().numpy()
+    want = orc.moe_ffn(Q4_K, Q4_K, gate_b, up_b, down_b, d_model, d_ff, E, x, ids, wts, orc.ACT_GGML)
+    close(got, want, 1e-3)      # a re-quantized code of the intermediate may move by one step (last bit of expf)
+    gate(got, want)
+    assert np.median(np.abs(got - want)) <= 1e-6 * np.abs(want).max()
+    for t in (g, u, d):
+        t.free()
+
+
+@pytest.mark.parametrize("d_model,d_ff,top,B,down_t", [(1024, 1280, 3, 2, Q6_K), (4096, 256, 1, 1, Q4_K), (256, 4096, 2, 3, Q6_K),
+                                                        (1280, 768, 8, 1, Q4_K), (2048, 512, 16, 1, Q6_K), (768, 1024, 5, 3, Q4_K)])
+def test_moe_ffn_expert_per_pair_shapes(ctx, orc, d_model, d_ff, top, B, down_t):
+    """The same route over the row lengths it maps differently: 1 to 16 whole rows a wave step (K = 4096 .. 256),
+    steps whose lanes do not fill the wave (K = 768, 1280: 5 and 3 rows of 12 and 20 lanes), row counts that leave
+    the last step ragged, 1 to 16 pairs a token, Q6_K down experts."""
+    from magnitude_amd import ACT_GGML
+    E = 24
+    rng = np.random.default_rng(d_model + d_ff + top)
+    enc = lambda t, rows, cols: encode(t, (rng.standard_normal((E * rows, cols)) * 0.03).astype(np.float32)).reshape(E, rows, -1)
+    gate_b, up_b, down_b = enc(Q4_K, d_ff, d_model), enc(Q4_K, d_ff, d_model), enc(down_t, d_model, d_ff)
+    ids, wts = routing(rng, B, top, E)
+    x = rng.standard_normal((B, d_model)).astype(np.float32)
+    g = ctx.upload(Q4_K, d_model, d_ff, gate_b, n_expert=E)
+    u = ctx.upload(Q4_K, d_model, d_ff, up_b, n_expert=E)
+    d = ctx.upload(down_t, d_ff, d_model, down_b, n_expert=E)
+    got = ctx.moe_ffn(g, u, d, dev(x), dev(ids), dev(wts), ACT_GGML).cpu().numpy()
+    want = orc.moe_ffn(Q4_K, down_t, gate_b, up_b, down_b, d_model, d_ff, E, x, ids, wts, orc.ACT_GGML)
+    close(got, want, 1e-3)
+    gate(got, want)
+    assert np.median(np.abs(got - want)) <= 2e-6 * np.abs(want).max()
+    for t in (g, u, d):
+        t.free()
+
+
+@pytest.mark.parametrize("qtype,k,n", [(Q4_K, 768, 100), (Q6_K, 1280, 37), (Q4_K, 4096, 5), (Q6_K, 256, 333)])
+def test_mul_mat_id_expert_per_pair_ragged_rows(ctx, orc, qtype, k, n):
+    """MUL_MAT_ID alone on that route: row counts that are no multiple of the rows a step covers, a shared activation
+    row per token and one per slot, and an id that names no expert (reported, the context stays usable)."""
+    from magnitude_amd import ACT_GGML, QprojError
+    E, top, B = 12, 4, 3
+    rng = np.random.default_rng(k + n)
+    blocks = encode(qtype, (rng.standard_normal((E * n, k)) * 0.05).astype(np.float32)).reshape(E, n, -1)
+    w = ctx.upload(qtype, k, n, blocks, n_expert=E)
+    ids, _ = routing(rng, B, top, E)
+    for rows in (1, top):
+        x = rng.standard_normal((B, rows, k)).astype(np.float32)
+        got = ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML).cpu().numpy()
+        close(got, orc.mul_mat_id(qtype, blocks, k, n, E, x, ids), 2e-5)
+    bad = ids.copy()
+    bad[1, 2] = E
+    with pytest.raises(QprojError):
+        ctx.mul_mat_id(w, dev(x), dev(bad), ACT_GGML)
+    got = ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML).cpu().numpy()
+    close(got, orc.mul_mat_id(qtype, blocks, k, n, E, x, ids), 2e-5)
+    w.free()
+
+
 # ---------------------------------------------------------------- RMS norm in front of the projections
 
 @pytest.mark.parametrize("m,k", [(1, 4096), (5, 14336), (3, 20480), (7, 288), (64, 4096)])
