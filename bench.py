@@ -628,9 +628,9 @@ def main():
                 f"({res[-1]['GBps']:.0f} GB/s from HBM); one draw replayed: {ms1 * 1e3:.1f} us ({res[-1]['cache_resident']['GBps']:.0f} GB/s, "
                 f"{byts1 / 1e6:.0f} MB, may sit in the Infinity Cache)")
         out["moe"] = {"experts": E, "top": top, "d_model": dm, "d_ff": dff, "batches": res,
-                      "note": "3 to 6 launches per call ([quantize,] [group,] gate/up+SwiGLU, [quantize,] down, combine: the grouped "
-                              "kernel quantizes its own rows when experts have few pairs, and skips the grouping pass for "
-                              "up to 16 pairs); the rotation over three weight sets and several id draws is replayed as one "
+                      "note": "2 launches per call up to 64 pairs (gate/up+SwiGLU, down+combine: an expert read per pair, rows "
+                              "quantized in the prologue), else 5 (group+quantize, gate/up+SwiGLU, quantize, down, combine); "
+                              "the rotation over three weight sets and several id draws is replayed as one "
                               "HIP graph; GBps counts the distinct experts of each call"}
         for exps in sets:
             for w in exps.values():
