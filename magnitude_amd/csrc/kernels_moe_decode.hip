@@ -51,10 +51,12 @@ __device__ __forceinline__ float slot_sum(float v, int vlane, int lpr) {
     return v;
 }
 
-template <int QT, bool SWIGLU, bool COMBINE>
+// R: row steps a unit covers (two where a wave has several units of short rows: fewer, larger requests)
+template <int QT, bool SWIGLU, bool COMBINE, int R>
 __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArgs g) {
+    static_assert(!SWIGLU || R == 1, "gate / up already load two tensors a unit");
     extern __shared__ __align__(16) uint8_t smem[];
-    constexpr int NT = SWIGLU ? 2 : 1;
+    constexpr int NT = SWIGLU ? 2 : R;   // register sets a unit loads
     const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6);
     const int K = (int)g.w0.K, nb = (int)g.w0.nb, N = (int)g.w0.N;
     const int lpr = 4 * nb, S = 64 / lpr;
@@ -65,7 +67,7 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
     const int p0 = grp * g.group, G = g.group;
     const int r0 = j * g.rows_per_wg;
     const int r1 = min(N, r0 + g.rows_per_wg);
-    const int steps = r1 > r0 ? (r1 - r0 + S - 1) / S : 0;
+    const int steps = r1 > r0 ? (r1 - r0 + S * R - 1) / (S * R) : 0;   // units a pair has here
     const int units = G * steps;
     const int n_u = units > wave ? (units - wave + kWaves - 1) / kWaves : 0;   // this wave's units: wave, wave + 16, ..
 
@@ -111,7 +113,7 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
         Unit u;
         const int idx = wave + kWaves * i;
         u.s = idx / steps;
-        u.row = r0 + (idx - u.s * steps) * S;
+        u.row = r0 + (idx - u.s * steps) * S * R;
         const int e = uniform(g.ids[p0 + u.s]);
         u.ok = e >= 0 && e < g.n_expert;
         u.expert = u.ok ? e : 0;   // a pair without an expert is left out; its loads go somewhere valid
@@ -121,12 +123,16 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
         const Unit u = unit_of(i);
         RowPtr<QT> rp;
         rp.set(g.w0, (int64_t)u.expert * N + u.row);
-        const uint32_t rel = (uint32_t)min(slot, r1 - 1 - u.row);
-        raw[0].load(rp, (uint32_t)(vlane >> 2), vlane, rel);
         if constexpr (SWIGLU) {
+            const uint32_t rel = (uint32_t)min(slot, r1 - 1 - u.row);
+            raw[0].load(rp, (uint32_t)(vlane >> 2), vlane, rel);
             RowPtr<QT> ru;
             ru.set(g.w1, (int64_t)u.expert * N + u.row);
             raw[NT - 1].load(ru, (uint32_t)(vlane >> 2), vlane, rel);
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r)   // rows past the end of the range repeat its last row
+                raw[r].load(rp, (uint32_t)(vlane >> 2), vlane, (uint32_t)min(r * S + slot, r1 - 1 - u.row));
         }
     };
     auto consume = [&](const Raw<QT> (&raw)[NT], int i) {
@@ -140,12 +146,15 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
             f.unpack(raw[t], vlane);
             acc[t] = slot_sum(live ? dx.dot(f) : 0.f, vlane, lpr);
         }
-        const int row = u.row + slot;
-        if (live && vlane == 0 && row < r1) {
-            float r = acc[0];
-            if constexpr (SWIGLU) r = (r / (1.0f + expf(-r))) * acc[NT - 1];
-            if constexpr (COMBINE) res[u.s * g.rows_per_wg + (row - r0)] = u.ok ? r : 0.f;
-            else if (u.ok) g.y[(int64_t)(p0 + u.s) * N + row] = r;
+#pragma unroll
+        for (int t = 0; t < (SWIGLU ? 1 : R); ++t) {
+            const int row = u.row + t * S + slot;
+            if (live && vlane == 0 && row < r1) {
+                float r = acc[t];
+                if constexpr (SWIGLU) r = (r / (1.0f + expf(-r))) * acc[NT - 1];
+                if constexpr (COMBINE) res[u.s * g.rows_per_wg + (row - r0)] = u.ok ? r : 0.f;
+                else if (u.ok) g.y[(int64_t)(p0 + u.s) * N + row] = r;
+            }
         }
     };
 
@@ -205,9 +214,9 @@ int cu_count() {
     return n;
 }
 
-template <int QT, bool SWIGLU, bool COMBINE>
+template <int QT, bool SWIGLU, bool COMBINE, int R = 1>
 hipError_t launch_typed(const MoeDecodeArgs &g, unsigned grid, size_t lds, hipStream_t s) {
-    auto kern = &moe_decode_kernel<QT, SWIGLU, COMBINE>;
+    auto kern = &moe_decode_kernel<QT, SWIGLU, COMBINE, R>;
     static size_t allowed = 48 * 1024;
     if (lds > allowed) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -266,11 +275,16 @@ hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, co
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     if (dry_run()) return hipSuccess;
     const unsigned grid = (unsigned)(n_groups * g.wgs_per_group);
+    // two row steps a unit where a wave would otherwise walk four or more units of rows that fill under 4 KB a step
+    static const int two_env = tuning_int("QPROJ_MOE_DECODE_TWO_STEPS", -1);
+    const bool two = two_env >= 0 ? two_env != 0 : (!swiglu && group * steps_per_wg >= 4 * kWaves);
     if (w.type == kTypeQ4_K) {
         if (swiglu) return launch_typed<kTypeQ4_K, true, false>(g, grid, lds, s);
+        if (two) return combine_weights ? launch_typed<kTypeQ4_K, false, true, 2>(g, grid, lds, s) : launch_typed<kTypeQ4_K, false, false, 2>(g, grid, lds, s);
         return combine_weights ? launch_typed<kTypeQ4_K, false, true>(g, grid, lds, s) : launch_typed<kTypeQ4_K, false, false>(g, grid, lds, s);
     }
     if (swiglu) return launch_typed<kTypeQ6_K, true, false>(g, grid, lds, s);
+    if (two) return combine_weights ? launch_typed<kTypeQ6_K, false, true, 2>(g, grid, lds, s) : launch_typed<kTypeQ6_K, false, false, 2>(g, grid, lds, s);
     return combine_weights ? launch_typed<kTypeQ6_K, false, true>(g, grid, lds, s) : launch_typed<kTypeQ6_K, false, false>(g, grid, lds, s);
 }
 
