@@ -18,9 +18,11 @@ constexpr int kDecodeThreads = 1024;
 constexpr int kDecodeWaves = kDecodeThreads / 64;
 
 // activations into LDS: FUSE quantizes fp32 rows here; otherwise planes quantized earlier are copied
-// 256-wide pieces of the activation rows a wave fetches ahead of its first weights: four registers' worth,
-// shared out over the rows (one row: K up to 16384 is covered, two rows: 8192, four rows: 4096)
-constexpr int kPrefetchedPieces = 4;
+// 256-wide pieces of an activation row that a wave fetches ahead of its first weights: four a row for one or two
+// rows (K up to 16384 is covered; pieces fetched inside the quantizing loop instead come one after the other, a trip to
+// L2 each: the down projection at two rows, 3.5 pieces a row and wave, 20.2 -> 17.5 us with one-row steps, then
+// this), one a row for four rows
+__host__ __device__ constexpr int prefetched_pieces(int mt) { return mt <= 2 ? 4 : 1; }
 
 template <int QT, int MT, bool FUSE>
 __device__ __forceinline__ void stage_activations(uint8_t *smem, const GemvArgs &args, int64_t K, int kpad,
@@ -38,7 +40,7 @@ __device__ __forceinline__ void stage_activations(uint8_t *smem, const GemvArgs 
             for (int ch = wave; ch < n_chunks; ch += kDecodeWaves) {
                 const int e0 = ch * 256 + 4 * lane;
                 float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-                constexpr int kPer = kPrefetchedPieces / MT;   // pieces per row the caller fetched
+                constexpr int kPer = prefetched_pieces(MT);   // pieces per row the caller fetched
                 if (first && ch < wave + kDecodeWaves * kPer)
                     v = first[m * kPer + (ch - wave) / kDecodeWaves];
                 else if (have && e0 < K) v = *reinterpret_cast<const float4 *>(x + e0);
@@ -208,9 +210,9 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     // The wave's piece of the activation row is requested BEFORE the first weights: loads return in order, and
     // behind a step of weights coming from HBM the quantizing prologue would wait two microseconds for sixteen
     // bytes that sit in L2 (phase clocks: staging 3000-4400 cycles of a workgroup's 25000).
-    float4 x_first[kPrefetchedPieces];
+    float4 x_first[MT * prefetched_pieces(MT)];
     if (FUSE) {
-        constexpr int kPer = kPrefetchedPieces / MT;
+        constexpr int kPer = prefetched_pieces(MT);
 #pragma unroll
         for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -223,10 +225,10 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     // RMS norm fused in front of the quantizer (the launcher only asks for it when the prefetched pieces are the
     // whole row): weights of the norm fetched with the row, sum of squares over the workgroup in the order of
     // the standalone kernel, then the pieces are replaced by (x * scale) * gamma.
-    float4 g_first[kPrefetchedPieces / MT];
+    float4 g_first[prefetched_pieces(MT)];
     if (FUSE && args.norm) {
 #pragma unroll
-        for (int i = 0; i < kPrefetchedPieces / MT; ++i) {
+        for (int i = 0; i < prefetched_pieces(MT); ++i) {
             const int e0 = (wave + kDecodeWaves * i) * 256 + 4 * lane;
             g_first[i] = make_float4(1.f, 1.f, 1.f, 1.f);
             if (args.norm_gamma && e0 < K) g_first[i] = *reinterpret_cast<const float4 *>(args.norm_gamma + e0);
@@ -236,7 +238,7 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     issue_rows(buf_a, 0, 0);  // in flight while the activations are staged
     if (FUSE && args.norm) {
         __shared__ double norm_partial[kDecodeWaves];
-        constexpr int kPer = kPrefetchedPieces / MT;
+        constexpr int kPer = prefetched_pieces(MT);
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
             double sq = 0.0;
@@ -410,17 +412,20 @@ hipError_t launch_decode_mt(const GemvArgs &args, int mt, hipStream_t s) {
         if (mt == 2) return one_chunk ? launch_decode<QT, 2, 2, true, FUSE, true>(args, s) : launch_decode<QT, 2, 2, false, FUSE, true>(args, s);
         return hipErrorInvalidValue;
     }
+    // two rows per step only when every wave has at least two rows to walk (with 1.5 rows per wave, split
+    // 2 + 1 over a pair of waves, two-row steps measured slower: q/k/v 7.4 against 6.4 us; with one row a wave
+    // a two-row step fetches that row twice)
+    int64_t rows_total = 0;
+    for (int i = 0; i < args.n_targets; ++i) rows_total += args.t[i].w.N;
+    static const int two_rows_env = tuning_int("QPROJ_DECODE_TWO_ROWS", -1);
+    const bool pairs = two_rows_env >= 0 ? two_rows_env != 0 : rows_total >= (int64_t)2 * cu_count() * kDecodeWaves;
     switch (mt) {
-    case 1: {
-        // two rows per step only when every wave has at least two rows to walk (with 1.5 rows per wave, split
-        // 2 + 1 over a pair of waves, two-row steps measured slower: q/k/v 7.4 against 6.4 us)
-        int64_t rows_total = 0;
-        for (int i = 0; i < args.n_targets; ++i) rows_total += args.t[i].w.N;
-        const bool pairs = rows_total >= (int64_t)2 * cu_count() * kDecodeWaves;
+    case 1:
         if (one_chunk) return pairs ? launch_decode<QT, 1, 2, true, FUSE>(args, s) : launch_decode<QT, 1, 1, true, FUSE>(args, s);
         return pairs ? launch_decode<QT, 1, 2, false, FUSE>(args, s) : launch_decode<QT, 1, 1, false, FUSE>(args, s);
-    }
-    case 2: return one_chunk ? launch_decode<QT, 2, 2, true, FUSE>(args, s) : launch_decode<QT, 2, 2, false, FUSE>(args, s);
+    case 2:
+        if (one_chunk) return pairs ? launch_decode<QT, 2, 2, true, FUSE>(args, s) : launch_decode<QT, 2, 1, true, FUSE>(args, s);
+        return pairs ? launch_decode<QT, 2, 2, false, FUSE>(args, s) : launch_decode<QT, 2, 1, false, FUSE>(args, s);
     case 4: return launch_decode<QT, 4, 1, false, FUSE>(args, s);
     default: return hipErrorInvalidValue;
     }
@@ -429,7 +434,7 @@ hipError_t launch_decode_mt(const GemvArgs &args, int mt, hipStream_t s) {
 }  // namespace
 
 bool decode_kernel_norm_fits(int mt, int64_t K) {
-    return mt >= 1 && mt <= kPrefetchedPieces && K <= (int64_t)256 * kDecodeWaves * (kPrefetchedPieces / mt);
+    return mt >= 1 && mt <= 4 && K <= (int64_t)256 * kDecodeWaves * prefetched_pieces(mt);
 }
 
 // the largest K whose activation rows fit the LDS image (mt rows)
