@@ -21,7 +21,7 @@ constexpr int kDecodeWaves = kDecodeThreads / 64;
 // 256-wide pieces of an activation row that a wave fetches ahead of its first weights: four a row for one or two
 // rows (K up to 16384 is covered; pieces fetched inside the quantizing loop instead come one after the other, a trip to
 // L2 each: the down projection at two rows, 3.5 pieces a row and wave, 20.2 -> 17.5 us with one-row steps, then
-// this), one a row for four rows
+// this), one a row for four rows (which take this kernel for K <= 4096 only)
 __host__ __device__ constexpr int prefetched_pieces(int mt) { return mt <= 2 ? 4 : 1; }
 
 template <int QT, int MT, bool FUSE>
@@ -426,7 +426,10 @@ hipError_t launch_decode_mt(const GemvArgs &args, int mt, hipStream_t s) {
     case 2:
         if (one_chunk) return pairs ? launch_decode<QT, 2, 2, true, FUSE>(args, s) : launch_decode<QT, 2, 1, true, FUSE>(args, s);
         return pairs ? launch_decode<QT, 2, 2, false, FUSE>(args, s) : launch_decode<QT, 2, 1, false, FUSE>(args, s);
-    case 4: return launch_decode<QT, 4, 1, false, FUSE>(args, s);
+    case 4:
+        if constexpr (QT == kTypeQ4_K)
+            if (one_chunk) return launch_decode<QT, 4, 1, true, FUSE>(args, s);
+        return launch_decode<QT, 4, 1, false, FUSE>(args, s);
     default: return hipErrorInvalidValue;
     }
 }

@@ -342,7 +342,11 @@ bool use_mfma_grouped(int type, int64_t K) {
 
 bool use_mfma_kernel(int type, int64_t M, int64_t K) {
     static const bool off = tuning_int("QPROJ_NO_MFMA_GEMV", 0) != 0;
-    static const int min_m = tuning_int("QPROJ_MFMA_MIN_M", 3);
+    // three and four rows of Q4_K with K <= 4096 stay on the decode kernel, which holds four activation rows in
+    // registers there and quantizes them in its prologue (gate+up at four rows 22.0 -> 20.2 us, o 10.6 -> 8.2; the
+    // longer rows of the down projection and the wider formats measured slower that way, 23.2 -> 25.3 us)
+    static const int forced = tuning_int("QPROJ_MFMA_MIN_M", 0);
+    const int min_m = forced > 0 ? forced : (type == kTypeQ4_K && K <= 4096 && decode_kernel_fits(type, 4, K)) ? 5 : 3;
     return !off && M >= min_m && mfma_gemv_fits(type, std::min<int64_t>(M, 16), K);
 }
 
