@@ -104,30 +104,39 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
         if (e < 0 || e >= g.n_expert) atomicOr(g.error_flag, 1);
     }
 
-    // unit u = (pair s of the group, row step st): experts are read by the wave itself (scalar loads)
+    // unit u = (row step st, pair s of the group), pairs running fastest: with 1, 2, 4, 8 or 16 pairs a group a wave
+    // (units wave, wave + 16, ..) stays with ONE pair, whose expert it reads once (a scalar load) and whose
+    // activation slices it keeps in registers; otherwise both are fetched again whenever the pair changes
     struct Unit {
-        int s, row, expert;
-        bool ok;
+        int s, row;
     };
     auto unit_of = [&](int i) {
         Unit u;
         const int idx = wave + kWaves * i;
-        u.s = idx / steps;
-        u.row = r0 + (idx - u.s * steps) * S * R;
-        const int e = uniform(g.ids[p0 + u.s]);
-        u.ok = e >= 0 && e < g.n_expert;
-        u.expert = u.ok ? e : 0;   // a pair without an expert is left out; its loads go somewhere valid
+        const int st = idx / G;
+        u.s = idx - st * G;
+        u.row = r0 + st * S * R;
         return u;
     };
+    auto expert_of = [&](int s_) {   // -1: the pair names no expert and is left out
+        const int e = uniform(g.ids[p0 + s_]);
+        return e >= 0 && e < g.n_expert ? e : -1;
+    };
+    int issue_s = -1, issue_e = -1;
     auto issue = [&](Raw<QT> (&raw)[NT], int i) {
         const Unit u = unit_of(i);
+        if (u.s != issue_s) {
+            issue_s = u.s;
+            issue_e = expert_of(u.s);
+        }
+        const int64_t first = (int64_t)(issue_e < 0 ? 0 : issue_e) * N + u.row;   // (a pair left out loads somewhere valid)
         RowPtr<QT> rp;
-        rp.set(g.w0, (int64_t)u.expert * N + u.row);
+        rp.set(g.w0, first);
         if constexpr (SWIGLU) {
             const uint32_t rel = (uint32_t)min(slot, r1 - 1 - u.row);
             raw[0].load(rp, (uint32_t)(vlane >> 2), vlane, rel);
             RowPtr<QT> ru;
-            ru.set(g.w1, (int64_t)u.expert * N + u.row);
+            ru.set(g.w1, first);
             raw[NT - 1].load(ru, (uint32_t)(vlane >> 2), vlane, rel);
         } else {
 #pragma unroll
@@ -135,10 +144,16 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
                 raw[r].load(rp, (uint32_t)(vlane >> 2), vlane, (uint32_t)min(r * S + slot, r1 - 1 - u.row));
         }
     };
+    int cur_s = -1;
+    bool cur_ok = false;
+    Dot<QT> dx;
     auto consume = [&](const Raw<QT> (&raw)[NT], int i) {
         const Unit u = unit_of(i);
-        Dot<QT> dx;
-        dx.load_x(xt, u.s, 0, vlane);
+        if (u.s != cur_s) {
+            cur_s = u.s;
+            cur_ok = expert_of(u.s) >= 0;
+            dx.load_x(xt, u.s, 0, vlane);
+        }
         float acc[NT];
 #pragma unroll
         for (int t = 0; t < NT; ++t) {
@@ -152,8 +167,8 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
             if (live && vlane == 0 && row < r1) {
                 float r = acc[t];
                 if constexpr (SWIGLU) r = (r / (1.0f + expf(-r))) * acc[NT - 1];
-                if constexpr (COMBINE) res[u.s * g.rows_per_wg + (row - r0)] = u.ok ? r : 0.f;
-                else if (u.ok) g.y[(int64_t)(p0 + u.s) * N + row] = r;
+                if constexpr (COMBINE) res[u.s * g.rows_per_wg + (row - r0)] = cur_ok ? r : 0.f;
+                else if (cur_ok) g.y[(int64_t)(p0 + u.s) * N + row] = r;
             }
         }
     };

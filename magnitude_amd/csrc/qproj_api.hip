@@ -484,8 +484,8 @@ bool grouped_pair_mode(int type, int64_t K, int64_t n_pairs, int64_t E) {
 }
 
 // A few decode tokens: the vector-ALU kernel that reads an expert once per PAIR and needs no grouping, quantizer
-// or combine launch.  Measured against the grouped route (128 experts, top-8, 2048 x 768, per call): 20.8 -> 14.8 us
-// at one token, 24.9 -> 19.2 at two, 41.0 -> 26.9 at four, 57.6 -> 43.0 at eight, level at twelve and sixteen; with
+// or combine launch.  Measured against the grouped route (128 experts, top-8, 2048 x 768, per call): 20.8 -> 15.0 us
+// at one token, 24.9 -> 18.8 at two, 41.0 -> 23.2 at four, 57.6 -> 36.2 at eight, level at twelve and sixteen; with
 // more pairs than experts the repeated reads of an expert outweigh the launches saved.
 bool moe_decode_route(int type, int64_t K, int64_t n_pairs, int64_t group, int64_t E) {
     static const bool on = tuning_int("QPROJ_NO_MOE_DECODE", 0) == 0;
