@@ -485,12 +485,14 @@ bool grouped_pair_mode(int type, int64_t K, int64_t n_pairs, int64_t E) {
 
 // A few decode tokens: the vector-ALU kernel that reads an expert once per PAIR and needs no grouping, quantizer
 // or combine launch.  Measured against the grouped route (128 experts, top-8, 2048 x 768, per call): 20.8 -> 15.0 us
-// at one token, 24.9 -> 18.8 at two, 41.0 -> 23.2 at four, 57.6 -> 36.2 at eight, level at twelve and sixteen; with
+// at one token, 24.9 -> 18.8 at two, 41.0 -> 23.2 at four, 57.6 -> 36.2 at eight, 74.1 -> 58.9 at sixteen, level at twenty to
+// twenty-four and worse at 32 (101 against 95 us); with
 // more pairs than experts the repeated reads of an expert outweigh the launches saved.
 bool moe_decode_route(int type, int64_t K, int64_t n_pairs, int64_t group, int64_t E) {
     static const bool on = tuning_int("QPROJ_NO_MOE_DECODE", 0) == 0;
-    static const int max_pairs = tuning_int("QPROJ_MOE_DECODE_MAX_PAIRS", 64);
-    return on && (n_pairs <= 16 || (n_pairs <= max_pairs && n_pairs <= E)) && moe_decode_fits(type, K, n_pairs, group);
+    static const int max_pairs = tuning_int("QPROJ_MOE_DECODE_MAX_PAIRS", 128);
+    static const int per_4_experts = tuning_int("QPROJ_MOE_DECODE_PAIRS_PER_4_EXPERTS", 4);
+    return on && (n_pairs <= 16 || (n_pairs <= max_pairs && 4 * n_pairs <= per_4_experts * E)) && moe_decode_fits(type, K, n_pairs, group);
 }
 
 int grouped_mt(int64_t n_pairs, int64_t E) {

@@ -523,9 +523,9 @@ def test_moe_ffn_many_experts(ctx, orc, moe, E):
     assert np.median(np.abs(got - want)) <= 1e-6 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("B,E", [(1, 128), (2, 128), (4, 128), (8, 128), (2, 16), (5, 40)])
+@pytest.mark.parametrize("B,E", [(1, 128), (2, 128), (4, 128), (8, 128), (16, 128), (2, 16), (5, 40)])
 def test_moe_ffn_few_tokens_take_an_expert_per_pair(ctx, orc, moe, B, E):
-    """Decode-sized batches (at most 64 pairs and no more pairs than experts, or up to 16 pairs): the route that
+    """Decode-sized batches (at most 128 pairs and no more pairs than experts, or up to 16 pairs): the route that
     needs no grouping pass - a set of workgroups per pair reads ids[p] itself, quantizes the pair's activation row,
     and the down projection adds a token's pairs with their routing weights in slot order.  One unit a wave at one
     token, several pipelined units a wave at eight."""
