@@ -423,9 +423,13 @@ hipError_t launch_decode_mt(const GemvArgs &args, int mt, hipStream_t s) {
     case 1:
         if (one_chunk) return pairs ? launch_decode<QT, 1, 2, true, FUSE>(args, s) : launch_decode<QT, 1, 1, true, FUSE>(args, s);
         return pairs ? launch_decode<QT, 1, 2, false, FUSE>(args, s) : launch_decode<QT, 1, 1, false, FUSE>(args, s);
-    case 2:
-        if (one_chunk) return pairs ? launch_decode<QT, 2, 2, true, FUSE>(args, s) : launch_decode<QT, 2, 1, true, FUSE>(args, s);
-        return pairs ? launch_decode<QT, 2, 2, false, FUSE>(args, s) : launch_decode<QT, 2, 1, false, FUSE>(args, s);
+    case 2: {
+        // (two rows of the wider formats walk one weight row a step whatever the row count: their two-row steps
+        // run out of registers -- Q6_K 4096 -> 14336 17.5 -> 13.9 us, Q8_0 8192 x 8192 20.1 -> 17.6)
+        const bool two = pairs && (QT == kTypeQ4_K || two_rows_env > 0);
+        if (one_chunk) return two ? launch_decode<QT, 2, 2, true, FUSE>(args, s) : launch_decode<QT, 2, 1, true, FUSE>(args, s);
+        return two ? launch_decode<QT, 2, 2, false, FUSE>(args, s) : launch_decode<QT, 2, 1, false, FUSE>(args, s);
+    }
     case 4:
         if constexpr (QT == kTypeQ4_K)
             if (one_chunk) return launch_decode<QT, 4, 1, true, FUSE>(args, s);

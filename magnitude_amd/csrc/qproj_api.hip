@@ -342,11 +342,13 @@ bool use_mfma_grouped(int type, int64_t K) {
 
 bool use_mfma_kernel(int type, int64_t M, int64_t K) {
     static const bool off = tuning_int("QPROJ_NO_MFMA_GEMV", 0) != 0;
-    // three and four rows of Q4_K with K <= 4096 stay on the decode kernel, which holds four activation rows in
-    // registers there and quantizes them in its prologue (gate+up at four rows 22.0 -> 20.2 us, o 10.6 -> 8.2; the
-    // longer rows of the down projection and the wider formats measured slower that way, 23.2 -> 25.3 us)
+    // Three and four rows stay on the decode kernel (one launch, quantizer in its prologue; Q4_K holds the four
+    // activation rows in registers) for K <= 4096 and for Q8_0 of any K.  Measured at 3 - 4 rows, this kernel ->
+    // decode kernel, us: Q4_K 4096x4096 10.8 -> 8.4, gate+up 22.0 -> 20.2; Q6_K 4096 -> 1024 13.1 -> 8.4, 4096 -> 14336
+    // 21.2 -> 18.5; Q8_0 4096x4096 13.5 -> 8.7, 4096 -> 14336 21.7 -> 17.4, 8192x8192 25.2 -> 22.6.  Longer rows of
+    // the K-quants lose there: Q4_K 14336 -> 4096 17.8 -> 21.9, 8192x8192 16.8 -> 19.1; Q6_K 14336 -> 4096 23.6 -> 24.8.
     static const int forced = tuning_int("QPROJ_MFMA_MIN_M", 0);
-    const int min_m = forced > 0 ? forced : (type == kTypeQ4_K && K <= 4096 && decode_kernel_fits(type, 4, K)) ? 5 : 3;
+    const int min_m = forced > 0 ? forced : ((K <= 4096 || type == kTypeQ8_0) && decode_kernel_fits(type, 4, K)) ? 5 : 3;
     return !off && M >= min_m && mfma_gemv_fits(type, std::min<int64_t>(M, 16), K);
 }
 

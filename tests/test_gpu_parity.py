@@ -323,10 +323,10 @@ def test_small_m_rows_equal_the_m1_result(ctx, orc, qtype):
     single = torch.cat([ctx.mul_mat(w, x[i:i + 1], ACT_GGML) for i in range(16)]).cpu().numpy()
     full = ctx.mul_mat(w, x, ACT_GGML).cpu().numpy()
     close(full, single, 2e-5)
-    decode_rows = 4 if qtype == Q4_K and k <= 4096 else 2
+    decode_rows = 4 if k <= 4096 or qtype == Q8_0 else 2
     for m in (2, 3, 4, 5, 8, 11):
         got = ctx.mul_mat(w, x[:m], ACT_GGML).cpu().numpy()
-        # the decode kernel serves up to 2 rows (4 of Q4_K with K <= 4096), the matrix-core kernel the rest up to 16:
+        # the decode kernel serves up to 2 rows (4 with K <= 4096 and for Q8_0), the matrix-core kernel the rest up to 16:
         # bitwise within each
         assert np.array_equal(got, (single if m <= decode_rows else full)[:m]), m
 
