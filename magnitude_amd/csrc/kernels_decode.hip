@@ -342,14 +342,6 @@ __global__ __launch_bounds__(kDecodeThreads) void gemv_decode_kernel(const GemvA
     }
 }
 
-int cu_count() {
-    static int n = [] {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
-        return v;
-    }();
-    return n;
-}
 
 template <int QT, int MT, int R, bool XREG, bool FUSE, bool PAIR = false>
 hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
@@ -442,6 +434,15 @@ hipError_t launch_decode_mt(const GemvArgs &args, int mt, hipStream_t s) {
 }
 
 }  // namespace
+
+int cu_count() {
+    static int n = [] {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+        return v;
+    }();
+    return n;
+}
 
 bool decode_kernel_norm_fits(int mt, int64_t K) {
     return mt >= 1 && mt <= 4 && K <= (int64_t)256 * kDecodeWaves * prefetched_pieces(mt);

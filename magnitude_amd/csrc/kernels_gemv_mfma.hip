@@ -828,16 +828,25 @@ struct Split {
     int n_chunks, chunk_sb, kw;
 };
 constexpr int kMaxSb16 = 16;   // super-blocks of 16 staged rows that fit LDS beside the wave regions (~66 KB)
-Split plan(int64_t K, int64_t M, int64_t total_rg, int W, int min_wgs = 200) {
+// `dense`: the launch is one workgroup a compute unit (eight waves of ~200 registers), so the K parts are chosen
+// with the chunks that LDS forces counted in, and a grid of a round and a bit is traded for one round of longer
+// workgroups.  (Before, 16 rows of K = 14336 got 8 K parts x 4 chunks = 512 workgroups, two rounds: the Q6_K down
+// projection 36.3 -> 26.9 us with 4 K parts, 256 workgroups; Q4_K 14336 -> 4096 28.0 -> 20.2, 8192 x 8192 28.7 ->
+// 21.8; 13824 -> 5120 at 8 rows 37.7 -> 27.5 with 4 K parts x 3 chunks = 240 workgroups instead of 8 x 2 = 320.)
+Split plan(int64_t K, int64_t M, int64_t total_rg, int W, int min_wgs = 200, bool dense = false, int cus = 256) {
     const int nb = (int)(K / 256);
     const int max_sb = M <= 8 ? 2 * kMaxSb16 : kMaxSb16;
+    int nc = (nb + max_sb - 1) / max_sb;
+    const int nc_forced = dense ? nc : 1;
     Split p;
     p.kw = 1;
-    while (p.kw < W && p.kw * 2 <= nb && total_rg * p.kw / W < min_wgs) p.kw *= 2;
-    const int rw = W / p.kw;
-    const int64_t wgs1 = (total_rg + rw - 1) / rw;
-    int nc = (nb + max_sb - 1) / max_sb;
+    while (p.kw < W && p.kw * 2 <= nb && total_rg * p.kw / W * nc_forced < min_wgs) p.kw *= 2;
+    auto wgs_of = [&](int kw) { return (total_rg + W / kw - 1) / (W / kw); };
+    if (dense && p.kw > 1 && wgs_of(p.kw) * nc > cus && wgs_of(p.kw / 2) * nc <= cus) p.kw /= 2;
+    const int64_t wgs1 = wgs_of(p.kw);
     if (wgs1 * nc < 128) nc = std::max(nc, (int)std::min<int64_t>(std::max(1, nb / p.kw), (255 + wgs1) / wgs1));
+    else if (dense && nc > 1 && wgs1 * nc * 10 < cus * 7)   // the sum over chunks is paid for anyway: fill the round
+        nc = std::max(nc, (int)std::min<int64_t>(std::max(1, nb / p.kw), cus / wgs1));
     p.chunk_sb = (nb + nc - 1) / nc;
     p.n_chunks = (nb + p.chunk_sb - 1) / p.chunk_sb;
     return p;
@@ -871,7 +880,7 @@ bool mfma_grouped_fits(int type, int64_t K) {
 }
 
 size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, int64_t total_rg) {
-    const Split p = plan(K, M, total_rg, waves_per_wg(type));
+    const Split p = plan(K, M, total_rg, waves_per_wg(type), 200, true, cu_count());
     return p.n_chunks > 1 ? (size_t)p.n_chunks * (size_t)M * (size_t)sum_n * 4 : 0;
 }
 
@@ -885,7 +894,7 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStr
     int64_t total_rg = 0;
     for (int i = 0; i < args.n_targets; ++i) total_rg += (args.t[i].w.N + 31) / 32;
     const int W = waves_per_wg(args.t[0].w.type);
-    const Split p = plan(args.a.K, args.M, total_rg, W);
+    const Split p = plan(args.a.K, args.M, total_rg, W, 200, true, cu_count());
     g.n_chunks = p.n_chunks;
     g.chunk_sb = p.chunk_sb;
     g.kw = p.kw;

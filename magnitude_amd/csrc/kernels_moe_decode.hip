@@ -220,15 +220,6 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
     }
 }
 
-int cu_count() {
-    static int n = [] {
-        int dev = 0, v = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
-        return v;
-    }();
-    return n;
-}
-
 template <int QT, bool SWIGLU, bool COMBINE, int R = 1>
 hipError_t launch_typed(const MoeDecodeArgs &g, unsigned grid, size_t lds, hipStream_t s) {
     auto kern = &moe_decode_kernel<QT, SWIGLU, COMBINE, R>;

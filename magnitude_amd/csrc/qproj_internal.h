@@ -98,6 +98,9 @@ struct Scratch {
 bool dry_run();
 void set_dry_run(bool on);
 
+// Compute units of the current device (256 when no device can be asked, e.g. in a dry run on a host without one).
+int cu_count();
+
 // Tuning knobs read from the environment exist only in builds made with -DQPROJ_TUNING (kernel-selection sweeps in
 // the lab); in the shipped library this returns `dflt` and no environment variable can change a numerics path.
 int tuning_int(const char *name, int dflt);
