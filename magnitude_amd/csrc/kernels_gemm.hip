@@ -951,8 +951,9 @@ hipError_t launch_gemm_q8_0(const WeightView &w, const ActView &a, int64_t M, fl
 
 // Which Q4_K kernel and how many stretches of K (one rule for the launcher and for the scratch sizing).  The
 // 128-token kernel (256 weight rows a workgroup, one workgroup per compute unit) wants about 192 workgroups or more:
-// a grid of 96..191 such tiles is doubled by cutting K in two, one of 48..95 quadrupled, never under twelve
-// super-blocks a stretch.  Everything else takes 64-token tiles with the stretches of q8k_tile_splits.
+// a grid of 48..191 such tiles is multiplied by cutting K into the stretches wide_tile_splits picks (64 tiles of
+// K = 14336: four; of K = 11008: three, 192 workgroups, where the halving rule before left half the chip idle).
+// Everything else takes 64-token tiles with the stretches of q8k_tile_splits.
 namespace {
 struct Q4Plan {
     bool wide;
@@ -963,8 +964,7 @@ Q4Plan q4k_plan(int64_t K, int64_t M, int64_t N, bool have_scratch) {
     const int64_t wide_tiles = ((N + 255) / 256) * ((M + 127) / 128);
     if (wide_env >= 0 ? wide_env != 0 : wide_tiles >= 192) return {true, 1};
     if (wide_env < 0 && have_scratch && (M * N) % 4 == 0 && wide_tiles >= 48) {
-        int n = wide_tiles >= 96 ? 2 : 4;
-        while (n > 1 && K / 256 < 12 * n) n >>= 1;
+        const int n = wide_tile_splits(wide_tiles, K / 256, M, N, cu_count(), 4.5);
         if (n > 1) return {true, n};
     }
     return {false, have_scratch ? q8k_tile_splits(K, M, N) : 1};

@@ -474,8 +474,9 @@ hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y
 }  // namespace
 
 // Which kernel and how many stretches of K.  The 128-token kernel (256 weight rows a workgroup, one workgroup per
-// compute unit) wants about 192 workgroups or more: a grid of 96..191 such tiles is doubled by cutting K in two, one of
-// 48..95 quadrupled, never under twelve super-blocks a stretch.  Smaller grids take 64-token tiles (128 rows, two
+// compute unit) wants about 192 workgroups or more: a grid of 48..191 such tiles is multiplied by cutting K into the
+// stretches wide_tile_splits picks (64 tiles of K = 14336: four; 80 tiles of K = 13824: three, 240 workgroups in one
+// round, where four made 320).  Smaller grids take 64-token tiles (128 rows, two
 // workgroups per compute unit) with the stretches of q8k_tile_splits, or 32-token tiles where K is too short for that.
 namespace {
 struct Q6Plan {
@@ -486,8 +487,7 @@ Q6Plan q6k_plan(int64_t K, int64_t M, int64_t N, bool have_scratch) {
     const int64_t wide_tiles = ((N + 255) / 256) * ((M + 127) / 128);
     if (wide_tiles >= 192) return {true, 1};
     if (have_scratch && (M * N) % 4 == 0 && wide_tiles >= 48) {
-        int n = wide_tiles >= 96 ? 2 : 4;
-        while (n > 1 && K / 256 < 12 * n) n >>= 1;
+        const int n = wide_tile_splits(wide_tiles, K / 256, M, N, cu_count(), 5.0);
         if (n > 1) return {true, n};
     }
     return {false, have_scratch ? q8k_tile_splits(K, M, N) : 1};

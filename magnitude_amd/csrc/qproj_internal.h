@@ -98,6 +98,25 @@ struct Scratch {
 bool dry_run();
 void set_dry_run(bool on);
 
+// Into how many stretches K is cut for a grid of `tiles` 128-token tiles (one workgroup a compute unit) that would
+// not fill the chip by itself: the cut that minimises rounds x (stretch + fixed cost) + the pass that adds the
+// partial tiles (M x N x 4 bytes a stretch written and read again), never under twelve super-blocks a stretch.
+// `us_per_sb`: what one super-block step of a full round takes (4.5 us for the Q4_K tile, 5 for Q6_K).
+inline int wide_tile_splits(int64_t tiles, int64_t nsb, int64_t M, int64_t N, int cus, double us_per_sb) {
+    int best = 1;
+    double best_cost = 1e300;
+    for (int n = 1; n <= 8 && (n == 1 || nsb / n >= 12); ++n) {
+        const int64_t per = (nsb + n - 1) / n, rounds = (tiles * n + cus - 1) / cus;
+        double cost = (double)rounds * ((double)per * us_per_sb + 8.0);
+        if (n > 1) cost += (double)n * (double)M * (double)N * 2.7e-6 + 5.0;
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = n;
+        }
+    }
+    return best;
+}
+
 // Compute units of the current device (256 when no device can be asked, e.g. in a dry run on a host without one).
 int cu_count();
 

@@ -1081,7 +1081,9 @@ def test_tiled_q4k_products_over_a_wide_range_of_activation_scales(ctx, orc, m, 
 BENCHED_PREFILL = (   # every (mode, type, K, N) x M the benchmark's prefill leg times (config 4 and the layer's other formats)
     [("q8x32", Q4_K, k, n) for (k, n) in ((4096, 14336), (14336, 4096), (4096, 4096))] +
     [("ggml", Q4_K, k, n) for (k, n) in ((4096, 14336), (14336, 4096), (4096, 4096))] +
-    [("ggml", Q6_K, 14336, 4096), ("ggml", Q8_0, 4096, 4096)])
+    [("ggml", Q6_K, 14336, 4096), ("ggml", Q8_0, 4096, 4096)] +
+    # shapes of other model sizes whose grids take other cuts of K (three stretches at 512 tokens)
+    [("ggml", Q4_K, 11008, 4096), ("ggml", Q6_K, 13824, 5120)])
 
 
 @pytest.mark.parametrize("m", [512, 2048, 4096])
