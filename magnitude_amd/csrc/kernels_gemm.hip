@@ -923,12 +923,14 @@ size_t q8k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N) {
     return n > 1 ? (size_t)n * M * N * 4 : 0;
 }
 
-// A grid of fewer than 192 tiles leaves the 256 compute units (two workgroups each) mostly idle and a
-// workgroup's K loop is latency-bound: K is then cut into 2 or 3 stretches done by different workgroups.
+// A grid of fewer than 192 tiles leaves the 256 compute units mostly idle and a workgroup's K loop is
+// latency-bound: K is then cut into stretches done by different workgroups, as many as fill one round (32 tiles of
+// K = 14336, Q8_0 at 64 - 128 tokens: 8 stretches instead of 3).
 int per32_splits(int64_t K, int64_t M, int64_t N) {
     static const int forced = tuning_int("QPROJ_PER32_SPLITS", 0);
     const int64_t tiles = ((N + BN - 1) / BN) * ((M + BM - 1) / BM);
-    int n = forced > 0 ? forced : tiles >= 192 ? 1 : tiles >= 96 ? 2 : 3;
+    // as many stretches as fill one round of workgroups (one a compute unit), eight at most
+    int n = forced > 0 ? forced : tiles >= 192 ? 1 : (int)std::min<int64_t>(8, std::max<int64_t>(1, cu_count() / tiles));
     if ((M * N) % 4 != 0) n = 1;
     while (n > 1 && K / 256 < 4 * n) --n;   // at least four super-blocks a stretch
     return n;
