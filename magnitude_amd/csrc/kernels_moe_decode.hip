@@ -1,11 +1,11 @@
-// MUL_MAT_ID for one or two decode tokens (at most 16 (token, expert) pairs) on the vector ALU: no grouping
-// pass, no matrix cores, no separate quantizer or combine launch.
+// MUL_MAT_ID for decode-sized batches (a few tokens; at most about one (token, expert) pair an expert) on the
+// vector ALU: no grouping pass, no matrix cores, no separate quantizer or combine launch.
 //
 // Every pair has its own expert matrix and, for the down projection, its own activation row, so the launch is
 // a set of independent short GEMVs: a workgroup of 16 waves serves a run of weight rows for a GROUP of pairs
 // (one pair; or the n_used pairs of one token when their results are combined here).  It quantizes the
 // group's activation rows into LDS with the arithmetic of the standalone quantizer, and its waves then walk
-// (pair, row step) units.  Expert rows are short (K = 768 .. 4096), so a step covers S = 64 / (4 K/256) whole
+// (row step, pair) units.  Expert rows are short (K = 768 .. 4096), so a step covers S = 64 / (4 K/256) whole
 // rows at once: lane = (row slot, super-block, quarter of the super-block), the row slots' partial dot products
 // are summed over their own lanes only.  Consecutive rows of a matrix are consecutive in memory, so a step's
 // loads cover one contiguous stretch.  With gate and up given, a step walks the same rows of both and stores
@@ -212,10 +212,10 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
 
     if constexpr (COMBINE) {
         __syncthreads();
-        if (tid < r1 - r0) {
-            float s = __fmul_rn(res[tid], cwl[0]);
-            for (int q = 1; q < G; ++q) s = __fadd_rn(s, __fmul_rn(res[q * g.rows_per_wg + tid], cwl[q]));
-            g.y[(int64_t)grp * N + r0 + tid] = s;
+        for (int i = tid; i < r1 - r0; i += kThreads) {
+            float s = __fmul_rn(res[i], cwl[0]);
+            for (int q = 1; q < G; ++q) s = __fadd_rn(s, __fmul_rn(res[q * g.rows_per_wg + i], cwl[q]));
+            g.y[(int64_t)grp * N + r0 + i] = s;
         }
     }
 }
@@ -272,10 +272,11 @@ hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, co
     // compute units, a unit or two a wave, at least half the waves of a workgroup busy.  The registers of a 16-wave
     // workgroup leave room for one a compute unit, so the grid stays within one round.
     const int64_t max_wgs = std::max<int64_t>(1, (int64_t)cu_count() / n_groups);
-    const int64_t steps_per_wg = std::max<int64_t>((steps_total + max_wgs - 1) / max_wgs, std::max<int64_t>(1, kWaves / 2 / group));
+    int64_t steps_per_wg = std::max<int64_t>((steps_total + max_wgs - 1) / max_wgs, std::max<int64_t>(1, kWaves / 2 / group));
+    // the results a workgroup combines wait in LDS: 48 KB of them at most (more workgroups a group beyond that)
+    if (combine_weights) steps_per_wg = std::min<int64_t>(steps_per_wg, std::max<int64_t>(1, 48 * 1024 / 4 / group / S));
     g.rows_per_wg = (int)(steps_per_wg * S);
     g.wgs_per_group = (int)((w.N + g.rows_per_wg - 1) / g.rows_per_wg);
-    if (combine_weights && g.rows_per_wg > kThreads) return hipErrorInvalidValue;   // one thread adds one output row
     const size_t lds = (size_t)group * w.K + (((size_t)group * nb * 4 + 15) & ~(size_t)15) + (size_t)group * (w.K / 16) * 2 +
                        (combine_weights ? (size_t)group * (g.rows_per_wg + 1) * 4 : 0);
     if (lds > 160 * 1024) return hipErrorInvalidValue;

@@ -575,6 +575,30 @@ def test_moe_ffn_expert_per_pair_shapes(ctx, orc, d_model, d_ff, top, B, down_t)
         t.free()
 
 
+def test_moe_ffn_expert_per_pair_many_tokens_one_expert_each(ctx, orc):
+    """100 tokens that name one expert each (no more pairs than experts): more groups than a round of workgroups
+    gives one workgroup a token, which then walks all 2304 output rows and adds them in passes of its threads."""
+    from magnitude_amd import ACT_GGML
+    d_model, d_ff, E, B, base = 2304, 256, 100, 100, 6
+    rng = np.random.default_rng(4242)
+    enc = lambda rows, cols: encode(Q4_K, (rng.standard_normal((base * rows, cols)) * 0.03).astype(np.float32)).reshape(base, rows, -1)
+    pick = rng.integers(0, base, size=E)
+    gate_b, up_b, down_b = (np.ascontiguousarray(t[pick]) for t in (enc(d_ff, d_model), enc(d_ff, d_model), enc(d_model, d_ff)))
+    ids = rng.permutation(E)[:B].astype(np.int32).reshape(B, 1)
+    wts = rng.uniform(0.5, 1.5, size=(B, 1)).astype(np.float32)
+    x = rng.standard_normal((B, d_model)).astype(np.float32)
+    g = ctx.upload(Q4_K, d_model, d_ff, gate_b, n_expert=E)
+    u = ctx.upload(Q4_K, d_model, d_ff, up_b, n_expert=E)
+    d = ctx.upload(Q4_K, d_ff, d_model, down_b, n_expert=E)
+    got = ctx.moe_ffn(g, u, d, dev(x), dev(ids), dev(wts), ACT_GGML).cpu().numpy()
+    want = orc.moe_ffn(Q4_K, Q4_K, gate_b, up_b, down_b, d_model, d_ff, E, x, ids, wts, orc.ACT_GGML)
+    close(got, want, 1e-3)
+    gate(got, want)
+    assert np.median(np.abs(got - want)) <= 2e-6 * np.abs(want).max()
+    for t in (g, u, d):
+        t.free()
+
+
 @pytest.mark.parametrize("qtype,k,n", [(Q4_K, 768, 100), (Q6_K, 1280, 37), (Q4_K, 4096, 5), (Q6_K, 256, 333)])
 def test_mul_mat_id_expert_per_pair_ragged_rows(ctx, orc, qtype, k, n):
     """MUL_MAT_ID alone on that route: row counts that are no multiple of the rows a step covers, a shared activation
