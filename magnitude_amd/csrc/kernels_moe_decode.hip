@@ -7,7 +7,7 @@
 // group's activation rows into LDS with the arithmetic of the standalone quantizer, and its waves then walk
 // (row step, pair) units.  Expert rows are short (K = 768 .. 4096), so a step covers S = 64 / (4 K/256) whole
 // rows at once: lane = (row slot, super-block, quarter of the super-block), the row slots' partial dot products
-// are summed over their own lanes only.  Consecutive rows of a matrix are consecutive in memory, so a step's
+// are summed over their own lanes only.  (Longer rows, LONGK: one row a unit, walked 4096 weights a step.)  Consecutive rows of a matrix are consecutive in memory, so a step's
 // loads cover one contiguous stretch.  With gate and up given, a step walks the same rows of both and stores
 // silu(gate . x) * (up . x); with routing weights given, the workgroup adds its pairs' results in slot order,
 // each product rounded first, which is what the separate combine pass does.
@@ -52,14 +52,17 @@ __device__ __forceinline__ float slot_sum(float v, int vlane, int lpr) {
 }
 
 // R: row steps a unit covers (two where a wave has several units of short rows: fewer, larger requests)
-template <int QT, bool SWIGLU, bool COMBINE, int R>
+// LONGK: rows of more than 4096 weights -- a unit is one row, walked in steps of 16 super-blocks
+template <int QT, bool SWIGLU, bool COMBINE, int R, bool LONGK = false>
 __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArgs g) {
     static_assert(!SWIGLU || R == 1, "gate / up already load two tensors a unit");
+    static_assert(!LONGK || R == 1, "long rows are walked one at a time");
     extern __shared__ __align__(16) uint8_t smem[];
     constexpr int NT = SWIGLU ? 2 : R;   // register sets a unit loads
     const int tid = threadIdx.x, lane = tid & 63, wave = uniform(tid >> 6);
     const int K = (int)g.w0.K, nb = (int)g.w0.nb, N = (int)g.w0.N;
-    const int lpr = 4 * nb, S = 64 / lpr;
+    const int lpr = LONGK ? 64 : 4 * nb, S = 64 / lpr;
+    const int nch = LONGK ? (nb + 15) / 16 : 1;   // steps a unit
     const bool live = lane < S * lpr;
     const int slot = live ? lane / lpr : 0;
     const int vlane = live ? lane - slot * lpr : 0;   // idle lanes repeat a valid address and add nothing
@@ -69,7 +72,7 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
     const int r1 = min(N, r0 + g.rows_per_wg);
     const int steps = r1 > r0 ? (r1 - r0 + S * R - 1) / (S * R) : 0;   // units a pair has here
     const int units = G * steps;
-    const int n_u = units > wave ? (units - wave + kWaves - 1) / kWaves : 0;   // this wave's units: wave, wave + 16, ..
+    const int n_u = (units > wave ? (units - wave + kWaves - 1) / kWaves : 0) * nch;   // this wave's units (wave, wave + 16, ..) x their steps
 
     // LDS: the group's quantized activation rows, then the results to combine
     int8_t *sq = reinterpret_cast<int8_t *>(smem);
@@ -112,7 +115,7 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
     };
     auto unit_of = [&](int i) {
         Unit u;
-        const int idx = wave + kWaves * i;
+        const int idx = wave + kWaves * (LONGK ? i / nch : i);
         const int st = idx / G;
         u.s = idx - st * G;
         u.row = r0 + st * S * R;
@@ -132,7 +135,15 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
         const int64_t first = (int64_t)(issue_e < 0 ? 0 : issue_e) * N + u.row;   // (a pair left out loads somewhere valid)
         RowPtr<QT> rp;
         rp.set(g.w0, first);
-        if constexpr (SWIGLU) {
+        if constexpr (LONGK) {   // lanes past the end of the row repeat its last block
+            const uint32_t blk = (uint32_t)min((i % nch) * 16 + (lane >> 2), nb - 1);
+            raw[0].load(rp, blk, lane, 0);
+            if constexpr (SWIGLU) {
+                RowPtr<QT> ru;
+                ru.set(g.w1, first);
+                raw[NT - 1].load(ru, blk, lane, 0);
+            }
+        } else if constexpr (SWIGLU) {
             const uint32_t rel = (uint32_t)min(slot, r1 - 1 - u.row);
             raw[0].load(rp, (uint32_t)(vlane >> 2), vlane, rel);
             RowPtr<QT> ru;
@@ -147,19 +158,40 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
     int cur_s = -1;
     bool cur_ok = false;
     Dot<QT> dx;
+    float part[NT];   // LONGK: the row's sum so far
+#pragma unroll
+    for (int t = 0; t < NT; ++t) part[t] = 0.f;
     auto consume = [&](const Raw<QT> (&raw)[NT], int i) {
         const Unit u = unit_of(i);
         if (u.s != cur_s) {
             cur_s = u.s;
             cur_ok = expert_of(u.s) >= 0;
-            dx.load_x(xt, u.s, 0, vlane);
+            if constexpr (!LONGK) dx.load_x(xt, u.s, 0, vlane);
         }
         float acc[NT];
+        if constexpr (LONGK) {
+            const int c = i % nch, left = nb - c * 16;          // super-blocks left in the row from this step on
+            const bool there = (lane >> 2) < left;
+            dx.load_x(xt, u.s, c * 4096, there ? lane : (lane & 3));   // (lanes past the end read the step's first block)
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
-            Frag<QT> f;
-            f.unpack(raw[t], vlane);
-            acc[t] = slot_sum(live ? dx.dot(f) : 0.f, vlane, lpr);
+            for (int t = 0; t < NT; ++t) {
+                Frag<QT> f;
+                f.unpack(raw[t], lane);
+                part[t] += there ? dx.dot(f) : 0.f;
+            }
+            if (c + 1 < nch) return;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                acc[t] = slot_sum(part[t], lane, 64);
+                part[t] = 0.f;
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                Frag<QT> f;
+                f.unpack(raw[t], vlane);
+                acc[t] = slot_sum(live ? dx.dot(f) : 0.f, vlane, lpr);
+            }
         }
 #pragma unroll
         for (int t = 0; t < (SWIGLU ? 1 : R); ++t) {
@@ -177,11 +209,15 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
     if (n_u > 0) issue(buf_a, 0);   // in flight while the activations are quantized
 
     if (COMBINE && tid < G) cwl[tid] = cw_mine;
+    auto x_piece = [&](int c) {
+        const int s = c / nb, ch = c - s * nb;
+        return *reinterpret_cast<const float4 *>(g.x + (int64_t)((p0 + s) / g.x_div) * K + ch * 256 + 4 * lane);
+    };
+    float4 x_next = x_first[kAhead - 1];   // pieces beyond the first two are requested one round ahead
     for (int c = wave, a = 0; c < n_chunks; c += kWaves, ++a) {
         const int s = c / nb, ch = c - s * nb;
-        float4 v = x_first[kAhead - 1];
-        if (a == 0) v = x_first[0];
-        else if (a >= kAhead) v = *reinterpret_cast<const float4 *>(g.x + (int64_t)((p0 + s) / g.x_div) * K + ch * 256 + 4 * lane);
+        const float4 v = a == 0 ? x_first[0] : x_next;
+        if (a >= 1 && c + kWaves < n_chunks) x_next = x_piece(c + kWaves);
         int bsum;
         float dd;
         const uint32_t packed = wave_quantize_q8k(v, lane, bsum, dd);
@@ -220,9 +256,9 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
     }
 }
 
-template <int QT, bool SWIGLU, bool COMBINE, int R = 1>
+template <int QT, bool SWIGLU, bool COMBINE, int R = 1, bool LONGK = false>
 hipError_t launch_typed(const MoeDecodeArgs &g, unsigned grid, size_t lds, hipStream_t s) {
-    auto kern = &moe_decode_kernel<QT, SWIGLU, COMBINE, R>;
+    auto kern = &moe_decode_kernel<QT, SWIGLU, COMBINE, R, LONGK>;
     static size_t allowed = 48 * 1024;
     if (lds > allowed) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -235,9 +271,18 @@ hipError_t launch_typed(const MoeDecodeArgs &g, unsigned grid, size_t lds, hipSt
 
 }  // namespace
 
+namespace {
+constexpr size_t kLdsBudget = 158 * 1024;
+// LDS of the group's quantized rows: codes, scales (padded to 16 bytes), block sums
+size_t staged_bytes(int64_t K, int64_t group) {
+    return (size_t)group * K + (((size_t)group * (K / 256) * 4 + 15) & ~(size_t)15) + (size_t)group * (K / 16) * 2;
+}
+}  // namespace
+
 bool moe_decode_fits(int type, int64_t K, int64_t n_pairs, int64_t group) {
-    return (type == kTypeQ4_K || type == kTypeQ6_K) && K % 256 == 0 && K >= 256 && K <= 4096 && n_pairs >= 1 &&
-           n_pairs <= (1 << 20) && group >= 1 && group <= kMaxGroup && n_pairs % group == 0;
+    return (type == kTypeQ4_K || type == kTypeQ6_K) && K % 256 == 0 && K >= 256 && K <= (1 << 20) && n_pairs >= 1 &&
+           n_pairs <= (1 << 20) && group >= 1 && group <= kMaxGroup && n_pairs % group == 0 &&
+           staged_bytes(K, group) + (size_t)group * 4 * 64 + 64 <= kLdsBudget;   // room for 64 result rows a pair at least
 }
 
 // args: t[0] (and t[1] = up when swiglu) expert stacks, x fp32 rows, x_div, ids, n_pairs, error_flag as for the
@@ -265,7 +310,9 @@ hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, co
     g.y = args.t[0].y;
     g.cw = combine_weights;
     g.group = group;
-    const int nb = (int)w.nb, S = 64 / (4 * nb);
+    const int nb = (int)w.nb;
+    const bool long_k = nb > 16;
+    const int S = long_k ? 1 : 64 / (4 * nb);
     const int n_groups = args.n_pairs / group;
     const int64_t steps_total = (w.N + S - 1) / S;
     // The launch is latency-bound (all loads of the call are in flight at once): the rows are spread over all
@@ -273,18 +320,30 @@ hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, co
     // workgroup leave room for one a compute unit, so the grid stays within one round.
     const int64_t max_wgs = std::max<int64_t>(1, (int64_t)cu_count() / n_groups);
     int64_t steps_per_wg = std::max<int64_t>((steps_total + max_wgs - 1) / max_wgs, std::max<int64_t>(1, kWaves / 2 / group));
-    // the results a workgroup combines wait in LDS: 48 KB of them at most (more workgroups a group beyond that)
-    if (combine_weights) steps_per_wg = std::min<int64_t>(steps_per_wg, std::max<int64_t>(1, 48 * 1024 / 4 / group / S));
+    // the results a workgroup combines wait in LDS: 48 KB of them at most, less beside long staged rows (more
+    // workgroups a group beyond that)
+    const size_t staged = staged_bytes(w.K, group);
+    if (combine_weights) {
+        const size_t room = std::min<size_t>(48 * 1024, kLdsBudget - staged - 64);
+        steps_per_wg = std::min<int64_t>(steps_per_wg, std::max<int64_t>(1, (int64_t)(room / 4 / group / S)));
+    }
     g.rows_per_wg = (int)(steps_per_wg * S);
     g.wgs_per_group = (int)((w.N + g.rows_per_wg - 1) / g.rows_per_wg);
-    const size_t lds = (size_t)group * w.K + (((size_t)group * nb * 4 + 15) & ~(size_t)15) + (size_t)group * (w.K / 16) * 2 +
-                       (combine_weights ? (size_t)group * (g.rows_per_wg + 1) * 4 : 0);
+    const size_t lds = staged + (combine_weights ? (size_t)group * (g.rows_per_wg + 1) * 4 : 0);
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     if (dry_run()) return hipSuccess;
     const unsigned grid = (unsigned)(n_groups * g.wgs_per_group);
     // two row steps a unit where a wave would otherwise walk four or more units of rows that fill under 4 KB a step
     static const int two_env = tuning_int("QPROJ_MOE_DECODE_TWO_STEPS", -1);
-    const bool two = two_env >= 0 ? two_env != 0 : (!swiglu && group * steps_per_wg >= 4 * kWaves);
+    const bool two = !long_k && (two_env >= 0 ? two_env != 0 : (!swiglu && group * steps_per_wg >= 4 * kWaves));
+    if (long_k) {
+        if (w.type == kTypeQ4_K) {
+            if (swiglu) return launch_typed<kTypeQ4_K, true, false, 1, true>(g, grid, lds, s);
+            return combine_weights ? launch_typed<kTypeQ4_K, false, true, 1, true>(g, grid, lds, s) : launch_typed<kTypeQ4_K, false, false, 1, true>(g, grid, lds, s);
+        }
+        if (swiglu) return launch_typed<kTypeQ6_K, true, false, 1, true>(g, grid, lds, s);
+        return combine_weights ? launch_typed<kTypeQ6_K, false, true, 1, true>(g, grid, lds, s) : launch_typed<kTypeQ6_K, false, false, 1, true>(g, grid, lds, s);
+    }
     if (w.type == kTypeQ4_K) {
         if (swiglu) return launch_typed<kTypeQ4_K, true, false>(g, grid, lds, s);
         if (two) return combine_weights ? launch_typed<kTypeQ4_K, false, true, 2>(g, grid, lds, s) : launch_typed<kTypeQ4_K, false, false, 2>(g, grid, lds, s);

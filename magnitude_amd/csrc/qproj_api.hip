@@ -490,11 +490,14 @@ bool grouped_pair_mode(int type, int64_t K, int64_t n_pairs, int64_t E) {
 // at one token, 24.9 -> 18.8 at two, 41.0 -> 23.2 at four, 57.6 -> 36.2 at eight, 74.1 -> 58.9 at sixteen, level at twenty to
 // twenty-four and worse at 32 (101 against 95 us); with
 // more pairs than experts the repeated reads of an expert outweigh the launches saved.
-bool moe_decode_route(int type, int64_t K, int64_t n_pairs, int64_t group, int64_t E) {
+// (Up to 16 pairs take it whatever the expert count while an expert matrix is small, two million weights at most: launches
+// weigh more than bytes there.  Large experts do not: 8 experts of 4096 x 14336, 16 pairs: 214 us grouped, 220 us this way.)
+bool moe_decode_route(int type, int64_t K, int64_t N, int64_t n_pairs, int64_t group, int64_t E) {
     static const bool on = tuning_int("QPROJ_NO_MOE_DECODE", 0) == 0;
     static const int max_pairs = tuning_int("QPROJ_MOE_DECODE_MAX_PAIRS", 128);
     static const int per_4_experts = tuning_int("QPROJ_MOE_DECODE_PAIRS_PER_4_EXPERTS", 4);
-    return on && (n_pairs <= 16 || (n_pairs <= max_pairs && 4 * n_pairs <= per_4_experts * E)) && moe_decode_fits(type, K, n_pairs, group);
+    const bool few = n_pairs <= 16 && K * N <= ((int64_t)2 << 20);
+    return on && (few || (n_pairs <= max_pairs && 4 * n_pairs <= per_4_experts * E)) && moe_decode_fits(type, K, n_pairs, group);
 }
 
 int grouped_mt(int64_t n_pairs, int64_t E) {
@@ -1091,7 +1094,7 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     if (B == 0) return QPROJ_OK;
     QP_HIP(ctx, hipSetDevice(ctx->device));
     const int64_t K = w->K, n_pairs = B * n_used, rows = B * nb1;
-    if (moe_decode_route(w->type, K, n_pairs, 1, w->E)) {
+    if (moe_decode_route(w->type, K, w->N, n_pairs, 1, w->E)) {
         GemvArgs g{};
         g.n_targets = 1;
         g.t[0].w = w->view;
@@ -1187,7 +1190,7 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     float *e = reinterpret_cast<float *>(ws + off_e);
     const int mt = grouped_mt(n_pairs, E);
 
-    if (moe_decode_route(gate->type, d_model, n_pairs, 1, E) && moe_decode_route(down->type, d_ff, n_pairs, n_used, E)) {
+    if (moe_decode_route(gate->type, d_model, d_ff, n_pairs, 1, E) && moe_decode_route(down->type, d_ff, d_model, n_pairs, n_used, E)) {
         GemvArgs g{};
         g.n_targets = 2;
         g.t[0].w = gate->view;

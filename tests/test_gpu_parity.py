@@ -575,6 +575,32 @@ def test_moe_ffn_expert_per_pair_shapes(ctx, orc, d_model, d_ff, top, B, down_t)
         t.free()
 
 
+@pytest.mark.parametrize("B,down_t", [(1, Q4_K), (2, Q6_K)])
+def test_moe_ffn_expert_per_pair_long_rows(ctx, orc, B, down_t):
+    """Experts whose rows are longer than one 4096-weight step (17 and 18 super-blocks: a full step and a ragged
+    one): a unit is one row walked step by step, the last step's idle lanes add nothing."""
+    from magnitude_amd import ACT_GGML
+    d_model, d_ff, E, top = 4352, 4608, 3, 2
+    rng = np.random.default_rng(17 + B)
+    enc = lambda t, rows, cols: encode(t, (rng.standard_normal((E * rows, cols)) * 0.02).astype(np.float32)).reshape(E, rows, -1)
+    gate_b, up_b, down_b = enc(Q4_K, d_ff, d_model), enc(Q4_K, d_ff, d_model), enc(down_t, d_model, d_ff)
+    ids, wts = routing(rng, B, top, E)
+    x = rng.standard_normal((B, d_model)).astype(np.float32)
+    g = ctx.upload(Q4_K, d_model, d_ff, gate_b, n_expert=E)
+    u = ctx.upload(Q4_K, d_model, d_ff, up_b, n_expert=E)
+    d = ctx.upload(down_t, d_ff, d_model, down_b, n_expert=E)
+    got = ctx.moe_ffn(g, u, d, dev(x), dev(ids), dev(wts), ACT_GGML).cpu().numpy()
+    want = orc.moe_ffn(Q4_K, down_t, gate_b, up_b, down_b, d_model, d_ff, E, x, ids, wts, orc.ACT_GGML)
+    close(got, want, 1e-3)
+    gate(got, want)
+    assert np.median(np.abs(got - want)) <= 2e-6 * np.abs(want).max()
+    xs = rng.standard_normal((B, top, d_ff)).astype(np.float32)          # MUL_MAT_ID alone, a row per slot
+    got = ctx.mul_mat_id(d, dev(xs), dev(ids), ACT_GGML).cpu().numpy()
+    close(got, orc.mul_mat_id(down_t, down_b, d_ff, d_model, E, xs, ids), 2e-5)
+    for t in (g, u, d):
+        t.free()
+
+
 def test_moe_ffn_expert_per_pair_many_tokens_one_expert_each(ctx, orc):
     """100 tokens that name one expert each (no more pairs than experts): more groups than a round of workgroups
     gives one workgroup a token, which then walks all 2304 output rows and adds them in passes of its threads."""
