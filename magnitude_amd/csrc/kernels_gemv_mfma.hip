@@ -524,9 +524,10 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
             n_rows = 1;
         } else {
             if (slot >= g.active[g.n_expert]) return;
-            expert = g.active[slot];
-            pair0 = g.offsets[expert];
-            n_rows = g.offsets[expert + 1] - pair0;
+            const int4 rec = reinterpret_cast<const int4 *>(g.active + active_slots_offset(g.n_expert))[slot];
+            expert = rec.x;   // (one load: the list position's expert, first pair slot and pair count)
+            pair0 = rec.y;
+            n_rows = rec.z;
             if (n_rows <= 0) return;
         }
     } else {

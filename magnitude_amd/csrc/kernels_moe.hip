@@ -77,7 +77,9 @@ __device__ __forceinline__ void group_scan(int n_expert, int32_t *cnt, int32_t *
             before += tot[i];
             if (tot[i] > 0) {
                 const bool heavy = pass_rows > 0 && tot[i] > pass_rows;
-                active[heavy ? before_h : n_heavy + (before_f - before_h)] = e;
+                const int pos = heavy ? before_h : n_heavy + (before_f - before_h);
+                active[pos] = e;
+                reinterpret_cast<int4 *>(active + active_slots_offset(n_expert))[pos] = make_int4(e, before - tot[i], tot[i], 0);
                 ++before_f;
                 before_h += heavy;
             }

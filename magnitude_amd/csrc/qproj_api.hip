@@ -1111,7 +1111,7 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     const size_t off_order = p.total;
     const size_t off_offsets = off_order + align_up((size_t)n_pairs * 4);
     const size_t off_active = off_offsets + align_up((size_t)(w->E + 1) * 4);
-    const size_t total = off_active + align_up((size_t)(w->E + 1) * 4);
+    const size_t total = off_active + align_up(active_list_bytes(w->E));
     int rc = ensure_ws(ctx, total);
     if (rc) return rc;
     // few pairs an expert: the grouped kernel quantizes the rows it needs in its prologue
@@ -1173,7 +1173,7 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     const size_t off_offsets = off;
     off += align_up((size_t)(E + 1) * 4);
     const size_t off_active = off;
-    off += align_up((size_t)(E + 1) * 4);
+    off += align_up(active_list_bytes(E));
     const size_t off_h = off;
     off += align_up((size_t)(n_pairs * d_ff) * 4);
     const size_t off_hq = off;

@@ -74,7 +74,8 @@ struct GemvArgs {
     // expert-grouped mode (MUL_MAT_ID); null order = dense
     const int32_t *order;   // pair indices sorted by expert
     const int32_t *offsets; // [E+1] ranges into order
-    const int32_t *active;  // [E+1] experts that have pairs, ascending; [E] = how many
+    const int32_t *active;  // [E+1] experts that have pairs, ascending; [E] = how many; behind it (active_slots_offset)
+                            // one {expert, first pair slot, pairs, 0} record a list position
     int x_div;              // activation row of pair p is p / x_div
     // pair mode of the grouped matrix-core kernel (a handful of pairs, no grouping pass): a set of
     // workgroups per pair p multiplies row p / x_div by expert ids[p]; ids outside [0, E) raise *error_flag
@@ -116,6 +117,12 @@ inline int wide_tile_splits(int64_t tiles, int64_t nsb, int64_t M, int64_t N, in
     }
     return best;
 }
+
+// The busy-expert list of the grouping pass: n_expert + 1 ints (the list, then its length), then from a 16-byte boundary
+// one int4 {expert, its first slot in order[], its pairs, 0} per list position, so that a workgroup of the grouped
+// kernels learns all three from ONE load instead of a chain of two.
+__host__ __device__ inline int64_t active_slots_offset(int64_t n_expert) { return (n_expert + 1 + 3) & ~(int64_t)3; }   // in ints
+inline size_t active_list_bytes(int64_t n_expert) { return (size_t)(active_slots_offset(n_expert) + 4 * n_expert) * 4; }
 
 // Compute units of the current device (256 when no device can be asked, e.g. in a dry run on a host without one).
 int cu_count();
