@@ -434,6 +434,85 @@ __device__ __forceinline__ void stage_activations(const MfmaArgs &g, uint8_t *sm
     }
 }
 
+// The same staging in two halves for the expert-grouped launches, whose few rows (a handful of pairs an expert) are
+// one request or two a thread: `request` asks for everything -- codes, scales, block sums -- and `store` files it in
+// LDS.  In between the workgroup asks for its first weights.  Loads return in order: requested behind the weights
+// (as the one-piece version above is), these few kilobytes that sit in L2 came back only after the weights' trip to
+// HBM, one dependent round after the other -- 4.6 us of a workgroup's 12.5 (down projection, 64 tokens, phase clocks).
+template <int QT, int MT, int kThreads>
+struct StagedRows {
+    static constexpr int kPieces = 4;
+    uint4 v[kPieces], b0, b1;
+    int dst[kPieces];
+    float dval;
+    static __device__ __forceinline__ bool fits(int n_rows, int nsb) {
+        return QT != kTypeQ8_0 /* (its instances have no registers to spare) */ && n_rows * nsb * 16 <= kPieces * kThreads &&
+               n_rows * nsb * Cfg<QT>::kDx <= kThreads;
+    }
+    __device__ __forceinline__ void request(const MfmaArgs &g, const uint8_t *smem, const Layout &L, int c0, int nsb, int n_rows) {
+        const int tid = threadIdx.x, nb = (int)(g.a.K >> 8), row16 = nsb * 16, total = n_rows * row16;
+        const int *map = reinterpret_cast<const int *>(smem + L.off_map);
+        auto src_row = [&](int m) -> size_t { return (size_t)(map[m] / g.x_div); };
+#pragma unroll
+        for (int u = 0; u < kPieces; ++u) {
+            const int idx = min(u * kThreads + tid, total - 1);
+            const int m = idx / row16, j = idx - m * row16;
+            v[u] = *reinterpret_cast<const uint4 *>(g.a.qs + src_row(m) * g.a.K + (size_t)c0 * 256 + j * 16);
+            dst[u] = m * L.lda + j * 16;
+        }
+        constexpr int ND = Cfg<QT>::kDx;
+        const int nd = nsb * ND;
+        dval = 0.f;
+        if (tid < n_rows * nd) {
+            const int m = tid / nd, j = tid - m * nd;
+            dval = g.a.d[src_row(m) * (nb * ND) + c0 * ND + j];
+        }
+        b0 = b1 = make_uint4(0, 0, 0, 0);
+        if (QT != kTypeQ8_0 && tid < n_rows * nsb) {
+            const int m = tid / nsb, sb = tid - m * nsb;
+            const uint4 *src = reinterpret_cast<const uint4 *>(g.a.bsums + (src_row(m) * nb + c0 + sb) * 16);
+            b0 = src[0];
+            b1 = src[1];
+        }
+    }
+    __device__ __forceinline__ void store(uint8_t *smem, const Layout &L, int nsb, int n_rows) const {
+        const int tid = threadIdx.x;
+#pragma unroll
+        for (int u = 0; u < kPieces; ++u) *reinterpret_cast<uint4 *>(smem + dst[u]) = v[u];
+        constexpr int ND = Cfg<QT>::kDx;
+        const int nd = nsb * ND;
+        if (tid < n_rows * nd) {
+            const int m = tid / nd, j = tid - m * nd;
+            reinterpret_cast<float *>(smem + L.off_dx)[j * MT + m] = dval;
+        }
+        if constexpr (QT != kTypeQ8_0) {
+            if (tid < n_rows * nsb) {
+                const int m = tid / nsb, sb = tid - m * nsb;
+                const uint32_t w[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+                uint8_t *dstb = smem + L.off_aux + (sb * MT + m) * Cfg<QT>::kAux;
+                if constexpr (QT == kTypeQ4_K) {
+                    uint32_t hi[2] = {0, 0}, lo[2] = {0, 0};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const int s = (int)(int16_t)(w[j] & 0xffff) + (int)(int16_t)(w[j] >> 16);
+                        split_sum(s, hi[j >> 2], lo[j >> 2], j & 3);
+                    }
+                    *reinterpret_cast<uint4 *>(dstb) = make_uint4(hi[0], hi[1], lo[0], lo[1]);
+                } else {
+                    uint32_t hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
+#pragma unroll
+                    for (int j = 0; j < 16; ++j) {
+                        const int s = (int)(int16_t)((w[j >> 1] >> (16 * (j & 1))) & 0xffff);
+                        split_sum(s, hi[j >> 2], lo[j >> 2], j & 3);
+                    }
+                    *reinterpret_cast<uint4 *>(dstb) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+                    *reinterpret_cast<uint4 *>(dstb + 16) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+                }
+            }
+        }
+    }
+};
+
 // The same LDS image made from fp32 rows: each wave quantizes whole 256-element chunks (ggml's
 // quantize_row_q8_K, or eight quantize_row_q8_0 blocks for Q8_0 weights) exactly as the standalone
 // quantizer kernels do, so both routes stage identical bytes.  Two chunks are in flight per wave.
@@ -620,7 +699,9 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
                 // groups all lie past the end of the matrix (total = 0) only takes part in the staging and the barriers
                 int arg = 0, ai = 0, brg = 0, bi = 1, crg = 0, ci = 0;
                 while (bi >= per) { bi -= per; ++brg; }
-                if (total > 0) {
+                // rows quantized earlier, few enough for one request round: asked for AHEAD of the first weights
+                const bool rows_first = !g.x && StagedRows<QT, MT, W * 64>::fits(m_cnt, nsb);
+                if (!rows_first && total > 0) {
                     issue_at(sa, rg_a, arg, ai);
                     issue_at(sb_, rg_b, brg, bi);
                 }
@@ -630,10 +711,19 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
                                        : g.ids      ? pair0 + m0 + (int)threadIdx.x
                                                     : g.order[pair0 + m0 + (int)threadIdx.x];
                 __syncthreads();
-                if (g.x)
+                if (rows_first) {
+                    StagedRows<QT, MT, W * 64> rows;
+                    rows.request(g, smem, L, c0, nsb, m_cnt);
+                    if (total > 0) {
+                        issue_at(sa, rg_a, arg, ai);
+                        issue_at(sb_, rg_b, brg, bi);
+                    }
+                    rows.store(smem, L, nsb, m_cnt);
+                } else if (g.x) {
                     stage_quantize<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
-                else
+                } else {
                     stage_activations<QT, MT, W * 64, GROUPED>(g, smem, L, c0, nsb, m_cnt, m0);
+                }
                 __syncthreads();
 
                 float out[NT][NV];
