@@ -20,9 +20,18 @@ __device__ __forceinline__ float4 load_rows4(const float *__restrict__ x, const 
     return v;
 }
 
+// the launch's threads clear the job's rows between them, four floats a store
+__device__ __forceinline__ void zero_rows(const ZeroJob &z) {
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, nthr = (int64_t)gridDim.x * blockDim.x;
+    for (int i = 0; i < z.count; ++i)
+        for (int64_t e = tid * 4; e < z.n[i]; e += nthr * 4)
+            *reinterpret_cast<float4 *>(z.p[i] + e) = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
 __global__ __launch_bounds__(256) void quant_q8k_kernel(const float *__restrict__ x, const float *__restrict__ u, int64_t n_super,
                                                         int8_t *__restrict__ qs, float *__restrict__ d,
-                                                        int16_t *__restrict__ bsums) {
+                                                        int16_t *__restrict__ bsums, const ZeroJob zero) {
+    zero_rows(zero);
     const int64_t sb = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (sb >= n_super) return;  // whole wave leaves together
@@ -35,7 +44,9 @@ __global__ __launch_bounds__(256) void quant_q8k_kernel(const float *__restrict_
 template <bool FP16_SCALE>
 __global__ __launch_bounds__(256) void quant_q8_32_kernel(const float *__restrict__ x, const float *__restrict__ u, int64_t n_chunks256,
                                                           int64_t n_elems, int8_t *__restrict__ qs,
-                                                          float *__restrict__ d, int32_t *__restrict__ isum) {
+                                                          float *__restrict__ d, int32_t *__restrict__ isum,
+                                                          const ZeroJob zero) {
+    zero_rows(zero);
     const int64_t ch = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (ch >= n_chunks256) return;
@@ -138,10 +149,18 @@ hipError_t launch_minterm_rows(int kind, const float *d, const int16_t *bsums, c
 // msum / rs null: the min-term plane is not wanted (the decode, small-batch and expert-grouped kernels take the block
 // sums themselves)
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
-                               int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s, const float *u) {
+                               int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s, const float *u,
+                               const ZeroJob *zero) {
     const int64_t n = M * K;
     if (n == 0) return hipSuccess;
     if (kind != kActKindQ8_K && kind != kActKindQ8_0 && kind != kActKindQ8X32) return hipErrorInvalidValue;
+    ZeroJob zj{};
+    if (zero) {
+        if (msum || kind == kActKindQ8X32) return hipErrorInvalidValue;   // the launches below that carry the job
+        zj = *zero;
+        for (int i = 0; i < zj.count; ++i)
+            if (zj.n[i] % 4 != 0 || (reinterpret_cast<uintptr_t>(zj.p[i]) & 15) != 0) return hipErrorInvalidValue;
+    }
     if (dry_run()) return hipSuccess;
     // with the min-term plane wanted: one launch, a workgroup per row (measured against the quantizer followed by
     // the min-term launch: 4.6 against 7.1 us at 128 x 4096, 9.3 against 10.6 at 512 x 14336; many short rows are
@@ -160,11 +179,11 @@ hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, i
     const int64_t chunks = (n + 255) / 256;
     const dim3 grid((unsigned)((chunks + 3) / 4)), block(256);
     if (kind == kActKindQ8_K) {
-        hipLaunchKernelGGL(quant_q8k_kernel, grid, block, 0, s, x, u, n / 256, qs, d, bsums);
+        hipLaunchKernelGGL(quant_q8k_kernel, grid, block, 0, s, x, u, n / 256, qs, d, bsums, zj);
     } else if (kind == kActKindQ8_0) {
-        hipLaunchKernelGGL(quant_q8_32_kernel<true>, grid, block, 0, s, x, u, chunks, n, qs, d, isum);
+        hipLaunchKernelGGL(quant_q8_32_kernel<true>, grid, block, 0, s, x, u, chunks, n, qs, d, isum, zj);
     } else {
-        hipLaunchKernelGGL(quant_q8_32_kernel<false>, grid, block, 0, s, x, u, chunks, n, qs, d, isum);
+        hipLaunchKernelGGL(quant_q8_32_kernel<false>, grid, block, 0, s, x, u, chunks, n, qs, d, isum, zj);
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess || kind == kActKindQ8_0 || !msum) return e;

@@ -21,7 +21,11 @@
 // of a row group are summed through LDS in a fixed order.  When one workgroup cannot hold the
 // whole K range (LDS) or there would be too few workgroups, K is also cut into chunks whose
 // results go to a scratch buffer that a second small kernel sums in chunk order, so results do
-// not depend on scheduling.
+// not depend on scheduling.  Exactly two chunks, with output rows that the quantizer launch in
+// front has cleared, add their results to the output themselves (float add at the memory side,
+// nothing returned): two addends on zero give the same sum in either order, so this does not
+// depend on scheduling either, and the summing launch goes.  (The memory-side adder may flush a
+// sum below the smallest normal float to zero.)
 #include <stdlib.h>
 
 #include <algorithm>
@@ -52,6 +56,7 @@ struct MfmaArgs {
     ActView a;
     const float *x;        // non-null: fp32 activation rows [rows][K], quantized by every workgroup in its prologue
     int M, n_chunks, chunk_sb, kw, rw, n_wgs;
+    int add_out;           // dense mode, two chunks, output rows cleared before the launch: both chunks add to y
     // expert-grouped mode (MUL_MAT_ID): activation rows of expert e are the pairs order[offsets[e]..offsets[e+1])
     const int32_t *order;
     const int32_t *offsets;
@@ -854,14 +859,20 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
             }
         }
         if (kp == 0 && rows_ok) {
-            float *dst = GROUPED || g.n_chunks == 1 ? y : part + (size_t)c * g.M * N;
+            const bool add = !GROUPED && g.add_out;
+            float *dst = GROUPED || g.n_chunks == 1 || add ? y : part + (size_t)c * g.M * N;
             const int n = row0 + nl;
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
                 const int m = 8 * (v >> 2) + 4 * h + (v & 3);
                 float r = out[0][v];
                 if constexpr (SWIGLU) r = (r / (1.0f + expf(-r))) * out[NT - 1][v];
-                if (m < m_cnt && n < N) dst[(size_t)(GROUPED ? map[m] : m0 + m) * N + n] = r;
+                if (m < m_cnt && n < N) {
+                    float *o = dst + (size_t)(GROUPED ? map[m] : m0 + m) * N + n;
+                    // two addends on zero: the sum does not depend on which chunk arrives first
+                    if (add) unsafeAtomicAdd(o, r);
+                    else *o = r;
+                }
             }
         }
     }
@@ -898,7 +909,7 @@ hipError_t launch_one(const MfmaArgs &g, hipStream_t s) {
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)g.n_wgs), dim3(W * 64), (size_t)L.total, s, g);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess || g.n_chunks == 1) return e;
+    if (e != hipSuccess || g.n_chunks == 1 || g.add_out) return e;
     size_t n_out = 0;
     for (int i = 0; i < g.n_targets; ++i) n_out = std::max(n_out, (size_t)g.M * (size_t)g.t[i].w.N);
     const unsigned blocks = (unsigned)std::min<size_t>(256, (n_out + 255) / 256);
@@ -975,6 +986,11 @@ size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, in
     return p.n_chunks > 1 ? (size_t)p.n_chunks * (size_t)M * (size_t)sum_n * 4 : 0;
 }
 
+bool mfma_gemv_two_chunks(int type, int64_t K, int64_t M, int64_t total_rg) {
+    static const bool off = tuning_int("QPROJ_NO_CHUNK_ADD", 0) != 0;
+    return !off && plan(K, M, total_rg, waves_per_wg(type), 200, true, cu_count()).n_chunks == 2;
+}
+
 hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStream_t s) {
     MfmaArgs g{};
     g.n_targets = args.n_targets;
@@ -991,6 +1007,7 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStr
     g.kw = p.kw;
     g.rw = W / p.kw;
     g.rg_loop = 1;
+    g.add_out = args.y_zeroed && mfma_gemv_two_chunks(args.t[0].w.type, args.a.K, args.M, total_rg);
     int wg = 0;
     size_t part_off = 0;
     for (int i = 0; i < args.n_targets; ++i) {
@@ -1005,7 +1022,7 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStr
     }
     g.n_wgs = wg;
     // the per-chunk results of all targets lie one behind the other in the scratch: refuse what would not fit
-    if (g.n_chunks > 1 && (!scratch.p || part_off * sizeof(float) > scratch.bytes)) return hipErrorInvalidValue;
+    if (g.n_chunks > 1 && !g.add_out && (!scratch.p || part_off * sizeof(float) > scratch.bytes)) return hipErrorInvalidValue;
     return launch_typed<kDense>(g, args.t[0].w.type, args.M <= 8, W, s);
 }
 

@@ -207,14 +207,14 @@ RowQuantJob quantize_job(const ActPlanes &p, uint8_t *base, const float *x, int6
 
 // minterm: also the min-term plane and the row normalisers that only the tiled Q4_K kernels read (a second, small launch)
 hipError_t run_quantize(qproj_ctx *ctx, const ActPlanes &p, uint8_t *base, const float *x, int64_t M, int64_t K,
-                        bool minterm = true, const float *swiglu_u = nullptr) {
+                        bool minterm = true, const float *swiglu_u = nullptr, const ZeroJob *zero = nullptr) {
     const bool mt = minterm && (p.kind == kActKindQ8_K || p.kind == kActKindQ8X32);
     return launch_quantize_act(p.kind, x, M, K, reinterpret_cast<int8_t *>(base + p.off_qs),
                                reinterpret_cast<float *>(base + p.off_d),
                                reinterpret_cast<int16_t *>(base + p.off_aux),
                                mt ? reinterpret_cast<uint16_t *>(base + p.off_msum) : nullptr,
                                reinterpret_cast<int32_t *>(base + p.off_aux),
-                               mt ? reinterpret_cast<float *>(base + p.off_rs) : nullptr, ctx->stream, swiglu_u);
+                               mt ? reinterpret_cast<float *>(base + p.off_rs) : nullptr, ctx->stream, swiglu_u, zero);
 }
 
 ActView act_rows(const ActView &a, int64_t m0) {
@@ -402,9 +402,29 @@ bool dense_fuses_quantizer(const qproj_weight *w, int64_t M) {
     return on && M <= 16 && use_mfma_kernel(w->type, M, w->K);
 }
 
-// x_f32: non-null when `a` carries no planes and the kernel quantizes these rows itself (small batches only)
+// The quantizer launch in front of the small-batch kernel clears the output rows where a pass of that kernel cuts K
+// in two chunks: the chunks then add themselves to the output and the launch that summed them goes (8B down
+// projection, 14336 -> 4096 Q6_K, at 4 and 8 rows).  Fills `z` and answers true when that is the case.
+bool dense_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *const *y, ZeroJob &z) {
+    if (takes_tiled(w[0], M) || !use_mfma_kernel(w[0]->type, M, w[0]->K)) return false;
+    int64_t rgs = 0;
+    for (int i = 0; i < n; ++i) rgs += (w[i]->N + 31) / 32;
+    bool any = mfma_gemv_two_chunks(w[0]->type, w[0]->K, std::min<int64_t>(M, 16), rgs);
+    if (M > 16 && M % 16) any = any || mfma_gemv_two_chunks(w[0]->type, w[0]->K, M % 16, rgs);
+    if (!any) return false;
+    z.count = n;
+    for (int i = 0; i < n; ++i) {
+        z.p[i] = y[i];
+        z.n[i] = M * w[i]->N;
+        if (z.n[i] % 4 != 0 || (reinterpret_cast<uintptr_t>(y[i]) & 15) != 0) return false;
+    }
+    return true;
+}
+
+// x_f32: non-null when `a` carries no planes and the kernel quantizes these rows itself (small batches only);
+// y_zeroed: the output rows were cleared by the quantizer launch (dense_clears_rows)
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
-                    float *const *y, const Scratch &sc, const float *x_f32 = nullptr) {
+                    float *const *y, const Scratch &sc, const float *x_f32 = nullptr, bool y_zeroed = false) {
     // Beyond the rows one pass of the small-batch kernel takes: the tiled product, weights reused across a tile of
     // tokens, K cut into stretches where the grid would leave the chip idle.  (Measured, 8B shapes: Q4_K 17..47
     // rows 19-72 us in steps of 16 against 15-31 us tiled; Q6_K pays from 32 rows on.)
@@ -437,6 +457,7 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
             g.x = x_f32;   // (only with M <= 16: a single pass)
             g.M = (int)mc;
             g.x_div = 1;
+            g.y_zeroed = y_zeroed;
             QP_HIP(ctx, launch_gemv_mfma(g, sc, ctx->stream));
         }
         return QPROJ_OK;
@@ -855,6 +876,8 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
         uint8_t *ws = wsp.base;
         // the min-term plane (a second small launch, one wave a row) only where a tiled Q4_K kernel will read it
         const bool minterm = act == kActQ8X32 || (w[0]->type == kTypeQ4_K && takes_tiled(w[0], M));
+        ZeroJob zero{};
+        bool y_zeroed = false;
         if (norm) {   // norm, weights and quantizer in one launch
             if (p.kind == kActKindQ8X32 && K % 256 != 0)
                 return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_rms_norm_mul_mat: the per-32 format needs K % 256 == 0");
@@ -865,12 +888,13 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
                                         reinterpret_cast<int32_t *>(ws + p.off_aux),
                                         minterm ? reinterpret_cast<float *>(ws + p.off_rs) : nullptr, ctx->stream));
         } else {
-            QP_HIP(ctx, run_quantize(ctx, p, ws, x_dev, M, K, minterm, swiglu_u));
+            y_zeroed = act == kActGGML && !minterm && dense_clears_rows(n, w, M, y_dev, zero);
+            QP_HIP(ctx, run_quantize(ctx, p, ws, x_dev, M, K, minterm, swiglu_u, y_zeroed ? &zero : nullptr));
         }
         const ActView a = act_view(p, ws, K);
         // the partial results lie behind the activation planes; `extra` is all a launcher may use of it
         const Scratch sc{extra ? reinterpret_cast<float *>(ws + p.total) : nullptr, extra};
-        if (act == kActGGML) return run_dense_q8act(ctx, n, w, a, M, y_dev, sc);
+        if (act == kActGGML) return run_dense_q8act(ctx, n, w, a, M, y_dev, sc, nullptr, y_zeroed);
         for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], sc, ctx->stream));
         return QPROJ_OK;
     }

@@ -71,6 +71,8 @@ struct GemvArgs {
     bool swiglu_pair;          // decode kernel: targets 0 and 1 are gate and up of one FFN (same K and N); a wave
                                // walks row r of both and stores silu(gate_r . x) * (up_r . x) to t[0].y
     int M;                 // activation rows in this launch (dense mode), <= MT
+    bool y_zeroed;         // small-batch kernel, dense mode: the output rows hold zeros when the launch starts (the
+                           // quantizer launch in front of it cleared them), so two K chunks may add themselves
     // expert-grouped mode (MUL_MAT_ID); null order = dense
     const int32_t *order;   // pair indices sorted by expert
     const int32_t *offsets; // [E+1] ranges into order
@@ -140,10 +142,18 @@ hipError_t launch_repack_to_gguf(int type, const WeightView &w, uint8_t *gguf, i
 // (msum and rs may be null together: the min-term plane of the tiled Q4_K kernels is then not made)
 hipError_t launch_rms_norm(int kind, const float *x, const float *gamma, float eps, int64_t M, int64_t K, float *y,
                            int8_t *qs, float *d, int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s);
-// u non-null: the rows quantized are silu(x) * u (the swiglu between gate / up and the down projection)
+// Output rows that a quantizer launch clears on the side (n[i] floats at p[i], n[i] % 4 == 0, 16-byte aligned): the
+// projection launched behind it may then add partial results into them instead of storing them.
+struct ZeroJob {
+    int count;
+    float *p[kMaxTargets];
+    int64_t n[kMaxTargets];
+};
+// u non-null: the rows quantized are silu(x) * u (the swiglu between gate / up and the down projection);
+// zero (only without the min-term plane, Q8_K and Q8_0 kinds): see ZeroJob
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
                                int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s,
-                               const float *u = nullptr);
+                               const float *u = nullptr, const ZeroJob *zero = nullptr);
 // the min-term plane and the row normalisers from planes already quantized (one wave per row)
 hipError_t launch_minterm_rows(int kind, const float *d, const int16_t *bsums, const int32_t *isum, int64_t M, int64_t K,
                                uint16_t *msum, float *rs, hipStream_t s);
@@ -156,6 +166,9 @@ hipError_t launch_gemv_decode(const GemvArgs &args, int mt, bool fuse_quantize, 
 // results when K > 4096 (mfma_gemv_scratch_bytes, 0 if none is needed)
 bool mfma_gemv_fits(int type, int64_t M, int64_t K);
 size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, int64_t total_row_groups);
+// true when the launch cuts K in exactly two chunks: with the output rows cleared beforehand (GemvArgs::y_zeroed) the
+// two partial results add themselves to the output (0 + a + b is a + b in either order) and the summing launch goes
+bool mfma_gemv_two_chunks(int type, int64_t K, int64_t M, int64_t total_row_groups);
 hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStream_t s);
 // expert-grouped form (args.order / args.offsets); K / 256 must not exceed 16 (mfma_grouped_fits)
 bool mfma_grouped_fits(int type, int64_t K);

@@ -331,6 +331,35 @@ def test_small_m_rows_equal_the_m1_result(ctx, orc, qtype):
         assert np.array_equal(got, (single if m <= decode_rows else full)[:m]), m
 
 
+@pytest.mark.parametrize("qtype,k,n,ms", [(Q6_K, 14336, 4096, (3, 4, 8, 16, 24)), (Q4_K, 14336, 4096, (5, 8, 21)),
+                                            (Q8_0, 14336, 2048, (5, 8)), (Q6_K, 14336, 1056, (7,))])
+def test_two_k_chunks_add_themselves_like_the_summing_launch(ctx, qtype, k, n, ms):
+    """Small batches of long rows: the matrix-core kernel cuts K in chunks.  With exactly two chunks (the 8B down
+    projection at 3..8 rows) the quantizer launch of qproj_mul_mat clears the output rows and both chunks add their
+    partial results to them; activations quantized beforehand (qproj_mul_mat_quantized) keep the partial results in
+    scratch and the launch that sums them in chunk order.  0 + a + b = a + b in either order, so the two routes must
+    agree bit for bit - whatever the output buffer held before, and on a second call into the same buffer."""
+    from magnitude_amd import ACT_GGML, synth
+    w = ctx.upload_from_device(qtype, k, n, synth.random_weight(qtype, n, k, seed=8100 + n, device="cuda"))
+    g = torch.Generator(device="cuda")
+    g.manual_seed(12)
+    for m in ms:
+        x = torch.randn((m, k), generator=g, device="cuda")
+        out = torch.full((m, n), float("nan"), device="cuda")
+        ctx.mul_mat(w, x, ACT_GGML, out=out)
+        first = out.clone()
+        ctx.mul_mat(w, x, ACT_GGML, out=out)
+        ref = ctx.mul_mat_quantized([w], ctx.quantize_activations_raw(x, ACT_GGML, qtype), ACT_GGML, m,
+                                    [torch.full((m, n), float("nan"), device="cuda")])[0]
+        assert torch.isfinite(ref).all()
+        assert torch.equal(first, ref), m
+        assert torch.equal(out, ref), m
+        want = (ctx.dequantize(w).double() @ x.double().T).T
+        rel = ((ref.double() - want).norm() / want.norm()).item()
+        assert rel < 2e-2, (m, rel)   # int8 activations against the fp64 product of the dequantized weights
+    w.free()
+
+
 def test_mul_mat_multi_equals_separate_calls(ctx, orc):
     from magnitude_amd import ACT_GGML
     k = 4096
