@@ -3,7 +3,8 @@
 //
 // Every pair has its own expert matrix and, for the down projection, its own activation row, so the launch is
 // a set of independent short GEMVs: a workgroup of 16 waves serves a run of weight rows for a GROUP of pairs
-// (one pair; or the n_used pairs of one token when their results are combined here).  It quantizes the
+// (one pair; the n_used pairs of one token when their results are combined here; or, with more pairs than the
+// compute units have workgroups for, a few consecutive pairs that read the same activation row).  It quantizes the
 // group's activation rows into LDS with the arithmetic of the standalone quantizer, and its waves then walk
 // (row step, pair) units.  Expert rows are short (K = 768 .. 4096), so a step covers S = 64 / (4 K/256) whole
 // rows at once: lane = (row slot, super-block, quarter of the super-block), the row slots' partial dot products
@@ -33,6 +34,7 @@ struct MoeDecodeArgs {
     float *y;                // [n_pairs][N]; with routing weights [n_pairs / group][N]
     const float *cw;         // routing weights [n_pairs], or null
     int group;               // pairs a workgroup serves
+    int x_shared;            // the pairs of a group all read ONE activation row (group divides x_div): staged once
     int wgs_per_group;       // workgroups that share the rows of a group
     int rows_per_wg;         // a multiple of the rows a step covers
 };
@@ -68,6 +70,7 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
     const int vlane = live ? lane - slot * lpr : 0;   // idle lanes repeat a valid address and add nothing
     const int grp = (int)blockIdx.x / g.wgs_per_group, j = (int)blockIdx.x - grp * g.wgs_per_group;
     const int p0 = grp * g.group, G = g.group;
+    const int GS = g.x_shared ? 1 : G;   // activation rows staged
     const int r0 = j * g.rows_per_wg;
     const int r1 = min(N, r0 + g.rows_per_wg);
     const int steps = r1 > r0 ? (r1 - r0 + S * R - 1) / (S * R) : 0;   // units a pair has here
@@ -76,10 +79,10 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
 
     // LDS: the group's quantized activation rows, then the results to combine
     int8_t *sq = reinterpret_cast<int8_t *>(smem);
-    const int d_bytes = (G * nb * 4 + 15) & ~15;   // the block sums behind it are read eight bytes at a time
-    float *sd = reinterpret_cast<float *>(smem + G * K);
-    int16_t *sb = reinterpret_cast<int16_t *>(smem + G * K + d_bytes);
-    float *res = reinterpret_cast<float *>(smem + G * K + d_bytes + G * (K / 16) * 2);
+    const int d_bytes = (GS * nb * 4 + 15) & ~15;   // the block sums behind it are read eight bytes at a time
+    float *sd = reinterpret_cast<float *>(smem + GS * K);
+    int16_t *sb = reinterpret_cast<int16_t *>(smem + GS * K + d_bytes);
+    float *res = reinterpret_cast<float *>(smem + GS * K + d_bytes + GS * (K / 16) * 2);
     float *cwl = res + G * g.rows_per_wg;
     XTile xt;
     xt.qs = sq;
@@ -88,7 +91,7 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
     xt.kt = K;
 
     // the wave's first piece of the activation rows is requested ahead of its first weights (loads return in order)
-    const int n_chunks = G * nb;
+    const int n_chunks = GS * nb;
     constexpr int kAhead = 2;
     float4 x_first[kAhead];
 #pragma unroll
@@ -166,13 +169,13 @@ __global__ __launch_bounds__(kThreads) void moe_decode_kernel(const MoeDecodeArg
         if (u.s != cur_s) {
             cur_s = u.s;
             cur_ok = expert_of(u.s) >= 0;
-            if constexpr (!LONGK) dx.load_x(xt, u.s, 0, vlane);
+            if constexpr (!LONGK) dx.load_x(xt, g.x_shared ? 0 : u.s, 0, vlane);
         }
         float acc[NT];
         if constexpr (LONGK) {
             const int c = i % nch, left = nb - c * 16;          // super-blocks left in the row from this step on
             const bool there = (lane >> 2) < left;
-            dx.load_x(xt, u.s, c * 4096, there ? lane : (lane & 3));   // (lanes past the end read the step's first block)
+            dx.load_x(xt, g.x_shared ? 0 : u.s, c * 4096, there ? lane : (lane & 3));   // (lanes past the end read the step's first block)
 #pragma unroll
             for (int t = 0; t < NT; ++t) {
                 Frag<QT> f;
@@ -292,9 +295,42 @@ bool moe_decode_fits(int type, int64_t K, int64_t n_pairs, int64_t group) {
 hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, const float *combine_weights, int n_used,
                              hipStream_t s) {
     const WeightView &w = args.t[0].w;
-    const int group = combine_weights ? n_used : 1;
-    if (!moe_decode_fits(w.type, w.K, args.n_pairs, group) || !args.x || !args.ids || !args.error_flag || args.x_div < 1 ||
-        n_expert < 1 || w.N < 1 || w.N > (1 << 24) || (swiglu && combine_weights))
+    if (args.n_pairs < 1 || args.x_div < 1 || w.nb < 1) return hipErrorInvalidValue;
+    const int nb = (int)w.nb;
+    const bool long_k = nb > 16;
+    const int S = long_k ? 1 : 64 / (4 * nb);
+    const int64_t steps_total = (w.N + S - 1) / S;
+    // The launch is latency-bound (all loads of the call are in flight at once): the rows are spread over all
+    // compute units, a unit or two a wave, at least half the waves of a workgroup busy.  The registers of a 16-wave
+    // workgroup leave room for one a compute unit, so the grid stays within one round.
+    const auto steps_for = [&](int group) {
+        const int64_t max_wgs = std::max<int64_t>(1, (int64_t)cu_count() / (args.n_pairs / group));
+        return std::max<int64_t>((steps_total + max_wgs - 1) / max_wgs, std::max<int64_t>(1, kWaves / 2 / group));
+    };
+    const auto grid_for = [&](int group) {
+        const int64_t per = steps_for(group) * S;
+        return (int64_t)(args.n_pairs / group) * ((w.N + per - 1) / per);
+    };
+    // Pairs a workgroup serves.  Combined results: the pairs of a token.  Otherwise one - unless that leaves compute
+    // units without a workgroup (more pairs than half the units: 160 pairs were 160 workgroups): then 2, 4, 8 or 16
+    // pairs that read the same activation row (consecutive pairs of a token), staged once, share a set of workgroups,
+    // whichever count fills the round best.
+    int group = combine_weights ? n_used : 1;
+    static const bool no_share = tuning_int("QPROJ_MOE_DECODE_NO_SHARED_ROW", 0) != 0;
+    if (!combine_weights && !no_share && grid_for(1) * 8 < (int64_t)cu_count() * 7) {
+        int64_t best = grid_for(1);
+        for (int c = 2; c <= kMaxGroup; c *= 2) {
+            if (args.n_pairs % c != 0 || args.x_div % c != 0) continue;
+            const int64_t gr = grid_for(c);
+            if (gr <= cu_count() && gr > best) {
+                best = gr;
+                group = c;
+            }
+        }
+    }
+    const bool x_shared = !combine_weights && group > 1;
+    if (!moe_decode_fits(w.type, w.K, args.n_pairs, x_shared ? 1 : group) || args.n_pairs % group != 0 || !args.x || !args.ids ||
+        !args.error_flag || n_expert < 1 || w.N < 1 || w.N > (1 << 24) || (swiglu && combine_weights))
         return hipErrorInvalidValue;
     if (swiglu && (args.n_targets != 2 || args.t[1].w.type != w.type || args.t[1].w.K != w.K || args.t[1].w.N != w.N))
         return hipErrorInvalidValue;
@@ -310,19 +346,12 @@ hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, co
     g.y = args.t[0].y;
     g.cw = combine_weights;
     g.group = group;
-    const int nb = (int)w.nb;
-    const bool long_k = nb > 16;
-    const int S = long_k ? 1 : 64 / (4 * nb);
+    g.x_shared = x_shared ? 1 : 0;
     const int n_groups = args.n_pairs / group;
-    const int64_t steps_total = (w.N + S - 1) / S;
-    // The launch is latency-bound (all loads of the call are in flight at once): the rows are spread over all
-    // compute units, a unit or two a wave, at least half the waves of a workgroup busy.  The registers of a 16-wave
-    // workgroup leave room for one a compute unit, so the grid stays within one round.
-    const int64_t max_wgs = std::max<int64_t>(1, (int64_t)cu_count() / n_groups);
-    int64_t steps_per_wg = std::max<int64_t>((steps_total + max_wgs - 1) / max_wgs, std::max<int64_t>(1, kWaves / 2 / group));
+    int64_t steps_per_wg = steps_for(group);
     // the results a workgroup combines wait in LDS: 48 KB of them at most, less beside long staged rows (more
     // workgroups a group beyond that)
-    const size_t staged = staged_bytes(w.K, group);
+    const size_t staged = staged_bytes(w.K, x_shared ? 1 : group);
     if (combine_weights) {
         const size_t room = std::min<size_t>(48 * 1024, kLdsBudget - staged - 64);
         steps_per_wg = std::min<int64_t>(steps_per_wg, std::max<int64_t>(1, (int64_t)(room / 4 / group / S)));

@@ -552,12 +552,14 @@ def test_moe_ffn_many_experts(ctx, orc, moe, E):
     assert np.median(np.abs(got - want)) <= 1e-6 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("B,E", [(1, 128), (2, 128), (4, 128), (8, 128), (16, 128), (2, 16), (5, 40)])
+@pytest.mark.parametrize("B,E", [(1, 128), (2, 128), (4, 128), (8, 128), (16, 128), (2, 16), (5, 40),
+                                 (11, 128), (12, 128), (20, 128), (24, 128)])
 def test_moe_ffn_few_tokens_take_an_expert_per_pair(ctx, orc, moe, B, E):
-    """Decode-sized batches (at most 128 pairs and no more pairs than experts, or up to 16 pairs): the route that
-    needs no grouping pass - a set of workgroups per pair reads ids[p] itself, quantizes the pair's activation row,
-    and the down projection adds a token's pairs with their routing weights in slot order.  One unit a wave at one
-    token, several pipelined units a wave at eight."""
+    """Decode-sized batches (no more pairs than experts, half as many again for small experts, 192 at most; or up
+    to 16 pairs): the route that needs no grouping pass - a set of workgroups per pair reads ids[p] itself,
+    quantizes the pair's activation row, and the down projection adds a token's pairs with their routing weights
+    in slot order.  One unit a wave at one token, several pipelined units a wave at eight; from 11 tokens on a
+    set of gate / up workgroups serves the eight pairs of a token, whose activation row it stages once."""
     from magnitude_amd import ACT_GGML
     d_model, d_ff, top = moe["d_model"], moe["d_ff"], 8
     rng = np.random.default_rng(700 + 10 * B + E)
@@ -674,6 +676,25 @@ def test_mul_mat_id_expert_per_pair_ragged_rows(ctx, orc, qtype, k, n):
         ctx.mul_mat_id(w, dev(x), dev(bad), ACT_GGML)
     got = ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML).cpu().numpy()
     close(got, orc.mul_mat_id(qtype, blocks, k, n, E, x, ids), 2e-5)
+    w.free()
+
+
+@pytest.mark.parametrize("qtype,k,n", [(Q4_K, 2048, 768), (Q6_K, 768, 300), (Q4_K, 8192, 40)])
+def test_mul_mat_id_pairs_of_a_token_share_a_staged_row(ctx, orc, qtype, k, n):
+    """MUL_MAT_ID alone with more pairs than half the compute units have workgroups for: the pairs of a token share
+    a set of workgroups that stages the token's activation row once (rows = 1), while with a row per slot every
+    pair keeps its own set."""
+    from magnitude_amd import ACT_GGML
+    E, top, B = 128, 8, 11
+    rng = np.random.default_rng(k + n + 5)
+    blocks = encode(qtype, (rng.standard_normal((E * n, k)) * 0.05).astype(np.float32)).reshape(E, n, -1)
+    w = ctx.upload(qtype, k, n, blocks, n_expert=E)
+    ids, _ = routing(rng, B, top, E)
+    ids[3, :4] = ids[2, :4]
+    for rows in (1, top):
+        x = rng.standard_normal((B, rows, k)).astype(np.float32)
+        got = ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML).cpu().numpy()
+        close(got, orc.mul_mat_id(qtype, blocks, k, n, E, x, ids), 2e-5)
     w.free()
 
 
