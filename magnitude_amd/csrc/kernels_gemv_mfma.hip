@@ -937,7 +937,7 @@ constexpr int kMaxSb16 = 16;   // super-blocks of 16 staged rows that fit LDS be
 // 21.8; 13824 -> 5120 at 8 rows 37.7 -> 27.5 with 4 K parts x 3 chunks = 240 workgroups instead of 8 x 2 = 320.)
 Split plan(int64_t K, int64_t M, int64_t total_rg, int W, int min_wgs = 200, bool dense = false, int cus = 256) {
     const int nb = (int)(K / 256);
-    const int max_sb = M <= 8 ? 2 * kMaxSb16 : kMaxSb16;
+    const int max_sb = M <= 8 ? 2 * kMaxSb16 : M <= 16 ? kMaxSb16 : kMaxSb16 / 2;
     int nc = (nb + max_sb - 1) / max_sb;
     const int nc_forced = dense ? nc : 1;
     Split p;
@@ -962,18 +962,34 @@ hipError_t launch_w(const MfmaArgs &g, int W, hipStream_t s) {
     return launch_one<QT, NI, 8, MODE>(g, s);
 }
 
+// ni: activation rows a pass in eights -- 1, 2, or (dense launches of eight waves only) 4: all 32 token rows of the
+// matrix instruction carry a row of their own, at the same number of matrix instructions
 template <int MODE>
-hipError_t launch_typed(const MfmaArgs &g, int type, bool small, int W, hipStream_t s) {
+hipError_t launch_typed(const MfmaArgs &g, int type, int ni, int W, hipStream_t s) {
+    if (ni == 4) {
+        if constexpr (MODE == kDense) {
+            if (W != 8) return hipErrorInvalidValue;
+            if (type == kTypeQ4_K) return launch_one<kTypeQ4_K, 4, 8, kDense>(g, s);
+            if (type == kTypeQ6_K) return launch_one<kTypeQ6_K, 4, 8, kDense>(g, s);
+            return launch_one<kTypeQ8_0, 4, 8, kDense>(g, s);
+        } else {
+            return hipErrorInvalidValue;
+        }
+    }
+    const bool small = ni == 1;
     if (type == kTypeQ4_K) return small ? launch_w<kTypeQ4_K, 1, MODE>(g, W, s) : launch_w<kTypeQ4_K, 2, MODE>(g, W, s);
     if (type == kTypeQ6_K) return small ? launch_w<kTypeQ6_K, 1, MODE>(g, W, s) : launch_w<kTypeQ6_K, 2, MODE>(g, W, s);
     return small ? launch_w<kTypeQ8_0, 1, MODE>(g, W, s) : launch_w<kTypeQ8_0, 2, MODE>(g, W, s);
 }
 
+// waves a workgroup of a dense launch: the 32-row instances exist for eight waves only
+int dense_waves(int type, int64_t M) { return M > 16 ? 8 : waves_per_wg(type); }
+
 }  // namespace
 
 bool mfma_gemv_fits(int type, int64_t M, int64_t K) {
     (void)type;
-    return M >= 1 && M <= 16 && K % 256 == 0;
+    return M >= 1 && M <= 32 && K % 256 == 0;
 }
 
 bool mfma_grouped_fits(int type, int64_t K) {
@@ -982,13 +998,13 @@ bool mfma_grouped_fits(int type, int64_t K) {
 }
 
 size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, int64_t total_rg) {
-    const Split p = plan(K, M, total_rg, waves_per_wg(type), 200, true, cu_count());
+    const Split p = plan(K, M, total_rg, dense_waves(type, M), 200, true, cu_count());
     return p.n_chunks > 1 ? (size_t)p.n_chunks * (size_t)M * (size_t)sum_n * 4 : 0;
 }
 
 bool mfma_gemv_two_chunks(int type, int64_t K, int64_t M, int64_t total_rg) {
     static const bool off = tuning_int("QPROJ_NO_CHUNK_ADD", 0) != 0;
-    return !off && plan(K, M, total_rg, waves_per_wg(type), 200, true, cu_count()).n_chunks == 2;
+    return !off && plan(K, M, total_rg, dense_waves(type, M), 200, true, cu_count()).n_chunks == 2;
 }
 
 hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStream_t s) {
@@ -1000,7 +1016,8 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStr
     g.x_div = 1;
     int64_t total_rg = 0;
     for (int i = 0; i < args.n_targets; ++i) total_rg += (args.t[i].w.N + 31) / 32;
-    const int W = waves_per_wg(args.t[0].w.type);
+    if (args.M < 1 || args.M > 32) return hipErrorInvalidValue;
+    const int W = dense_waves(args.t[0].w.type, args.M);
     const Split p = plan(args.a.K, args.M, total_rg, W, 200, true, cu_count());
     g.n_chunks = p.n_chunks;
     g.chunk_sb = p.chunk_sb;
@@ -1023,7 +1040,7 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStr
     g.n_wgs = wg;
     // the per-chunk results of all targets lie one behind the other in the scratch: refuse what would not fit
     if (g.n_chunks > 1 && !g.add_out && (!scratch.p || part_off * sizeof(float) > scratch.bytes)) return hipErrorInvalidValue;
-    return launch_typed<kDense>(g, args.t[0].w.type, args.M <= 8, W, s);
+    return launch_typed<kDense>(g, args.t[0].w.type, args.M <= 8 ? 1 : args.M <= 16 ? 2 : 4, W, s);
 }
 
 // Expert-grouped form: args.order / args.offsets list each expert's pairs; `swiglu` takes tensors 0 and 1
@@ -1083,8 +1100,8 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
     g.n_pairs = args.n_pairs;
     g.error_flag = args.error_flag;
     g.n_wgs = (int)((args.ids ? n_pairs : std::min<int64_t>(w.E, n_pairs)) * g.wgs_per_expert);
-    if (swiglu) return launch_typed<kGroupedSwiglu>(g, type, small, W, s);
-    return launch_typed<kGrouped>(g, type, small, W, s);
+    if (swiglu) return launch_typed<kGroupedSwiglu>(g, type, small ? 1 : 2, W, s);
+    return launch_typed<kGrouped>(g, type, small ? 1 : 2, W, s);
 }
 
 }  // namespace qproj

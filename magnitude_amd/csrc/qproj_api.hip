@@ -359,12 +359,22 @@ size_t per32_scratch_max(int n, const qproj_weight *const *w, int64_t M) {   // 
     return need;
 }
 
+// Rows a pass of the small-batch kernel takes: 16, or 32 once there are more than 16 (the matrix instruction has 32
+// token rows either way; more staged rows mean shorter K chunks).  Measured, 16-row passes or tiles -> 32-row
+// passes, us: Q4_K 4096 -> 14336 at 17 / 32 rows 27.0 / 27.8 (tiled) -> 20.8 / 22.0, 4096 x 4096 17.4 / 18.1 -> 15.8 / 16.3,
+// 14336 -> 4096 34.7 / 34.4 -> 25.4 / 26.0; Q8_0 4096 x 4096 26.1 / 30.2 -> 17.8 / 19.4, at 63 rows 55.8 -> 32.5.  Q6_K stays
+// with 16 rows: its 32-row instance runs out of registers (540 bytes a lane spilled: 44 -> 98 us at 17 rows).
+int64_t small_batch_pass(int type, int64_t M) {
+    static const int rows = tuning_int("QPROJ_MFMA_PASS_ROWS", 32) > 16 ? 32 : 16;
+    return M > 16 && type != kTypeQ6_K ? rows : 16;
+}
+
 // Which batches take the tiled matrix-core products (weights reused across a tile of tokens, K cut into stretches
 // where the grid would leave the chip idle) instead of passes of the 16-row small-batch kernel.  ONE predicate for
 // the dispatch and for the scratch sizing: the partial tiles of a K cut into stretches go to scratch that only this
 // rule provides.  Q8_0 from 64 rows on with K a multiple of 128; Q4_K and Q6_K from the row counts below.
 int tiled_min_m(int type) {
-    static const int q4 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q4K", 17));
+    static const int q4 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q4K", 33));
     static const int q6 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q6K", 32));
     return type == kTypeQ4_K ? q4 : type == kTypeQ6_K ? q6 : 64;
 }
@@ -388,8 +398,9 @@ size_t dense_scratch_bytes(int n, const qproj_weight *const *w, int64_t M) {
         sum_n += w[i]->N;
         rgs += (w[i]->N + 31) / 32;
     }
-    size_t need = mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, std::min<int64_t>(M, 16), sum_n, rgs);
-    if (M > 16 && M % 16) need = std::max(need, mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, M % 16, sum_n, rgs));
+    const int64_t pass = small_batch_pass(w[0]->type, M);
+    size_t need = mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, std::min<int64_t>(M, pass), sum_n, rgs);
+    if (M > pass && M % pass) need = std::max(need, mfma_gemv_scratch_bytes(w[0]->type, w[0]->K, M % pass, sum_n, rgs));
     return need;
 }
 
@@ -409,8 +420,9 @@ bool dense_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *co
     if (takes_tiled(w[0], M) || !use_mfma_kernel(w[0]->type, M, w[0]->K)) return false;
     int64_t rgs = 0;
     for (int i = 0; i < n; ++i) rgs += (w[i]->N + 31) / 32;
-    bool any = mfma_gemv_two_chunks(w[0]->type, w[0]->K, std::min<int64_t>(M, 16), rgs);
-    if (M > 16 && M % 16) any = any || mfma_gemv_two_chunks(w[0]->type, w[0]->K, M % 16, rgs);
+    const int64_t pass = small_batch_pass(w[0]->type, M);
+    bool any = mfma_gemv_two_chunks(w[0]->type, w[0]->K, std::min<int64_t>(M, pass), rgs);
+    if (M > pass && M % pass) any = any || mfma_gemv_two_chunks(w[0]->type, w[0]->K, M % pass, rgs);
     if (!any) return false;
     z.count = n;
     for (int i = 0; i < n; ++i) {
@@ -426,8 +438,8 @@ bool dense_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *co
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
                     float *const *y, const Scratch &sc, const float *x_f32 = nullptr, bool y_zeroed = false) {
     // Beyond the rows one pass of the small-batch kernel takes: the tiled product, weights reused across a tile of
-    // tokens, K cut into stretches where the grid would leave the chip idle.  (Measured, 8B shapes: Q4_K 17..47
-    // rows 19-72 us in steps of 16 against 15-31 us tiled; Q6_K pays from 32 rows on.)
+    // tokens, K cut into stretches where the grid would leave the chip idle.  (Measured, 8B shapes: Q4_K 33..47
+    // rows in passes of the small-batch kernel against 15-31 us tiled; Q6_K pays from 32 rows on.)
     const auto tiled = [&](const qproj_weight *t) { return takes_tiled(t, M); };
     if (tiled(w[0])) {
         if (w[0]->type == kTypeQ4_K && n >= 2 && n <= 3) {   // q/k/v, gate/up: one launch where the tiles allow it
@@ -445,8 +457,9 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
         return QPROJ_OK;
     }
     if (use_mfma_kernel(w[0]->type, M, w[0]->K)) {
-        for (int64_t m0 = 0; m0 < M; m0 += 16) {
-            const int64_t mc = std::min<int64_t>(16, M - m0);
+        const int64_t pass = small_batch_pass(w[0]->type, M);
+        for (int64_t m0 = 0; m0 < M; m0 += pass) {
+            const int64_t mc = std::min<int64_t>(pass, M - m0);
             GemvArgs g{};
             g.n_targets = n;
             for (int i = 0; i < n; ++i) {
