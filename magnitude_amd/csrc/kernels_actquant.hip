@@ -117,7 +117,9 @@ __global__ __launch_bounds__(kRowThreads) void quant_rows_minterm_kernel(const f
                                                                          int8_t *__restrict__ qs, float *__restrict__ d,
                                                                          int16_t *__restrict__ bsums,
                                                                          int32_t *__restrict__ isum,
-                                                                         uint16_t *__restrict__ msum, float *__restrict__ rs) {
+                                                                         uint16_t *__restrict__ msum, float *__restrict__ rs,
+                                                                         const ZeroJob zero) {
+    zero_rows(zero);
     extern __shared__ __align__(16) float row_lds[];
     __shared__ float wmax[kRowWaves];
     float *ld = row_lds;
@@ -156,7 +158,6 @@ hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, i
     if (kind != kActKindQ8_K && kind != kActKindQ8_0 && kind != kActKindQ8X32) return hipErrorInvalidValue;
     ZeroJob zj{};
     if (zero) {
-        if (msum || kind == kActKindQ8X32) return hipErrorInvalidValue;   // the launches below that carry the job
         zj = *zero;
         for (int i = 0; i < zj.count; ++i)
             if (zj.n[i] % 4 != 0 || (reinterpret_cast<uintptr_t>(zj.p[i]) & 15) != 0) return hipErrorInvalidValue;
@@ -171,9 +172,9 @@ hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, i
         const int nb = (int)(K / 256);
         const dim3 rgrid((unsigned)M), rblock(kRowThreads);
         if (kind == kActKindQ8_K)
-            hipLaunchKernelGGL(quant_rows_minterm_kernel<false>, rgrid, rblock, row_minterm_lds_bytes(false, nb), s, x, u, nb, qs, d, bsums, isum, msum, rs);
+            hipLaunchKernelGGL(quant_rows_minterm_kernel<false>, rgrid, rblock, row_minterm_lds_bytes(false, nb), s, x, u, nb, qs, d, bsums, isum, msum, rs, zj);
         else
-            hipLaunchKernelGGL(quant_rows_minterm_kernel<true>, rgrid, rblock, row_minterm_lds_bytes(true, nb), s, x, u, nb, qs, d, bsums, isum, msum, rs);
+            hipLaunchKernelGGL(quant_rows_minterm_kernel<true>, rgrid, rblock, row_minterm_lds_bytes(true, nb), s, x, u, nb, qs, d, bsums, isum, msum, rs, zj);
         return hipGetLastError();
     }
     const int64_t chunks = (n + 255) / 256;

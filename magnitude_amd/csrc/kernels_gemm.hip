@@ -578,7 +578,10 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const D
     // the rows' factors (normaliser / 16) go through the idle scale buffer: four rows per read, no load per store
     sm.dx[0][tid & 63] = rs_mine * (1.0f / kMinPrescale);
     __syncthreads();
-    float *out = gridDim.y > 1 ? part + (size_t)blockIdx.y * M * N : y;
+    // two stretches and no scratch: the output rows were cleared before the launch and both stretches add their
+    // tile to them (0 + a + b is a + b in either order, so the result does not depend on which arrives first)
+    const bool add = gridDim.y > 1 && part == nullptr;
+    float *out = gridDim.y > 1 && !add ? part + (size_t)blockIdx.y * M * N : y;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -588,7 +591,10 @@ __global__ __launch_bounds__(64 * NW, 2) void gemm_q4k_q8k_direct_kernel(const D
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int64_t m = m0 + j * 32 + 8 * g + 4 * lh + r;
-                if (m < M && n < N) out[m * N + n] = acc[j][4 * g + r] * f[r];
+                if (m < M && n < N) {
+                    if (add) unsafeAtomicAdd(out + m * N + n, acc[j][4 * g + r] * f[r]);
+                    else out[m * N + n] = acc[j][4 * g + r] * f[r];
+                }
             }
         }
     }
@@ -844,7 +850,10 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
     // the rows' factors (normaliser / 16) go through the idle scale buffer: four rows per read, no load per store
     sm.dx[0][tid & 127] = rs_mine * (1.0f / kMinPrescale);
     __syncthreads();
-    float *out = gridDim.y > 1 ? part + (size_t)blockIdx.y * M * N : y;
+    // two stretches and no scratch: the output rows were cleared before the launch and both stretches add their
+    // tile to them (0 + a + b is a + b in either order, so the result does not depend on which arrives first)
+    const bool add = gridDim.y > 1 && part == nullptr;
+    float *out = gridDim.y > 1 && !add ? part + (size_t)blockIdx.y * M * N : y;
 #pragma unroll
     for (int j = 0; j < JT; ++j) {
 #pragma unroll
@@ -854,7 +863,10 @@ __global__ __launch_bounds__(64 * NW, 1) void gemm_q4k_q8k_wide_kernel(const Wei
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int64_t m = m0 + j * 32 + 8 * g + 4 * lh + r;
-                if (m < M && n < N) out[m * N + n] = acc[j][4 * g + r] * f[r];
+                if (m < M && n < N) {
+                    if (add) unsafeAtomicAdd(out + m * N + n, acc[j][4 * g + r] * f[r]);
+                    else out[m * N + n] = acc[j][4 * g + r] * f[r];
+                }
             }
         }
     }
@@ -907,9 +919,18 @@ hipError_t launch_sum_parts(const float *part, int n_split, size_t n, float *y, 
 // compute unit = 512 places): below 384 tiles K is cut in 2, below 192 in 3, never under twelve super-blocks a
 // stretch (K = 4096 cut in two measured slower than whole: the pass that adds the partial tiles costs more
 // than the fuller grid gains).
-int q8k_tile_splits(int64_t K, int64_t M, int64_t N) {
+int q8k_tile_splits(int64_t K, int64_t M, int64_t N, bool add_ok) {
     static const int forced = tuning_int("QPROJ_Q8K_SPLITS", 0);
+    static const bool no_add = tuning_int("QPROJ_NO_TILE_ADD", 0) != 0;
     const int64_t tiles = ((N + 127) / 128) * ((M + 63) / 64);
+    // Two stretches that add themselves to cleared output rows cost no pass over partial tiles: from 96 tiles on that
+    // beats three stretches with the pass, and K = 4096 (eight super-blocks a stretch) is worth cutting while the whole-K
+    // tiles would not give every compute unit a workgroup.  Per call, us: 4096 x 4096 at 192 / 256 tokens 32.7 / 34.2 ->
+    // 26.5 / 28.8 (at 512 tokens, 256 tiles, the cut loses: 39.9 -> 42.8, so it stays whole); 4096 -> 14336 at 64 tokens
+    // 32.0 -> 27.7; 14336 -> 4096 at 192 / 256 tokens 65.3 / 67.6 -> 59.9 / 63.2.
+    if (add_ok && !no_add && forced <= 0 && (M * N) % 4 == 0 && tiles >= 96 && tiles < 384 && K / 256 >= 16 &&
+        (K / 256 >= 24 || tiles < 256))
+        return 2;
     int n = forced > 0 ? forced : tiles >= 384 ? 1 : tiles >= 192 ? 2 : tiles >= 96 ? 3 : 4;
     if ((M * N) % 4 != 0) n = 1;
     // a stretch is at least 12 super-blocks (the pass that adds the partial tiles has to be earned), 4 where the
@@ -919,7 +940,7 @@ int q8k_tile_splits(int64_t K, int64_t M, int64_t N) {
     return n;
 }
 size_t q8k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N) {
-    const int n = q8k_tile_splits(K, M, N);
+    const int n = q8k_tile_splits(K, M, N, false);
     return n > 1 ? (size_t)n * M * N * 4 : 0;
 }
 
@@ -961,7 +982,8 @@ struct Q4Plan {
     bool wide;
     int n_split;
 };
-Q4Plan q4k_plan(int64_t K, int64_t M, int64_t N, bool have_scratch) {
+// add_ok: the output rows hold zeros when the launch starts (Scratch::zeroed)
+Q4Plan q4k_plan(int64_t K, int64_t M, int64_t N, bool have_scratch, bool add_ok = false) {
     static const int wide_env = tuning_int("QPROJ_Q8K_WIDE", -1);
     const int64_t wide_tiles = ((N + 255) / 256) * ((M + 127) / 128);
     if (wide_env >= 0 ? wide_env != 0 : wide_tiles >= 192) return {true, 1};
@@ -969,9 +991,10 @@ Q4Plan q4k_plan(int64_t K, int64_t M, int64_t N, bool have_scratch) {
         const int n = wide_tile_splits(wide_tiles, K / 256, M, N, cu_count(), 4.5);
         if (n > 1) return {true, n};
     }
-    return {false, have_scratch ? q8k_tile_splits(K, M, N) : 1};
+    return {false, have_scratch || add_ok ? q8k_tile_splits(K, M, N, add_ok) : 1};
 }
 }  // namespace
+
 
 size_t q4k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N) {
     const Q4Plan p = q4k_plan(K, M, N, true);
@@ -982,9 +1005,13 @@ size_t q4k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N) {
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s) {
     if (w.type != kTypeQ4_K || a.kind != kActKindQ8_K || !a.msum || !a.rs || M <= 0) return hipErrorInvalidValue;
     if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 128 token rows of K bytes, 32 weight rows of K*144/256
-    const Q4Plan p = q4k_plan(w.K, M, w.N, scratch.p != nullptr);
-    if (p.n_split > 1 && (size_t)p.n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
+    const bool zeroed = (scratch.zeroed & 1u) != 0;
+    Q4Plan p = q4k_plan(w.K, M, w.N, scratch.p != nullptr, zeroed);
+    const bool add = zeroed && p.n_split == 2;   // both stretches add to the cleared rows: no partial tiles
+    if (zeroed && !add) p = q4k_plan(w.K, M, w.N, scratch.p != nullptr);
+    if (p.n_split > 1 && !add && (size_t)p.n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
     if (dry_run()) return hipSuccess;
+    float *const part = add ? nullptr : scratch.p;
     if (p.wide) {   // 128 tokens x 256 weight rows per workgroup, one workgroup per compute unit
         using Smem = WideSmem<8>;
         const auto kern = &gemm_q4k_q8k_wide_kernel<8>;
@@ -992,8 +1019,8 @@ hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, flo
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));
         if (attr != hipSuccess) return attr;
         const int64_t wide_tiles = ((w.N + 255) / 256) * ((M + 127) / 128);
-        hipLaunchKernelGGL(kern, dim3((unsigned)wide_tiles, (unsigned)p.n_split), dim3(512), sizeof(Smem), s, w, a, M, y, scratch.p);
-        if (p.n_split > 1) return launch_sum_parts(scratch.p, p.n_split, (size_t)M * w.N, y, s);
+        hipLaunchKernelGGL(kern, dim3((unsigned)wide_tiles, (unsigned)p.n_split), dim3(512), sizeof(Smem), s, w, a, M, y, part);
+        if (p.n_split > 1 && !add) return launch_sum_parts(scratch.p, p.n_split, (size_t)M * w.N, y, s);
         return hipGetLastError();
     }
     constexpr int NW = 4;   // 64 tokens x 128 weight rows per workgroup, two workgroups per compute unit
@@ -1006,9 +1033,42 @@ hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, flo
     tg.n = 1;
     tg.w[0] = w;
     tg.y[0] = y;
-    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, tg, a, M, scratch.p);
-    if (p.n_split > 1) return launch_sum_parts(scratch.p, p.n_split, (size_t)M * w.N, y, s);
+    hipLaunchKernelGGL(gemm_q4k_q8k_direct_kernel<NW>, grid, dim3(64 * NW), sizeof(Smem), s, tg, a, M, part);
+    if (p.n_split > 1 && !add) return launch_sum_parts(scratch.p, p.n_split, (size_t)M * w.N, y, s);
     return hipGetLastError();
+}
+
+namespace {
+// Which of n matrices over the same activation rows share ONE launch of the 64-token kernel: those that would take it
+// with K in one stretch (or are small enough to be better off together than cut).  The others (128-token tiles, K cut
+// into stretches) get launches of their own.  Fills joined[], returns how many (0 or >= 2).
+int q4k_joined_set(int n, const WeightView *w, int64_t M, bool have_scratch, bool planes_ok, int (&joined)[3]) {
+    static const int wide_env = tuning_int("QPROJ_Q8K_WIDE", -1);
+    static const bool off = tuning_int("QPROJ_Q8K_NO_MULTI", 0) != 0;
+    const bool can = !off && n >= 2 && n <= 3 && wide_env < 0 && planes_ok && M > 0;
+    int n_joined = 0;
+    for (int i = 0; i < n; ++i) {
+        const Q4Plan p = q4k_plan(w[i].K, M, w[i].N, have_scratch);
+        const bool fits = can && w[i].type == kTypeQ4_K && w[i].K == w[0].K && w[i].K <= (1 << 24) && !p.wide &&
+                          (p.n_split == 1 || ((w[i].N + 127) / 128) * ((M + 63) / 64) < 96);   // small ones are better off together than cut
+        if (fits) joined[n_joined++] = i;
+    }
+    return n_joined < 2 ? 0 : n_joined;
+}
+}  // namespace
+
+// bit i: matrix i of a launch_gemm_q8k_multi call gets a launch of its own that cuts K in two stretches which add
+// themselves, if its output rows are cleared beforehand
+uint32_t q4k_multi_adds(int n, const WeightView *w, int64_t M, bool have_scratch) {
+    int joined[3];
+    const int n_joined = n <= 3 ? q4k_joined_set(n, w, M, have_scratch, true, joined) : 0;
+    uint32_t mask = 0;
+    for (int i = 0; i < n; ++i) {
+        bool in = false;
+        for (int j = 0; j < n_joined; ++j) in = in || joined[j] == i;
+        if (!in && w[i].type == kTypeQ4_K && q4k_plan(w[i].K, M, w[i].N, have_scratch, true).n_split == 2) mask |= 1u << i;
+    }
+    return mask;
 }
 
 // The same for n matrices over the same activation rows.  One launch where every matrix would take the
@@ -1016,24 +1076,13 @@ hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, flo
 hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, int64_t M, float *const *y,
                                  const Scratch &scratch, hipStream_t s) {
     constexpr int NW = 4;
-    static const int wide_env = tuning_int("QPROJ_Q8K_WIDE", -1);
-    static const bool off = tuning_int("QPROJ_Q8K_NO_MULTI", 0) != 0;
-    // the matrices that would take the 64-token kernel with K in one stretch go together; the others (128-token
-    // tiles, K cut into stretches) get their own launches first
-    const bool can = !off && n >= 2 && n <= 3 && wide_env < 0 && a.kind == kActKindQ8_K && a.msum && a.rs && M > 0;
-    int joined[3], n_joined = 0;
-    for (int i = 0; i < n; ++i) {
-        const Q4Plan p = q4k_plan(w[i].K, M, w[i].N, scratch.p != nullptr);
-        const bool fits = can && w[i].type == kTypeQ4_K && w[i].K == w[0].K && w[i].K <= (1 << 24) && !p.wide &&
-                          (p.n_split == 1 || ((w[i].N + 127) / 128) * ((M + 63) / 64) < 96);   // small ones are better off together than cut
-        if (fits) joined[n_joined++] = i;
-    }
-    if (n_joined < 2) n_joined = 0;
+    int joined[3];
+    int n_joined = n <= 3 ? q4k_joined_set(n, w, M, scratch.p != nullptr, a.kind == kActKindQ8_K && a.msum && a.rs, joined) : 0;
     for (int i = 0; i < n; ++i) {
         bool in = false;
         for (int j = 0; j < n_joined; ++j) in = in || joined[j] == i;
         if (in) continue;
-        hipError_t e = launch_gemm_q8k(w[i], a, M, y[i], scratch, s);
+        hipError_t e = launch_gemm_q8k(w[i], a, M, y[i], scratch.for_target(i), s);
         if (e != hipSuccess) return e;
     }
     if (n_joined == 0 || dry_run()) return hipSuccess;

@@ -490,7 +490,7 @@ Q6Plan q6k_plan(int64_t K, int64_t M, int64_t N, bool have_scratch) {
         const int n = wide_tile_splits(wide_tiles, K / 256, M, N, cu_count(), 5.0);
         if (n > 1) return {true, n};
     }
-    return {false, have_scratch ? q8k_tile_splits(K, M, N) : 1};
+    return {false, have_scratch ? q8k_tile_splits(K, M, N, false) : 1};
 }
 }  // namespace
 

@@ -433,6 +433,28 @@ bool dense_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *co
     return true;
 }
 
+// The same for the tiled Q4_K kernels: the matrices of the call whose launch cuts K in exactly two stretches get their
+// output rows cleared by the quantizer launch, and the stretches add themselves (no partial tiles, no adding pass).
+// Returns the mask of those matrices and fills `z` with their rows.
+uint32_t tiled_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *const *y, bool have_scratch, ZeroJob &z) {
+    WeightView views[kMaxTargets];
+    for (int i = 0; i < n; ++i) views[i] = w[i]->view;
+    uint32_t mask = q4k_multi_adds(n, views, M, have_scratch);
+    z.count = 0;
+    for (int i = 0; i < n; ++i) {
+        if (!((mask >> i) & 1u)) continue;
+        const int64_t cnt = M * w[i]->N;
+        if (cnt % 4 != 0 || (reinterpret_cast<uintptr_t>(y[i]) & 15) != 0) {
+            mask &= ~(1u << i);
+            continue;
+        }
+        z.p[z.count] = y[i];
+        z.n[z.count] = cnt;
+        ++z.count;
+    }
+    return mask;
+}
+
 // x_f32: non-null when `a` carries no planes and the kernel quantizes these rows itself (small batches only);
 // y_zeroed: the output rows were cleared by the quantizer launch (dense_clears_rows)
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
@@ -450,7 +472,7 @@ int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const A
         }
         for (int i = 0; i < n; ++i) {
             const int t = w[0]->type;
-            QP_HIP(ctx, t == kTypeQ4_K   ? launch_gemm_q8k(w[i]->view, a, M, y[i], sc, ctx->stream)
+            QP_HIP(ctx, t == kTypeQ4_K   ? launch_gemm_q8k(w[i]->view, a, M, y[i], sc.for_target(i), ctx->stream)
                         : t == kTypeQ6_K ? launch_gemm_q6k_q8k(w[i]->view, a, M, y[i], sc, ctx->stream)
                                          : launch_gemm_q8_0(w[i]->view, a, M, y[i], sc, ctx->stream));
         }
@@ -894,6 +916,7 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
         const bool minterm = act == kActQ8X32 || (w[0]->type == kTypeQ4_K && takes_tiled(w[0], M));
         ZeroJob zero{};
         bool y_zeroed = false;
+        uint32_t tile_adds = 0;   // tiled Q4_K: the matrices whose two K stretches add themselves to cleared rows
         if (norm) {   // norm, weights and quantizer in one launch
             if (p.kind == kActKindQ8X32 && K % 256 != 0)
                 return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_rms_norm_mul_mat: the per-32 format needs K % 256 == 0");
@@ -905,11 +928,13 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
                                         minterm ? reinterpret_cast<float *>(ws + p.off_rs) : nullptr, ctx->stream));
         } else {
             y_zeroed = act == kActGGML && !minterm && dense_clears_rows(n, w, M, y_dev, zero);
-            QP_HIP(ctx, run_quantize(ctx, p, ws, x_dev, M, K, minterm, swiglu_u, y_zeroed ? &zero : nullptr));
+            if (act == kActGGML && w[0]->type == kTypeQ4_K && takes_tiled(w[0], M))
+                tile_adds = tiled_clears_rows(n, w, M, y_dev, extra > 0, zero);
+            QP_HIP(ctx, run_quantize(ctx, p, ws, x_dev, M, K, minterm, swiglu_u, y_zeroed || tile_adds ? &zero : nullptr));
         }
         const ActView a = act_view(p, ws, K);
         // the partial results lie behind the activation planes; `extra` is all a launcher may use of it
-        const Scratch sc{extra ? reinterpret_cast<float *>(ws + p.total) : nullptr, extra};
+        const Scratch sc{extra ? reinterpret_cast<float *>(ws + p.total) : nullptr, extra, tile_adds};
         if (act == kActGGML) return run_dense_q8act(ctx, n, w, a, M, y_dev, sc, nullptr, y_zeroed);
         for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], sc, ctx->stream));
         return QPROJ_OK;

@@ -93,6 +93,10 @@ struct GemvArgs {
 struct Scratch {
     float *p;
     size_t bytes;
+    uint32_t zeroed = 0;     // bit i: the output rows of the launcher's i-th tensor were cleared by the launch in front
+                             // (ZeroJob): a K cut in exactly two may add its two partial results straight to them and
+                             // needs neither scratch nor the adding pass
+    Scratch for_target(int i) const { return Scratch{p, bytes, (zeroed >> i) & 1u}; }
 };
 
 // Dry run: every launcher does its argument and capacity checks and returns without touching the device.  The
@@ -150,7 +154,7 @@ struct ZeroJob {
     int64_t n[kMaxTargets];
 };
 // u non-null: the rows quantized are silu(x) * u (the swiglu between gate / up and the down projection);
-// zero (only without the min-term plane, Q8_K and Q8_0 kinds): see ZeroJob
+// zero: see ZeroJob (carried by the first launch of the quantizer)
 hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, int8_t *qs, float *d,
                                int16_t *bsums, uint16_t *msum, int32_t *isum, float *rs, hipStream_t s,
                                const float *u = nullptr, const ZeroJob *zero = nullptr);
@@ -203,10 +207,12 @@ size_t per32_scratch_bytes(int64_t K, int64_t M, int64_t N);
 hipError_t launch_gemm_q8x32(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s);
 // Q4_K weights x ggml Q8_K activations (`a`), large M
 // `scratch`: q8k_tile_scratch_bytes(K, M, N) bytes (null: K is never split)
-int q8k_tile_splits(int64_t K, int64_t M, int64_t N);
+int q8k_tile_splits(int64_t K, int64_t M, int64_t N, bool add_ok);
 size_t q8k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N);
 hipError_t launch_sum_parts(const float *part, int n_split, size_t n, float *y, hipStream_t s);
 size_t q4k_tile_scratch_bytes(int64_t K, int64_t M, int64_t N);   // what launch_gemm_q8k asks of its scratch
+// bit i: with cleared output rows, matrix i of a tiled Q4_K call cuts K in two stretches that add themselves (Scratch::zeroed)
+uint32_t q4k_multi_adds(int n, const WeightView *w, int64_t M, bool have_scratch);
 hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, float *y, const Scratch &scratch, hipStream_t s);
 hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, int64_t M, float *const *y,
                                  const Scratch &scratch, hipStream_t s);

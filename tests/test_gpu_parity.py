@@ -387,6 +387,36 @@ def test_two_k_chunks_add_themselves_like_the_summing_launch(ctx, qtype, k, n, m
     w.free()
 
 
+@pytest.mark.parametrize("m,k,ns", [(192, 4096, (4096,)), (64, 4096, (14336,)), (256, 14336, (4096,)),
+                                     (192, 4096, (4096, 1024, 1024)), (130, 4096, (14336, 14336))])
+def test_two_k_stretches_of_a_tile_add_themselves(ctx, m, k, ns):
+    """Tiled Q4_K products on grids that leave compute units idle cut K into stretches.  Exactly two stretches, in a
+    call that quantizes its own activations, add their partial tiles to output rows that the quantizer launch
+    cleared (no scratch, no adding pass); qproj_mul_mat_quantized keeps partial tiles and the pass.  Same integer
+    sums, another fp32 order across the stretches: equal within a few ulp, the same on every call whatever the
+    output held before, and right against the fp64 product of the dequantized weights."""
+    from magnitude_amd import ACT_GGML, synth
+    ws = [ctx.upload_from_device(Q4_K, k, n, synth.random_weight(Q4_K, n, k, seed=8300 + i, device="cuda"))
+          for i, n in enumerate(ns)]
+    g = torch.Generator(device="cuda")
+    g.manual_seed(m)
+    x = torch.randn((m, k), generator=g, device="cuda")
+    outs = [torch.full((m, n), float("nan"), device="cuda") for n in ns]
+    ctx.mul_mat_multi(ws, x, ACT_GGML, outs=outs)
+    first = [o.clone() for o in outs]
+    ctx.mul_mat_multi(ws, x, ACT_GGML, outs=outs)
+    ref = ctx.mul_mat_quantized(ws, ctx.quantize_activations_raw(x, ACT_GGML, Q4_K), ACT_GGML, m,
+                                [torch.full((m, n), float("nan"), device="cuda") for n in ns])
+    for w, a, b, r in zip(ws, first, outs, ref):
+        assert torch.isfinite(a).all() and torch.equal(a, b)
+        scale = r.abs().max().item()
+        assert (a - r).abs().max().item() <= 2e-6 * scale
+        want = (ctx.dequantize(w).double() @ x.double().T).T
+        rel = ((a.double() - want).norm() / want.norm()).item()
+        assert rel < 2e-2, rel
+        w.free()
+
+
 def test_mul_mat_multi_equals_separate_calls(ctx, orc):
     from magnitude_amd import ACT_GGML
     k = 4096
