@@ -301,10 +301,19 @@ __device__ __forceinline__ void compute(const uint8_t *region, const uint8_t *sm
     } else if constexpr (QT == kTypeQ6_K) {
         using C = Cfg<kTypeQ6_K>;
         int isum[NV];
-#pragma unroll
-        for (int v = 0; v < NV; ++v) isum[v] = 0;
         const uint4 sc = *reinterpret_cast<const uint4 *>(region + C::kSc + n * 16);
         const uint32_t scw[4] = {sc.x, sc.y, sc.z, sc.w};
+        {   // -32 * sum_j sc_j * bsum_j first (block sums split as 64*hi + lo against the 16 scales): the integer sum
+            // starts from it, and the two results are gone before the sixteen products below need their registers
+            const uint8_t *aux = smem + L.off_aux + (ks * MT + mrow) * 32;
+            const uint2 bhi = *reinterpret_cast<const uint2 *>(aux + 8 * h);
+            const uint2 blo = *reinterpret_cast<const uint2 *>(aux + 16 + 8 * h);
+            const long bsc = h ? as_i64(sc.z, sc.w) : as_i64(sc.x, sc.y);
+            const v16i Ch = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64(bhi.x, bhi.y), bsc, z, 0, 0, 0);
+            const v16i Cl = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64(blo.x, blo.y), bsc, z, 0, 0, 0);
+#pragma unroll
+            for (int v = 0; v < NV; ++v) isum[v] = -32 * ((Ch[v] << 6) + Cl[v]);
+        }
 #pragma unroll
         for (int f = 0; f < 2; ++f)
 #pragma unroll
@@ -333,13 +342,6 @@ __device__ __forceinline__ void compute(const uint8_t *region, const uint8_t *sm
                 }
                 __builtin_amdgcn_sched_barrier(0);   // keeps the four groups' operand loads from piling up in registers
             }
-        // -32 * sum_j sc_j * bsum_j: block sums split as 64*hi + lo against the 16 scales
-        const uint8_t *aux = smem + L.off_aux + (ks * MT + mrow) * 32;
-        const uint2 bhi = *reinterpret_cast<const uint2 *>(aux + 8 * h);
-        const uint2 blo = *reinterpret_cast<const uint2 *>(aux + 16 + 8 * h);
-        const long bsc = h ? as_i64(sc.z, sc.w) : as_i64(sc.x, sc.y);
-        const v16i Ch = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64(bhi.x, bhi.y), bsc, z, 0, 0, 0);
-        const v16i Cl = __builtin_amdgcn_mfma_i32_32x32x16_i8(as_i64(blo.x, blo.y), bsc, z, 0, 0, 0);
         const float d = h2f(*reinterpret_cast<const uint32_t *>(region + C::kD + n * 4));
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
@@ -348,8 +350,7 @@ __device__ __forceinline__ void compute(const uint8_t *region, const uint8_t *sm
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int v = 4 * i + j;
-                const int corr = (Ch[v] << 6) + Cl[v];
-                out[v] = fmaf(dxv[j] * d, (float)(isum[v] - 32 * corr), out[v]);
+                out[v] = fmaf(dxv[j] * d, (float)isum[v], out[v]);
             }
         }
     } else {

@@ -362,11 +362,12 @@ size_t per32_scratch_max(int n, const qproj_weight *const *w, int64_t M) {   // 
 // Rows a pass of the small-batch kernel takes: 16, or 32 once there are more than 16 (the matrix instruction has 32
 // token rows either way; more staged rows mean shorter K chunks).  Measured, 16-row passes or tiles -> 32-row
 // passes, us: Q4_K 4096 -> 14336 at 17 / 32 rows 27.0 / 27.8 (tiled) -> 20.8 / 22.0, 4096 x 4096 17.4 / 18.1 -> 15.8 / 16.3,
-// 14336 -> 4096 34.7 / 34.4 -> 25.4 / 26.0; Q8_0 4096 x 4096 26.1 / 30.2 -> 17.8 / 19.4, at 63 rows 55.8 -> 32.5.  Q6_K stays
-// with 16 rows: its 32-row instance runs out of registers (540 bytes a lane spilled: 44 -> 98 us at 17 rows).
+// 14336 -> 4096 34.7 / 34.4 -> 25.4 / 26.0; Q8_0 4096 x 4096 26.1 / 30.2 -> 17.8 / 19.4, at 63 rows 55.8 -> 32.5; Q6_K
+// 14336 -> 4096 at 17 / 31 rows 44.0 / 48.1 -> 32.6 / 33.0, at 32 rows 39.9 (tiled) -> 34.0, 4096 x 4096 25.6 / 28.5 -> 17.7 / 18.1.
 int64_t small_batch_pass(int type, int64_t M) {
     static const int rows = tuning_int("QPROJ_MFMA_PASS_ROWS", 32) > 16 ? 32 : 16;
-    return M > 16 && type != kTypeQ6_K ? rows : 16;
+    (void)type;
+    return M > 16 ? rows : 16;
 }
 
 // Which batches take the tiled matrix-core products (weights reused across a tile of tokens, K cut into stretches
@@ -375,7 +376,7 @@ int64_t small_batch_pass(int type, int64_t M) {
 // rule provides.  Q8_0 from 64 rows on with K a multiple of 128; Q4_K and Q6_K from the row counts below.
 int tiled_min_m(int type) {
     static const int q4 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q4K", 33));
-    static const int q6 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q6K", 32));
+    static const int q6 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q6K", 33));
     return type == kTypeQ4_K ? q4 : type == kTypeQ6_K ? q6 : 64;
 }
 bool takes_tiled(const qproj_weight *t, int64_t M) {
@@ -460,8 +461,8 @@ uint32_t tiled_clears_rows(int n, const qproj_weight *const *w, int64_t M, float
 int run_dense_q8act(qproj_ctx *ctx, int n, const qproj_weight *const *w, const ActView &a, int64_t M,
                     float *const *y, const Scratch &sc, const float *x_f32 = nullptr, bool y_zeroed = false) {
     // Beyond the rows one pass of the small-batch kernel takes: the tiled product, weights reused across a tile of
-    // tokens, K cut into stretches where the grid would leave the chip idle.  (Measured, 8B shapes: Q4_K 33..47
-    // rows in passes of the small-batch kernel against 15-31 us tiled; Q6_K pays from 32 rows on.)
+    // tokens, K cut into stretches where the grid would leave the chip idle.  (Measured, 8B shapes, 33 rows: Q6_K
+    // 14336 -> 4096 50.9 us in two passes of the small-batch kernel against 41 us tiled, Q4_K 4096 -> 14336 42 against 29.)
     const auto tiled = [&](const qproj_weight *t) { return takes_tiled(t, M); };
     if (tiled(w[0])) {
         if (w[0]->type == kTypeQ4_K && n >= 2 && n <= 3) {   // q/k/v, gate/up: one launch where the tiles allow it
