@@ -1083,14 +1083,16 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
     // several microseconds.  A wave can take two row groups in a row (one stream of items) and pay the prologue
     // once; measured on the 128-expert FFN (K = 768 down, K = 2048 gate / up): worth it for grids beyond three
     // workgroups per compute unit (down at 8 and 64 tokens: 62.3 -> 58.8 and 115.5 -> 111.3 us), harmful for small
-    // grids (one token: 21.1 -> 22.9 us; gate / up at 64 tokens, 744 workgroups: 111.3 -> 128 us), and four in a
-    // row always lose.
+    // grids (one token: 21.1 -> 22.9 us; gate / up at 64 tokens, 744 workgroups: 111.3 -> 128 us).  Four in a row
+    // lost everywhere at first; with the shorter prologue they pay for the down projection where an expert has more
+    // than four pairs (16 staged rows a pass), Q4_K experts: 118.0 -> 111.4 us a call at 96 tokens, 121.8 -> 117.3 at
+    // 128, 169.0 -> 159.8 at 256 (Q6_K down experts, which keep the loop per row group there: 180.5 -> 184.9, so two).
     static const int forced_all = tuning_int("QPROJ_MOE_RG_LOOP", 0), forced_down = tuning_int("QPROJ_MOE_RG_LOOP_DOWN", 0);
     const int forced_loop = !swiglu && forced_down > 0 ? forced_down : forced_all;
     {
         const int64_t wgs1 = (args.ids ? n_pairs : std::min<int64_t>(w.E, n_pairs)) * ((rg_e + g.rw - 1) / g.rw);
         const int64_t cus = 256;
-        int loop = forced_loop > 0 ? forced_loop : wgs1 > 3 * cus ? 2 : 1;
+        int loop = forced_loop > 0 ? forced_loop : wgs1 > 3 * cus ? (!small && !swiglu && type == kTypeQ4_K ? 4 : 2) : 1;
         loop = (int)std::min<int64_t>(loop, std::max<int64_t>(1, rg_e / g.rw));
         while (loop > 1 && rg_e % ((int64_t)g.rw * loop) != 0) --loop;   // no half-empty last workgroup
         g.rg_loop = std::min(loop, 8);
