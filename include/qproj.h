@@ -20,7 +20,9 @@
  *   - weight bytes are handed over on the HOST in GGUF block layout, verbatim, and the
  *     library owns their device copy (ggml buffer set_tensor);
  *   - activations, ids and outputs are DEVICE pointers owned by the caller (ggml tensors
- *     living in backend buffers); all work is enqueued on the context's HIP stream;
+ *     living in backend buffers); all work is enqueued on the context's HIP stream.  Outputs
+ *     are ordinary device memory (hipMalloc; not host-coherent or managed allocations): some
+ *     launches add their partial results to them with the memory side's float adder;
  *   - a context is used by one thread at a time (the reference serialises native calls on one
  *     executor thread: /root/reference/design/inference/engine.md:49-50).
  *   - row-major, ggml element order: x is [M][K], y is [M][N], W is N rows of K weights.
