@@ -890,8 +890,10 @@ def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):
     for bit on every replay - with other eager work and synchronizations of the same context in between,
     and with new activation values written into the same buffers.  Covered: the decode kernel (M = 1),
     quantizer + small-batch kernel with K cut into chunks and the chunk sum (M = 8, Q6_K, K = 14336), the
-    tiled kernels with partial tiles added afterwards (M = 200, K = 14336), the MoE FFN with its grouping pass."""
-    from magnitude_amd import Context, ACT_GGML, ACT_Q8X32
+    tiled kernels with partial tiles added afterwards (M = 200, K = 14336), the MoE FFN with its grouping pass, and
+    the launches whose two K parts add themselves to output rows the quantizer clears (M = 8 on the 14336 -> 4096
+    Q6_K matrix, M = 192 on 4096 x 4096 Q4_K): the outputs hold NaN before every replay."""
+    from magnitude_amd import Context, ACT_GGML, ACT_Q8X32, synth
     stream = torch.cuda.Stream()
     c = Context(0, stream=stream.cuda_stream)
     try:
@@ -900,6 +902,8 @@ def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):
         k6, n6 = 14336, 128
         w6 = c.upload(Q6_K, k6, n6, make_weight(orc, Q6_K, n6, k6, seed=1500 + k6 + n6))
         w4l = c.upload(Q4_K, k6, n6, make_weight(orc, Q4_K, n6, k6, seed=1500 + k6 + n6))
+        w6big = c.upload_from_device(Q6_K, k6, 4096, synth.random_weight(Q6_K, 4096, k6, seed=31, device="cuda"))
+        w4sq = c.upload_from_device(Q4_K, k, 4096, synth.random_weight(Q4_K, 4096, k, seed=32, device="cuda"))
         E, d_model, d_ff, top, B = moe["E"], moe["d_model"], moe["d_ff"], 8, 8
         g = c.upload(Q4_K, d_model, d_ff, moe["gate"], n_expert=E)
         u = c.upload(Q4_K, d_model, d_ff, moe["up"], n_expert=E)
@@ -908,10 +912,12 @@ def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):
         ids, wts = routing(rng, B, top, E)
         ids_d, wts_d = dev(ids), dev(wts)
         xs = {"dec": torch.empty((1, k), device="cuda"), "small": torch.empty((8, k6), device="cuda"),
-              "tiled": torch.empty((200, k6), device="cuda"), "moe": torch.empty((B, d_model), device="cuda")}
+              "tiled": torch.empty((200, k6), device="cuda"), "moe": torch.empty((B, d_model), device="cuda"),
+              "mid": torch.empty((192, k), device="cuda")}
         ys = {"dec": torch.empty((1, n), device="cuda"), "small": torch.empty((8, n6), device="cuda"),
               "tiled6": torch.empty((200, n6), device="cuda"), "tiled4": torch.empty((200, n6), device="cuda"),
-              "per32": torch.empty((200, n6), device="cuda"), "moe": torch.empty((B, d_model), device="cuda")}
+              "per32": torch.empty((200, n6), device="cuda"), "moe": torch.empty((B, d_model), device="cuda"),
+              "small_add": torch.empty((8, 4096), device="cuda"), "tiled_add": torch.empty((192, 4096), device="cuda")}
 
         def fill(seed):
             gen = torch.Generator(device="cuda").manual_seed(seed)
@@ -926,6 +932,8 @@ def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):
             c.mul_mat(w4l, xs["tiled"], ACT_GGML, out=ys["tiled4"], sync=False)
             c.mul_mat(w4l, xs["tiled"], ACT_Q8X32, out=ys["per32"], sync=False)
             c.moe_ffn(g, u, d, xs["moe"], ids_d, wts_d, ACT_GGML, out=ys["moe"], sync=False)
+            c.mul_mat(w6big, xs["small"], ACT_GGML, out=ys["small_add"], sync=False)
+            c.mul_mat(w4sq, xs["mid"], ACT_GGML, out=ys["tiled_add"], sync=False)
 
         def eager(seed):
             fill(seed)
@@ -941,7 +949,7 @@ def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):
         for seed in (3, 4, 5):
             want = eager(seed)                     # eager work of the same context between the replays
             for t in ys.values():
-                t.zero_()
+                t.fill_(float("nan"))
             torch.cuda.synchronize()
             graph.replay()
             torch.cuda.synchronize()
