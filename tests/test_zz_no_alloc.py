@@ -36,6 +36,8 @@ CASES = [  # (type, K, rows of the tensors sharing the call, [M of the first cal
     (Q6_K, 14336, (512,), [130, 40]),            # tiled Q6_K kernel with stretches
     (Q8_0, 4096, (768,), [96, 64, 7]),           # tiled Q8_0 product, then the small-batch kernel
     (Q4_K, 4096, (1024, 256, 256), [64, 20]),    # q/k/v style launch of three tensors
+    (Q6_K, 14336, (4096,), [8, 4]),              # two K chunks that add themselves to rows the quantizer cleared
+    (Q4_K, 4096, (4096,), [192, 32, 17]),        # two K stretches of a tile that add themselves, then 32-row passes
 ]
 
 
