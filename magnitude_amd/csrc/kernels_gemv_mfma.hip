@@ -452,7 +452,7 @@ struct StagedRows {
     int dst[kPieces];
     float dval;
     static __device__ __forceinline__ bool fits(int n_rows, int nsb) {
-        return QT != kTypeQ8_0 /* (its instances have no registers to spare) */ && n_rows * nsb * 16 <= kPieces * kThreads &&
+        return QT != kTypeQ8_0 && MT <= 16 /* (those instances have no registers to spare) */ && n_rows * nsb * 16 <= kPieces * kThreads &&
                n_rows * nsb * Cfg<QT>::kDx <= kThreads;
     }
     __device__ __forceinline__ void request(const MfmaArgs &g, const uint8_t *smem, const Layout &L, int c0, int nsb, int n_rows) {
@@ -898,6 +898,8 @@ hipError_t launch_one(const MfmaArgs &g, hipStream_t s) {
         static const bool no_flat = tuning_int("QPROJ_MOE_NO_FLAT", 0) != 0;
         if (g.kw == 1 && !no_flat) return launch_one<QT, NI, W, MODE, true>(g, s);
     }
+    // K parts of a row group are summed through the waves' regions: a wave's partial tile must fit its region
+    if (g.kw > 1 && (MODE == kGroupedSwiglu ? 2 : 1) * (8 * NI) * 32 * 4 > Cfg<QT>::kRegion) return hipErrorInvalidValue;
     if (dry_run()) return hipSuccess;
     const Layout L = layout<QT, 8 * NI, W>(g.chunk_sb);
     auto kern = gemv_mfma_kernel<QT, NI, W, MODE, FLAT>;
@@ -974,7 +976,9 @@ hipError_t launch_typed(const MfmaArgs &g, int type, int ni, int W, hipStream_t 
             if (type == kTypeQ6_K) return launch_one<kTypeQ6_K, 4, 8, kDense>(g, s);
             return launch_one<kTypeQ8_0, 4, 8, kDense>(g, s);
         } else {
-            return hipErrorInvalidValue;
+            // expert-grouped: Q4_K experts with K of at most eight super-blocks (the staged rows of 32 pairs)
+            if (W != 8 || type != kTypeQ4_K) return hipErrorInvalidValue;
+            return launch_one<kTypeQ4_K, 4, 8, MODE>(g, s);
         }
     }
     const bool small = ni == 1;
@@ -1062,10 +1066,16 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
     // row map, staged rows: a chain of dependent loads) hides behind the other's weight stream.  Measured on the
     // 128-expert FFN against eight waves: 23.2 -> 21.1 us at one token, 121.9 -> 115.5 us at 64.
     static const int moe_waves = tuning_int("QPROJ_MOE_WAVES", 4);
-    const int W = type == kTypeQ4_K && (moe_waves == 4 || moe_waves == 8) ? moe_waves : waves_per_wg(type);
     const int64_t rg_e = (w.N + 31) / 32;
     const bool small = n_pairs <= 4 * w.E;   // few pairs an expert: 8 staged rows a pass are enough
-    Split p = plan(w.K, small ? 8 : 16, std::min<int64_t>(w.E, n_pairs) * rg_e, W);
+    // more than 16 pairs an expert (prompt-sized batches): 32 staged rows a pass halve the passes over an expert's
+    // weights (Q4_K experts whose K fits LDS beside 32 rows; eight waves, one workgroup a compute unit)
+    static const bool no_wide_pass = tuning_int("QPROJ_MOE_NO_32_ROW_PASS", 0) != 0;
+    bool wide_pass = !no_wide_pass && !args.ids && type == kTypeQ4_K && w.K / 256 <= kMaxSb16 / 2 && n_pairs > 16 * w.E;
+    // (only with K in one part a wave: the partial tiles of K parts, 32 rows x 32 x two tensors, would not fit a wave's region)
+    if (wide_pass && plan(w.K, 32, std::min<int64_t>(w.E, n_pairs) * rg_e, 8).kw != 1) wide_pass = false;
+    const int W = wide_pass ? 8 : type == kTypeQ4_K && (moe_waves == 4 || moe_waves == 8) ? moe_waves : waves_per_wg(type);
+    Split p = plan(w.K, small ? 8 : wide_pass ? 32 : 16, std::min<int64_t>(w.E, n_pairs) * rg_e, W);
     const int nb = (int)(w.K / 256);
     if (p.n_chunks != 1) {   // the grouped form keeps K inside one workgroup
         p.n_chunks = 1;
@@ -1103,8 +1113,9 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
     g.n_pairs = args.n_pairs;
     g.error_flag = args.error_flag;
     g.n_wgs = (int)((args.ids ? n_pairs : std::min<int64_t>(w.E, n_pairs)) * g.wgs_per_expert);
-    if (swiglu) return launch_typed<kGroupedSwiglu>(g, type, small ? 1 : 2, W, s);
-    return launch_typed<kGrouped>(g, type, small ? 1 : 2, W, s);
+    const int ni = small ? 1 : wide_pass ? 4 : 2;
+    if (swiglu) return launch_typed<kGroupedSwiglu>(g, type, ni, W, s);
+    return launch_typed<kGrouped>(g, type, ni, W, s);
 }
 
 }  // namespace qproj

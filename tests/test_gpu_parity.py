@@ -583,14 +583,14 @@ def test_moe_ffn_matches_oracle(ctx, orc, moe, B):
         close(gsep, gid, 2e-5)   # decode kernel vs grouped matrix-core kernel: same integer dots, other fp32 order
 
 
-@pytest.mark.parametrize("E", [72, 128])
-def test_moe_ffn_many_experts(ctx, orc, moe, E):
+@pytest.mark.parametrize("E,B", [(72, 64), (128, 64), (72, 160)])
+def test_moe_ffn_many_experts(ctx, orc, moe, E, B):
     """The FFN at the expert counts of the 128-expert configuration, where the grouped launches take their
-    many-workgroup shapes (8 staged rows a pass at E = 128, 16 at E = 72) and the quantizer of x rides in the
-    grouping launch."""
+    many-workgroup shapes (8 staged rows a pass at E = 128, 16 at E = 72; 32 with more than 16 pairs an expert,
+    a prompt-sized batch: E = 72, 160 tokens) and the quantizer of x rides in the grouping launch."""
     from magnitude_amd import ACT_GGML
-    d_model, d_ff, top, B = moe["d_model"], moe["d_ff"], 8, 64
-    rng = np.random.default_rng(300 + E)
+    d_model, d_ff, top = moe["d_model"], moe["d_ff"], 8
+    rng = np.random.default_rng(300 + E + B)
     pick = rng.integers(0, moe["E"], size=E)          # the fixture's 16 experts, repeated
     gate_b, up_b, down_b = (np.ascontiguousarray(moe[k][pick]) for k in ("gate", "up", "down"))
     ids, wts = routing(rng, B, top, E)
