@@ -184,6 +184,7 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
         return;
     }
     const int n_blocks = (n_pairs + 63) / 64;
+    const int id_bits = n_expert > 1 ? 32 - __builtin_clz((unsigned)(n_expert - 1)) : 0;
     int vid[kBlocksPerWave], rank[kBlocksPerWave];
     bool bad = false;
 #pragma unroll
@@ -201,14 +202,20 @@ __global__ __launch_bounds__(kGroupThreads) void moe_group_kernel(const int32_t 
         const int blk = wave + 16 * i;
         if (blk < n_blocks) {   // wave-uniform
             const int v = vid[i];
-            int r = 0, size = 0;
-            for (int j = 0; j < 64; ++j) {
-                const int ej = __builtin_amdgcn_readlane(v, j);
-                const unsigned long long m = __ballot(v == ej);
-                const int below = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
-                r = lane == j ? below : r;
-                size = lane == j ? __popcll(m) : size;
+            // the lanes of the block that hold the same expert: one ballot per bit of the id (and one for "names an
+            // expert at all") instead of one per lane
+            unsigned long long m = ~0ull;
+            {
+                const unsigned long long b = __ballot(v >= 0);
+                m &= v >= 0 ? b : ~b;
             }
+            for (int bit = 0; bit < id_bits; ++bit) {
+                const bool set = (v >> bit) & 1;
+                const unsigned long long b = __ballot(set);
+                m &= set ? b : ~b;
+            }
+            const int r = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0));
+            const int size = __popcll(m);
             rank[i] = r;
             if (r == 0 && v >= 0) tab[blk * n_expert + v] = size;
         }
