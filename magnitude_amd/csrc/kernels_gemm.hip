@@ -916,7 +916,7 @@ hipError_t launch_sum_parts(const float *part, int n_split, size_t n, float *y, 
 }
 
 // K stretches for the kernels that take ggml-format activations (64-token x 128-row tiles, two workgroups per
-// compute unit = 512 places): below 384 tiles K is cut in 2, below 192 in 3, never under twelve super-blocks a
+// compute unit = 512 places): below 384 tiles K is cut in 2, below 192 in 3, below 96 in 4, below 64 in 8, never under twelve super-blocks a
 // stretch (K = 4096 cut in two measured slower than whole: the pass that adds the partial tiles costs more
 // than the fuller grid gains).
 int q8k_tile_splits(int64_t K, int64_t M, int64_t N, bool add_ok) {
@@ -931,7 +931,11 @@ int q8k_tile_splits(int64_t K, int64_t M, int64_t N, bool add_ok) {
     if (add_ok && !no_add && forced <= 0 && (M * N) % 4 == 0 && tiles >= 96 && tiles < 384 && K / 256 >= 16 &&
         (K / 256 >= 24 || tiles < 256))
         return 2;
-    int n = forced > 0 ? forced : tiles >= 384 ? 1 : tiles >= 192 ? 2 : tiles >= 96 ? 3 : 4;
+    // (under 64 tiles - a down projection of 4096 rows at up to 64 tokens is 32 - eight stretches: 14336 -> 4096 at
+    // 33 / 64 tokens, four -> eight stretches, Q6_K 42.0 / 43.5 -> 29.7 / 31.1 us, Q4_K 35.6 / 37.4 -> 27.9 / 29.7; ten to
+    // fourteen were slower again, the pass over the partial tiles grows; 64 tiles keep four: seven 47.2 -> 46.1 for Q6_K
+    // and 40.5 -> 42.8 for Q4_K)
+    int n = forced > 0 ? forced : tiles >= 384 ? 1 : tiles >= 192 ? 2 : tiles >= 96 ? 3 : tiles >= 64 ? 4 : 8;
     if ((M * N) % 4 != 0) n = 1;
     // a stretch is at least 12 super-blocks (the pass that adds the partial tiles has to be earned), 4 where the
     // grid is under a fifth of the workgroups the chip holds and a workgroup's K loop is pure latency
