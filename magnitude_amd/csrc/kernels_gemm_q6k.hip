@@ -483,14 +483,31 @@ struct Q6Plan {
     bool wide;
     int n_split;
 };
+// Stretches of K for the 64-token tiles (128 rows, two workgroups a compute unit = 512 places).  This kernel's
+// workgroups are slow next to the pass that adds the partial tiles, so under 192 tiles it takes as many stretches as
+// fill the places once, eight at most, four super-blocks a stretch at least.  14336 -> 4096, per call, us, stretches of
+// the common rule -> these: 128 tokens (64 tiles) 4 -> 8: 49.0 -> 46.7; 160 / 192 tokens (96 tiles) 3 -> 5: 79.7 / 79.4 ->
+// 60.4 / 59.4; 256 tokens (128 tiles) 3 -> 4: 81.4 -> 72.4.
+int q6k_tile_splits(int64_t K, int64_t M, int64_t N) {
+    static const int forced = tuning_int("QPROJ_Q8K_SPLITS", 0);
+    const int64_t tiles = ((N + 127) / 128) * ((M + 63) / 64);
+    if (forced > 0 || tiles >= 192 || (M * N) % 4 != 0) return q8k_tile_splits(K, M, N, false);
+    int n = (int)std::min<int64_t>(8, std::max<int64_t>(1, 512 / tiles));
+    while (n > 1 && K / 256 < 4 * n) --n;
+    return n;
+}
+
 Q6Plan q6k_plan(int64_t K, int64_t M, int64_t N, bool have_scratch) {
     const int64_t wide_tiles = ((N + 255) / 256) * ((M + 127) / 128);
-    if (wide_tiles >= 192) return {true, 1};
+    // (from 160 tiles: 4096 -> 14336 at 320 / 384 tokens, 168 tiles, 98.5 / 98.0 -> 87.2 / 85.3 us; from 112 on it loses,
+    // 8192 x 8192 at 448 tokens 101 -> 147)
+    static const int wide_min = tuning_int("QPROJ_Q6K_WIDE_MIN_TILES", 160);
+    if (wide_tiles >= wide_min) return {true, 1};
     if (have_scratch && (M * N) % 4 == 0 && wide_tiles >= 48) {
         const int n = wide_tile_splits(wide_tiles, K / 256, M, N, cu_count(), 5.0);
         if (n > 1) return {true, n};
     }
-    return {false, have_scratch ? q8k_tile_splits(K, M, N, false) : 1};
+    return {false, have_scratch ? q6k_tile_splits(K, M, N) : 1};
 }
 }  // namespace
 
@@ -516,7 +533,10 @@ hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M,
         if (p.n_split > 1) return launch_sum_parts(scratch.p, p.n_split, (size_t)M * w.N, y, s);
         return hipGetLastError();
     }
-    if (p.n_split > 1 || ((w.N + 127) / 128) * ((M + 63) / 64) >= 384) return launch_q6k<4, 2>(w, a, M, y, scratch.p, p.n_split, s);
+    // 64-token tiles from 192 tiles on (32-token tiles below, twice the workgroups): 4096 -> 14336 at 160 / 192 tokens,
+    // 336 tiles, 74.2 / 76.8 -> 66.1 / 64.3 us; 4096 x 4096 at 384 tokens 49.4 -> 42.9 (the threshold was 384)
+    static const int tile64_min = tuning_int("QPROJ_Q6K_TILE64_MIN", 192);
+    if (p.n_split > 1 || ((w.N + 127) / 128) * ((M + 63) / 64) >= tile64_min) return launch_q6k<4, 2>(w, a, M, y, scratch.p, p.n_split, s);
     return launch_q6k<4, 1>(w, a, M, y, nullptr, 1, s);
 }
 
