@@ -380,7 +380,10 @@ int tiled_min_m(int type) {
     return type == kTypeQ4_K ? q4 : type == kTypeQ6_K ? q6 : 64;
 }
 bool takes_tiled(const qproj_weight *t, int64_t M) {
-    if (M < tiled_min_m(t->type)) return false;
+    // (Q6_K rows beyond 16384 weights: a 32-row pass of the small-batch kernel would stage K in more than eight chunks
+    // and add as many partial results - 28672 -> 8192 at 17 / 32 rows: 85.5 / 89.5 us in a pass, 72.9 / 77.7 tiled)
+    const bool long_q6 = t->type == kTypeQ6_K && t->K > 16384 && M > 16;
+    if (M < tiled_min_m(t->type) && !long_q6) return false;
     return t->type != kTypeQ8_0 || t->K % 128 == 0;
 }
 
