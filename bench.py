@@ -628,7 +628,7 @@ def main():
                 f"({res[-1]['GBps']:.0f} GB/s from HBM); one draw replayed: {ms1 * 1e3:.1f} us ({res[-1]['cache_resident']['GBps']:.0f} GB/s, "
                 f"{byts1 / 1e6:.0f} MB, may sit in the Infinity Cache)")
         out["moe"] = {"experts": E, "top": top, "d_model": dm, "d_ff": dff, "batches": res,
-                      "note": "2 launches per call up to 192 pairs (gate/up+SwiGLU, down+combine: an expert read per pair, rows "
+                      "note": "2 launches per call up to 256 pairs (gate/up+SwiGLU, down+combine: an expert read per pair, rows "
                               "quantized in the prologue), else 5 (group+quantize, gate/up+SwiGLU, quantize, down, combine); "
                               "the rotation over three weight sets and several id draws is replayed as one "
                               "HIP graph; GBps counts the distinct experts of each call"}

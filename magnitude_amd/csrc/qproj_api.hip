@@ -550,12 +550,14 @@ bool grouped_pair_mode(int type, int64_t K, int64_t n_pairs, int64_t E) {
 // at one token, 24.9 -> 18.8 at two, 41.0 -> 23.2 at four, 57.6 -> 36.2 at eight, 74.1 -> 58.9 at sixteen, 86.0 -> 73.7 at
 // twenty, 91.2 -> 84.2 at twenty-four, worse from 28 tokens on (97.6 against 92.8 us; 32: 101 against 95): with more pairs
 // than experts the repeated reads of an expert come to outweigh the launches saved.  So: as many pairs as experts
-// whatever the expert's size, half as many again while an expert matrix is small (two million weights at most).
+// whatever the expert's size, half as many again while an expert matrix is small (two million weights at most), 256 pairs at most.
 // (Up to 16 pairs take it whatever the expert count while an expert matrix is small: launches weigh more than bytes
 // there.  Large experts do not: 8 experts of 4096 x 14336, 16 pairs: 214 us grouped, 220 us this way.)
 bool moe_decode_route(int type, int64_t K, int64_t N, int64_t n_pairs, int64_t group, int64_t E) {
     static const bool on = tuning_int("QPROJ_NO_MOE_DECODE", 0) == 0;
-    static const int max_pairs = tuning_int("QPROJ_MOE_DECODE_MAX_PAIRS", 192);
+    // (one workgroup set a pair fills the chip at 256 pairs; 256 experts, top-8, 2048 x 512: 28 / 32 tokens 95.2 / 97.4 us
+    // grouped, 77.2 / 79.1 this way; 40 tokens, 320 pairs, 103.6 against 109.8)
+    static const int max_pairs = tuning_int("QPROJ_MOE_DECODE_MAX_PAIRS", 256);
     static const int per_4_experts = tuning_int("QPROJ_MOE_DECODE_PAIRS_PER_4_EXPERTS", 4);
     const bool small_expert = K * N <= ((int64_t)2 << 20);
     const bool few = n_pairs <= 16 && small_expert;

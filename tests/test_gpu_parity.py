@@ -609,9 +609,9 @@ def test_moe_ffn_many_experts(ctx, orc, moe, E, B):
 
 
 @pytest.mark.parametrize("B,E", [(1, 128), (2, 128), (4, 128), (8, 128), (16, 128), (2, 16), (5, 40),
-                                 (11, 128), (12, 128), (20, 128), (24, 128)])
+                                 (11, 128), (12, 128), (20, 128), (24, 128), (32, 256)])
 def test_moe_ffn_few_tokens_take_an_expert_per_pair(ctx, orc, moe, B, E):
-    """Decode-sized batches (no more pairs than experts, half as many again for small experts, 192 at most; or up
+    """Decode-sized batches (no more pairs than experts, half as many again for small experts, 256 at most; or up
     to 16 pairs): the route that needs no grouping pass - a set of workgroups per pair reads ids[p] itself,
     quantizes the pair's activation row, and the down projection adds a token's pairs with their routing weights
     in slot order.  One unit a wave at one token, several pipelined units a wave at eight; from 11 tokens on a
