@@ -57,6 +57,7 @@ struct MfmaArgs {
     const float *x;        // non-null: fp32 activation rows [rows][K], quantized by every workgroup in its prologue
     int M, n_chunks, chunk_sb, kw, rw, n_wgs;
     int add_out;           // dense mode, two chunks, output rows cleared before the launch: both chunks add to y
+    int64_t part_plane;    // expert-grouped mode with K in chunks: floats of one chunk's results, [n_pairs][N], in t[0].part
     // expert-grouped mode (MUL_MAT_ID): activation rows of expert e are the pairs order[offsets[e]..offsets[e+1])
     const int32_t *order;
     const int32_t *offsets;
@@ -596,8 +597,10 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
     float *y = g.t[0].y, *part = g.t[0].part;
     int c = 0, rs, expert = 0, pair0 = 0, n_rows = g.M;
     if constexpr (GROUPED) {
-        const int slot = (int)blockIdx.x / g.wgs_per_expert;   // the grid covers min(E, pairs) experts
-        rs = (int)blockIdx.x - slot * g.wgs_per_expert;
+        const int slotc = (int)blockIdx.x / g.wgs_per_expert;   // the grid covers min(E, pairs) experts x K chunks
+        rs = (int)blockIdx.x - slotc * g.wgs_per_expert;
+        const int slot = slotc / g.n_chunks;
+        c = slotc - slot * g.n_chunks;
         if (g.ids) {   // a workgroup set per pair
             if (slot >= g.n_pairs) return;
             expert = g.ids[slot];
@@ -637,6 +640,8 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
     const int N = (int)w.N;
     const int nb = (int)(g.a.K >> 8);
     const int c0 = c * g.chunk_sb, nsb = min(g.chunk_sb, nb - c0);
+    if constexpr (GROUPED)   // K in chunks: the chunk's results go to its plane of the scratch, a pass adds the planes
+        if (g.n_chunks > 1) y = part + (size_t)c * g.part_plane;
 
     // wave -> (row group, K part)
     const int rgl = wave / g.kw, kp = wave - rgl * g.kw;
@@ -912,7 +917,7 @@ hipError_t launch_one(const MfmaArgs &g, hipStream_t s) {
     }
     hipLaunchKernelGGL(kern, dim3((unsigned)g.n_wgs), dim3(W * 64), (size_t)L.total, s, g);
     hipError_t e = hipGetLastError();
-    if (e != hipSuccess || g.n_chunks == 1 || g.add_out) return e;
+    if (e != hipSuccess || g.n_chunks == 1 || g.add_out || MODE != kDense) return e;
     size_t n_out = 0;
     for (int i = 0; i < g.n_targets; ++i) n_out = std::max(n_out, (size_t)g.M * (size_t)g.t[i].w.N);
     const unsigned blocks = (unsigned)std::min<size_t>(256, (n_out + 255) / 256);
@@ -1002,6 +1007,23 @@ bool mfma_grouped_fits(int type, int64_t K) {
     return K % 256 == 0 && K / 256 <= kMaxSb16;
 }
 
+// Expert-grouped launches of rows longer than the staged rows of a pass allow (K / 256 > 32 with 8 rows a pass, > 16
+// with 16): K goes in chunks, one set of workgroups a chunk, each chunk's results to its own plane [n_pairs][N] of
+// the scratch, added up in chunk order by a pass afterwards.  Not for the gate / up launch with its SwiGLU epilogue.
+int mfma_grouped_chunks(int64_t K, int64_t n_pairs, int64_t E) {
+    const int nb = (int)(K / 256);
+    const int max_sb = n_pairs <= 4 * E ? 2 * kMaxSb16 : kMaxSb16;
+    return (nb + max_sb - 1) / max_sb;
+}
+bool mfma_grouped_chunked_fits(int type, int64_t K, int64_t N, int64_t n_pairs) {
+    (void)type;
+    return K % 256 == 0 && K / 256 > kMaxSb16 && (n_pairs * N) % 4 == 0;
+}
+size_t mfma_grouped_scratch_bytes(int64_t K, int64_t N, int64_t n_pairs, int64_t E) {
+    const int nc = mfma_grouped_chunks(K, n_pairs, E);
+    return nc > 1 ? (size_t)nc * (size_t)n_pairs * (size_t)N * 4 : 0;
+}
+
 size_t mfma_gemv_scratch_bytes(int type, int64_t K, int64_t M, int64_t sum_n, int64_t total_rg) {
     const Split p = plan(K, M, total_rg, dense_waves(type, M), 200, true, cu_count());
     return p.n_chunks > 1 ? (size_t)p.n_chunks * (size_t)M * (size_t)sum_n * 4 : 0;
@@ -1050,7 +1072,7 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStr
 
 // Expert-grouped form: args.order / args.offsets list each expert's pairs; `swiglu` takes tensors 0 and 1
 // as gate and up.  n_pairs only steers the launch shape (how many experts can be busy at once).
-hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool swiglu, hipStream_t s) {
+hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool swiglu, hipStream_t s, const Scratch &scratch) {
     MfmaArgs g{};
     g.n_targets = swiglu ? 2 : 1;
     g.a = args.a;
@@ -1077,17 +1099,28 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
     const int W = wide_pass ? 8 : type == kTypeQ4_K && (moe_waves == 4 || moe_waves == 8) ? moe_waves : waves_per_wg(type);
     Split p = plan(w.K, small ? 8 : wide_pass ? 32 : 16, std::min<int64_t>(w.E, n_pairs) * rg_e, W);
     const int nb = (int)(w.K / 256);
-    if (p.n_chunks != 1) {   // the grouped form keeps K inside one workgroup
+    // K stays inside one workgroup unless the staged rows of a pass do not fit: then the chunks LDS forces, no more
+    const int nc = wide_pass ? 1 : mfma_grouped_chunks(w.K, n_pairs, w.E);
+    if (nc > 1) {
+        if (swiglu || args.ids || !scratch.p || (size_t)nc * (size_t)n_pairs * (size_t)w.N * 4 > scratch.bytes ||
+            (n_pairs * w.N) % 4 != 0)
+            return hipErrorInvalidValue;
+        p.chunk_sb = (nb + nc - 1) / nc;
+        p.n_chunks = (nb + p.chunk_sb - 1) / p.chunk_sb;
+        while (p.kw > 1 && p.kw * 2 > p.chunk_sb) p.kw /= 2;   // K parts of a chunk, not of the row
+    } else {
         p.n_chunks = 1;
         p.chunk_sb = nb;
     }
-    g.n_chunks = 1;
+    g.n_chunks = p.n_chunks;
     g.chunk_sb = p.chunk_sb;
+    g.part_plane = n_pairs * w.N;
     g.kw = p.kw;
     g.rw = W / p.kw;
     for (int i = 0; i < g.n_targets; ++i) {
         g.t[i].w = args.t[i].w;
         g.t[i].y = args.t[i].y;
+        g.t[i].part = g.n_chunks > 1 ? scratch.p : nullptr;
     }
     // Short K makes a row group a few steps of work against a prologue (row map, staged rows, barriers) of
     // several microseconds.  A wave can take two row groups in a row (one stream of items) and pay the prologue
@@ -1112,10 +1145,12 @@ hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool 
     g.ids = args.ids;
     g.n_pairs = args.n_pairs;
     g.error_flag = args.error_flag;
-    g.n_wgs = (int)((args.ids ? n_pairs : std::min<int64_t>(w.E, n_pairs)) * g.wgs_per_expert);
+    g.n_wgs = (int)((args.ids ? n_pairs : std::min<int64_t>(w.E, n_pairs)) * g.n_chunks * g.wgs_per_expert);
     const int ni = small ? 1 : wide_pass ? 4 : 2;
     if (swiglu) return launch_typed<kGroupedSwiglu>(g, type, ni, W, s);
-    return launch_typed<kGrouped>(g, type, ni, W, s);
+    hipError_t e = launch_typed<kGrouped>(g, type, ni, W, s);
+    if (e != hipSuccess || g.n_chunks == 1 || dry_run()) return e;
+    return launch_sum_parts(scratch.p, g.n_chunks, (size_t)n_pairs * (size_t)w.N, args.t[0].y, s);
 }
 
 }  // namespace qproj

@@ -565,6 +565,18 @@ bool moe_decode_route(int type, int64_t K, int64_t N, int64_t n_pairs, int64_t g
     return on && (few || (n_pairs <= max_pairs && 4 * n_pairs <= per4 * E)) && moe_decode_fits(type, K, n_pairs, group);
 }
 
+// Expert rows too long for the staged rows of the grouped matrix-core kernel (K > 4096): from `min_mt` pairs an expert
+// on (the rows a pass of the plain grouped kernel would take) that kernel walks K in chunks and a pass adds the chunks'
+// results; below, the plain grouped kernel on the vector ALU.  8 experts, top-2, 4096 x 14336 (the down projection is
+// the long one), per call, plain kernel -> chunks: 219 -> 189 us at 8 tokens, 270 -> 184 at 16, 409 -> 254 at 32,
+// 1231 -> 352 at 64.
+int grouped_mt(int64_t n_pairs, int64_t E);
+bool grouped_long_rows(const qproj_weight *w, int64_t n_pairs) {
+    static const int min_mt = tuning_int("QPROJ_GROUPED_LONG_MIN_MT", 2);
+    return min_mt > 0 && !use_mfma_grouped(w->type, w->K) && grouped_mt(n_pairs, w->E) >= min_mt &&
+           mfma_grouped_chunked_fits(w->type, w->K, w->N, n_pairs);
+}
+
 int grouped_mt(int64_t n_pairs, int64_t E) {
     if (n_pairs * 4 <= E) return 1;
     if (n_pairs <= E) return 2;
@@ -1182,7 +1194,10 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     const size_t off_order = p.total;
     const size_t off_offsets = off_order + align_up((size_t)n_pairs * 4);
     const size_t off_active = off_offsets + align_up((size_t)(w->E + 1) * 4);
-    const size_t total = off_active + align_up(active_list_bytes(w->E));
+    const size_t off_parts = off_active + align_up(active_list_bytes(w->E));
+    const bool long_rows = grouped_long_rows(w, n_pairs);
+    const size_t parts_bytes = long_rows ? mfma_grouped_scratch_bytes(K, w->N, n_pairs, w->E) : 0;
+    const size_t total = off_parts + align_up(parts_bytes);
     int rc = ensure_ws(ctx, total);
     if (rc) return rc;
     // few pairs an expert: the grouped kernel quantizes the rows it needs in its prologue
@@ -1215,6 +1230,9 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     g.x_div = nb1 == 1 ? (int)n_used : 1;
     if (use_mfma_grouped(w->type, K))
         QP_HIP(ctx, launch_gemv_mfma_grouped(g, n_pairs, false, ctx->stream));
+    else if (long_rows)
+        QP_HIP(ctx, launch_gemv_mfma_grouped(g, n_pairs, false, ctx->stream,
+                                             Scratch{reinterpret_cast<float *>(ctx->ws + off_parts), parts_bytes}));
     else
         QP_HIP(ctx, launch_gemv_q8act(g, grouped_mt(n_pairs, w->E), (int)w->E, ctx->stream));
     return QPROJ_OK;
@@ -1251,6 +1269,10 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     off += ph.total;
     const size_t off_e = off;
     off += align_up((size_t)(n_pairs * d_model) * 4);
+    const bool long_down = grouped_long_rows(down, n_pairs);
+    const size_t parts_bytes = long_down ? mfma_grouped_scratch_bytes(d_ff, d_model, n_pairs, E) : 0;
+    const size_t off_parts = off;
+    off += align_up(parts_bytes);
     int rc = ensure_ws(ctx, off);
     if (rc) return rc;
     uint8_t *ws = ctx->ws;
@@ -1337,6 +1359,9 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     gd.x_div = 1;
     if (use_mfma_grouped(down->type, d_ff))
         QP_HIP(ctx, launch_gemv_mfma_grouped(gd, n_pairs, false, ctx->stream));
+    else if (long_down)
+        QP_HIP(ctx, launch_gemv_mfma_grouped(gd, n_pairs, false, ctx->stream,
+                                             Scratch{reinterpret_cast<float *>(ws + off_parts), parts_bytes}));
     else
         QP_HIP(ctx, launch_gemv_q8act(gd, mt, (int)E, ctx->stream));
     QP_HIP(ctx, launch_moe_combine(e, weights_dev, B, n_used, d_model, y_dev, ctx->stream));

@@ -176,7 +176,12 @@ bool mfma_gemv_two_chunks(int type, int64_t K, int64_t M, int64_t total_row_grou
 hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStream_t s);
 // expert-grouped form (args.order / args.offsets); K / 256 must not exceed 16 (mfma_grouped_fits)
 bool mfma_grouped_fits(int type, int64_t K);
-hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool swiglu, hipStream_t s);
+// longer rows, not for the SwiGLU launch: K in chunks whose results go to `scratch` (mfma_grouped_scratch_bytes) and are
+// added by a pass afterwards; n_pairs * N must be a multiple of 4
+bool mfma_grouped_chunked_fits(int type, int64_t K, int64_t N, int64_t n_pairs);
+size_t mfma_grouped_scratch_bytes(int64_t K, int64_t N, int64_t n_pairs, int64_t E);
+hipError_t launch_gemv_mfma_grouped(const GemvArgs &args, int64_t n_pairs, bool swiglu, hipStream_t s,
+                                    const Scratch &scratch = Scratch{nullptr, 0});
 hipError_t launch_gemv_f32(const GemvArgs &args, int mt, int n_experts_grid, hipStream_t s);
 // h[i] = silu(g[i]) * u[i], the expression of ggml's swiglu on floats
 hipError_t launch_swiglu(const float *g, const float *u, size_t n, float *h, hipStream_t s);

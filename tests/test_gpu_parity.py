@@ -754,6 +754,48 @@ def test_mul_mat_id_pairs_of_a_token_share_a_staged_row(ctx, orc, qtype, k, n):
     w.free()
 
 
+@pytest.mark.parametrize("qtype,k,n", [(Q4_K, 8448, 200), (Q6_K, 14336, 96), (Q8_0, 5120, 130)])
+def test_mul_mat_id_long_expert_rows_go_in_chunks(ctx, orc, qtype, k, n):
+    """Experts with rows of more than 4096 weights (a Mixtral-class down projection) and several pairs an expert:
+    the grouped matrix-core kernel stages K in chunks - one set of workgroups a chunk, a pass adds the chunks'
+    results in order - instead of leaving the call to the vector-ALU kernel.  8 and 16 staged rows a pass, a
+    ragged last chunk, one activation row per token and one per slot."""
+    from magnitude_amd import ACT_GGML
+    E, top = 6, 2
+    rng = np.random.default_rng(k + n)
+    blocks = encode(qtype, (rng.standard_normal((E * n, k)) * 0.05).astype(np.float32)).reshape(E, n, -1)
+    w = ctx.upload(qtype, k, n, blocks, n_expert=E)
+    for B in (8, 24, 60):
+        ids, _ = routing(rng, B, top, E)
+        for rows in (1, top):
+            x = rng.standard_normal((B, rows, k)).astype(np.float32)
+            got = ctx.mul_mat_id(w, dev(x), dev(ids), ACT_GGML).cpu().numpy()
+            close(got, orc.mul_mat_id(qtype, blocks, k, n, E, x, ids), 2e-5)
+    w.free()
+
+
+def test_moe_ffn_long_down_rows_go_in_chunks(ctx, orc):
+    """The FFN with an intermediate row of 8192: gate / up keep K = d_model inside a workgroup, the down projection
+    walks its K in chunks."""
+    from magnitude_amd import ACT_GGML
+    E, top, B, d_model, d_ff = 4, 2, 24, 512, 8192
+    rng = np.random.default_rng(91)
+    enc = lambda t, rows, cols: encode(t, (rng.standard_normal((E * rows, cols)) * 0.03).astype(np.float32)).reshape(E, rows, -1)
+    gate_b, up_b, down_b = enc(Q4_K, d_ff, d_model), enc(Q4_K, d_ff, d_model), enc(Q6_K, d_model, d_ff)
+    ids, wts = routing(rng, B, top, E)
+    x = rng.standard_normal((B, d_model)).astype(np.float32)
+    g = ctx.upload(Q4_K, d_model, d_ff, gate_b, n_expert=E)
+    u = ctx.upload(Q4_K, d_model, d_ff, up_b, n_expert=E)
+    d = ctx.upload(Q6_K, d_ff, d_model, down_b, n_expert=E)
+    got = ctx.moe_ffn(g, u, d, dev(x), dev(ids), dev(wts), ACT_GGML).cpu().numpy()
+    want = orc.moe_ffn(Q4_K, Q6_K, gate_b, up_b, down_b, d_model, d_ff, E, x, ids, wts, orc.ACT_GGML)
+    close(got, want, 1e-3)
+    gate(got, want)
+    assert np.median(np.abs(got - want)) <= 2e-6 * np.abs(want).max()
+    for t in (g, u, d):
+        t.free()
+
+
 # ---------------------------------------------------------------- RMS norm in front of the projections
 
 @pytest.mark.parametrize("m,k", [(1, 4096), (5, 14336), (3, 20480), (7, 288), (64, 4096)])
