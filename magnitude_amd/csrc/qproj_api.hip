@@ -1269,10 +1269,15 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     off += ph.total;
     const size_t off_e = off;
     off += align_up((size_t)(n_pairs * d_model) * 4);
-    const bool long_down = grouped_long_rows(down, n_pairs);
-    const size_t parts_bytes = long_down ? mfma_grouped_scratch_bytes(d_ff, d_model, n_pairs, E) : 0;
+    // rows too long for one pass of the grouped matrix-core kernel go in K chunks (grouped_long_rows); gate and up then
+    // take a launch each (the SwiGLU epilogue needs whole sums) and the swiglu is formed by the quantizer behind them
+    const bool long_down = grouped_long_rows(down, n_pairs), long_gate = grouped_long_rows(gate, n_pairs);
+    const size_t parts_bytes = std::max(long_down ? mfma_grouped_scratch_bytes(d_ff, d_model, n_pairs, E) : 0,
+                                        long_gate ? mfma_grouped_scratch_bytes(d_model, d_ff, n_pairs, E) : 0);
     const size_t off_parts = off;
     off += align_up(parts_bytes);
+    const size_t off_h2 = off;
+    if (long_gate) off += align_up((size_t)(n_pairs * d_ff) * 4);
     int rc = ensure_ws(ctx, off);
     if (rc) return rc;
     uint8_t *ws = ctx->ws;
@@ -1337,11 +1342,28 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     g.offsets = offsets;
     g.active = active;
     g.x_div = (int)n_used;
-    if (use_mfma_grouped(gate->type, d_model))
+    const float *swiglu_u = nullptr;   // non-null: h holds the gate products, this the up products
+    if (use_mfma_grouped(gate->type, d_model)) {
         QP_HIP(ctx, launch_gemv_mfma_grouped(g, n_pairs, true, ctx->stream));
-    else
+    } else if (long_gate) {
+        float *h2 = reinterpret_cast<float *>(ws + off_h2);
+        const Scratch parts{reinterpret_cast<float *>(ws + off_parts), parts_bytes};
+        GemvArgs gu = g;
+        g.n_targets = 1;
+        gu.n_targets = 1;
+        gu.t[0].w = up->view;
+        gu.t[0].y = h2;
+        QP_HIP(ctx, launch_gemv_mfma_grouped(g, n_pairs, false, ctx->stream, parts));
+        QP_HIP(ctx, launch_gemv_mfma_grouped(gu, n_pairs, false, ctx->stream, parts));
+        swiglu_u = h2;
+        if (fuse_h) {   // the down launch quantizes fp32 rows itself: they must be the swiglu by then
+            QP_HIP(ctx, launch_swiglu(h, h2, (size_t)(n_pairs * d_ff), h, ctx->stream));
+            swiglu_u = nullptr;
+        }
+    } else {
         QP_HIP(ctx, launch_moe_swiglu_gemv(g, mt, (int)E, ctx->stream));
-    if (!fuse_h) QP_HIP(ctx, run_quantize(ctx, ph, ws + off_hq, h, n_pairs, d_ff, false));
+    }
+    if (!fuse_h) QP_HIP(ctx, run_quantize(ctx, ph, ws + off_hq, h, n_pairs, d_ff, false, swiglu_u));
     GemvArgs gd{};
     if (pair_mode) {
         gd.ids = ids_dev;
