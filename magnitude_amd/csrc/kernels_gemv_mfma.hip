@@ -954,7 +954,11 @@ Split plan(int64_t K, int64_t M, int64_t total_rg, int W, int min_wgs = 200, boo
     auto wgs_of = [&](int kw) { return (total_rg + W / kw - 1) / (W / kw); };
     if (dense && p.kw > 1 && wgs_of(p.kw) * nc > cus && wgs_of(p.kw / 2) * nc <= cus) p.kw /= 2;
     const int64_t wgs1 = wgs_of(p.kw);
-    if (wgs1 * nc < 128) nc = std::max(nc, (int)std::min<int64_t>(std::max(1, nb / p.kw), (255 + wgs1) / wgs1));
+    // few workgroups: more chunks - in a dense launch (one workgroup a compute unit) as many as still make ONE round
+    // (96 row-group sets of K = 8192 got three chunks, 288 workgroups, a round and an eighth: Q4_K 8192 -> 3072 at
+    // 4 / 8 rows 20.6 / 20.8 us against 15.8 at 16 rows, whose two chunks are 192)
+    if (wgs1 * nc < 128)
+        nc = std::max(nc, (int)std::min<int64_t>(std::max(1, nb / p.kw), dense ? std::max<int64_t>(1, cus / wgs1) : (255 + wgs1) / wgs1));
     else if (dense && nc > 1 && wgs1 * nc * 10 < cus * 7)   // the sum over chunks is paid for anyway: fill the round
         nc = std::max(nc, (int)std::min<int64_t>(std::max(1, nb / p.kw), cus / wgs1));
     p.chunk_sb = (nb + nc - 1) / nc;
