@@ -373,11 +373,14 @@ int64_t small_batch_pass(int type, int64_t M) {
 // Which batches take the tiled matrix-core products (weights reused across a tile of tokens, K cut into stretches
 // where the grid would leave the chip idle) instead of passes of the 16-row small-batch kernel.  ONE predicate for
 // the dispatch and for the scratch sizing: the partial tiles of a K cut into stretches go to scratch that only this
-// rule provides.  Q8_0 from 64 rows on with K a multiple of 128; Q4_K and Q6_K from the row counts below.
+// rule provides.  From the row counts below (Q8_0 with K a multiple of 128).
 int tiled_min_m(int type) {
     static const int q4 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q4K", 33));
     static const int q6 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q6K", 33));
-    return type == kTypeQ4_K ? q4 : type == kTypeQ6_K ? q6 : 64;
+    // (Q8_0 took two 32-row passes up to 63 rows: 8192 -> 3072 at 33 / 63 rows 36.8 / 44.6 us against 27.5 / 27.8 tiled,
+    // 14336 -> 4096 49.6 / 60.9 against 40.4 / 41.1; at 17..32 rows the one pass stays ahead, 23.6 - 25.8 against 27.2 - 27.7)
+    static const int q8 = std::max(3, tuning_int("QPROJ_TILED_MIN_M_Q8_0", 33));
+    return type == kTypeQ4_K ? q4 : type == kTypeQ6_K ? q6 : q8;
 }
 bool takes_tiled(const qproj_weight *t, int64_t M) {
     // (Q6_K rows beyond 16384 weights: a 32-row pass of the small-batch kernel would stage K in more than eight chunks
