@@ -80,6 +80,47 @@ class Timer:
         return [a.elapsed_time(b) for a, b in evs]
 
 
+def median(samples):
+    """the reference's median (inference/crates/icn-parity/src/compare.rs:757-766): mean of the two middle samples
+    of an even count"""
+    v = sorted(float(x) for x in samples)
+    mid = len(v) // 2
+    return (v[mid - 1] + v[mid]) / 2.0 if len(v) % 2 == 0 else v[mid]
+
+
+def summarize(samples):
+    """median and median absolute deviation of raw samples, as the reference's comparator summarizes a measurement
+    (compare.rs:727-733), plus the count; `rel_mad` = MAD / median"""
+    med = median(samples)
+    mad = median([abs(float(x) - med) for x in samples])
+    return {"median": med, "mad": mad, "rel_mad": mad / med if med > 0 else 0.0, "n": len(samples)}
+
+
+MIN_SAMPLES, MIN_WARMUP = 30, 5      # every per-kernel figure: at least this many timed samples after this many warm-ups
+
+
+def physical_cores():
+    """(physical cores, logical CPUs) this process may run on: distinct (package, core) pairs over the CPUs of its
+    affinity mask, from /sys/devices/system/cpu/cpuN/topology (the reference runs one thread a physical core:
+    inference/parity/profiles/pr.toml:41)"""
+    try:
+        cpus = sorted(os.sched_getaffinity(0))
+    except AttributeError:
+        cpus = list(range(os.cpu_count() or 1))
+    cores = set()
+    for c in cpus:
+        base = f"/sys/devices/system/cpu/cpu{c}/topology/"
+        try:
+            with open(base + "physical_package_id") as f:
+                pkg = f.read().strip()
+            with open(base + "core_id") as f:
+                core = f.read().strip()
+            cores.add((pkg, core))
+        except OSError:
+            cores.add(("?", str(c)))
+    return len(cores), len(cpus)
+
+
 def capture(torch, stream, fn):
     """Captures fn() (launches on `stream` only) into a HIP graph; returns replay() or None."""
     try:
@@ -134,6 +175,18 @@ def measured_traffic(summary="decode_gate_up_q4k.txt"):
     return traffic, f"profiles/{summary} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel sources {digest})"
 
 
+def recorded_streaming_probe(summary="decode_gate_up_q4k.txt"):
+    """[low, high] microseconds that a kernel of the decode kernel's grid which only streams the 66 MB of a gate+up
+    launch was measured at (committed profile summary, line `streaming_probe_us: lo hi`); None when not recorded"""
+    try:
+        for line in open(os.path.join(ROOT, "profiles", summary)):
+            if line.startswith("streaming_probe_us:"):
+                return [float(v) for v in line.split(":")[1].split()]
+    except (OSError, ValueError):
+        pass
+    return None
+
+
 def _r(v, nd=4):
     return None if v is None else round(float(v), nd)
 
@@ -151,34 +204,48 @@ def compact_line(out, details_path=None):
     for k in ("pct_hbm_peak", "tokens_per_s_projection_only"):
         if out.get(k) is not None:
             line[k] = _r(out[k], 2)
+    if out.get("step_stats"):
+        st = out["step_stats"]
+        line["value_stats"] = {"statistic": "median + MAD over per-step samples", "median_ms": _r(st["median"], 5),
+                               "mad_ms": _r(st["mad"], 5), "rel_mad": _r(st["rel_mad"], 4), "n": st["n"]}
     rf = out.get("roofline")
     if rf:
         line["roofline"] = {k: (_r(rf[k]) if isinstance(rf.get(k), float) else rf.get(k))
                             for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "traffic_source", "kernel",
-                                      "bytes_per_launch", "us_per_launch", "launches_timed")}
+                                      "bytes_per_launch", "us_per_launch", "mad_us", "rel_mad", "samples", "launches_timed",
+                                      "launch_us", "streaming_probe_us")
+                            if k in rf}
         line["decode_kernels_us"] = {k: _r(v["us_per_launch"], 2) for k, v in rf.get("other_kernels", {}).items()}
     cb = out.get("cpu_baseline")
     if cb:
         line["cpu_baseline"] = {k: (_r(cb[k]) if isinstance(cb.get(k), float) else cb.get(k))
-                                for k in ("value", "unit", "cores", "kind", "sample", "host_cpus", "one_thread_GBps", "isa")
+                                for k in ("value", "unit", "cores", "kind", "sample", "host_cpus", "host_physical_cores",
+                                          "thread_policy", "rel_mad", "one_thread_GBps", "isa")
                                 if k in cb}
     if "verify" in out:
         line["verify_us"] = {f"M{r['M']}_{r['group']}": _r(r["us_per_launch"], 2) for r in out["verify"]["shapes"]}
+        if all("us_rows_quantized_earlier" in r for r in out["verify"]["shapes"]):
+            line["verify_us_rows_quantized_earlier"] = {f"M{r['M']}_{r['group']}": _r(r["us_rows_quantized_earlier"], 2)
+                                                        for r in out["verify"]["shapes"]}
     if "q8_0" in out:
         line["q8_0_gemv"] = {"us": _r(out["q8_0"]["us_per_launch"], 2), "frac_hbm_peak": _r(out["q8_0"]["frac_hbm_peak"])}
     for key, tag in (("prefill", "prefill_q8x32"), ("prefill_ggml_acts", "prefill_q8k")):
         if key in out:
             pf = out[key]
             line[tag] = {"headline_tops": _r(pf["headline_tops"], 1), "frac_int8_peak": _r(pf["headline_frac_int8_peak"]),
+                         "rel_mad": _r(pf.get("headline_rel_mad")), "samples": pf.get("samples_per_shape"),
                          "peak_tops": INT8_PEAK_TOPS, "shape": "M4096 K4096 N14336 Q4_K",
                          "tops": {f"{r.get('type', 'Q4_K')}_M{r['M']}_K{r['K']}_N{r['N']}": _r(r["gemm_tops"], 0)
                                   for r in pf["shapes"]}}
+            for k in ("bound", "floor_tops", "floor"):
+                if k in pf:
+                    line[tag][k] = pf[k]
     if "moe" in out:
-        line["moe_ffn"] = {f"B{r['B']}": {"us": _r(r["ms"] * 1e3, 1), "GBps": _r(r["GBps"], 0),
+        line["moe_ffn"] = {f"B{r['B']}": {"us": _r(r["ms"] * 1e3, 1), "GBps": _r(r["GBps"], 0), "rel_mad": _r(r.get("rel_mad")),
                                           "MB_cycled": _r(r.get("bytes_cycled", 0) / 1e6, 0)}
                            for r in out["moe"]["batches"]}
     if "llama_bench" in out:
-        med = lambda v: sorted(v)[len(v) // 2]
+        med = median
         toks = {r["output"]["operation"].split(".")[1]: med(r["measurements"][1]["samples"]) for r in out["llama_bench"]}
         line["llama_bench_projections_only"] = {"pp512_tok_s": _r(toks.get("prompt-processing"), 0),
                                                 "tg128_tok_s": _r(toks.get("token-generation"), 1)}
@@ -301,25 +368,34 @@ def main():
         step()
         ctx.sync()
         def timed(run):
+            """K steps between two synchronizations (the quoted time), with an event after every step on the library's
+            stream so that the spread over the steps is known too"""
             for _ in range(args.warmup):
                 run()
             torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(args.steps):
-                run()
-            torch.cuda.synchronize()
-            return (time.perf_counter() - t0) / args.steps
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+            with torch.cuda.stream(stream):
+                t0 = time.perf_counter()
+                evs[0].record(stream)
+                for i in range(args.steps):
+                    run()
+                    evs[i + 1].record(stream)
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) / args.steps
+            return dt, [evs[i].elapsed_time(evs[i + 1]) for i in range(args.steps)]
 
         # The 128 launches of a step are issued either one by one or as a replay of a HIP graph; both are timed
         # (warmup + the same number of steps each) and the step is quoted on the faster route.  Issued one by
         # one the host stays ahead of the device here (a launch costs it about 6 us, the average kernel 9 us),
         # and the replay has measured 3 % slower than that on this runtime.
-        modes = {"eager": timed(step)}
+        runs = {"eager": timed(step)}
         replay = None if args.no_graph else capture(torch, stream, step)
         if replay is not None:
-            modes["hip_graph"] = timed(replay)
+            runs["hip_graph"] = timed(replay)
+        modes = {k: v[0] for k, v in runs.items()}
         best = min(modes, key=modes.get)
         dt = modes[best]
+        out["step_stats"] = summarize(runs[best][1])          # ms per step, one sample a step (events)
         out["config"]["launch_route"] = best
         out["config"]["hip_graph"] = best == "hip_graph"
         out["ms_per_step_by_route"] = {k: v * 1e3 for k, v in modes.items()}
@@ -333,10 +409,34 @@ def main():
             f"{1.0 / dt:.0f} tok/s (projections only)  [" +
             ", ".join(f"{k} {v * 1e3:.3f} ms" for k, v in modes.items()) + "]")
 
+    # ------------------------------------------------------------------ fixed cost of a launch
+    launch_us = None
+    if legs & {"roofline", "moe"}:
+        # the fixed cost of a launch, measured in this run from the smallest launch the library has (one 256 x 64 Q4_K
+        # projection of one row: a single workgroup), 64 of them a graph replay; the calibration records below carry it
+        # (launch_microseconds, inference/crates/icn-server/src/main.rs:1313-1325)
+        tiny = ctx.upload_from_device(Q4_K, 256, 64, synth.random_weight(Q4_K, 64, 256, seed=3, device=dev))
+        x_tiny, y_tiny = torch.randn((1, 256), generator=g, device=dev), torch.empty((1, 64), device=dev)
+
+        def tiny_launches():
+            for _ in range(64):
+                ctx.mul_mat_multi([tiny], x_tiny, ACT_GGML, outs=[y_tiny], sync=False)
+        tiny_launches()
+        ctx.sync()
+        run = (None if args.no_graph else capture(torch, stream, tiny_launches)) or tiny_launches
+        for _ in range(MIN_WARMUP):
+            run()
+        torch.cuda.synchronize()
+        launch_stats = summarize([s_ / 64 * 1e3 for s_ in timer.samples_ms(run, max(MIN_SAMPLES, args.steps))])
+        launch_us = launch_stats["median"]
+        out["launch_us"] = launch_stats
+        log(f"[bench] smallest launch (one workgroup): {launch_us:.2f} us a launch (MAD {launch_stats['mad']:.3f})")
+        tiny.free()
+
     # ------------------------------------------------------------------ roofline leg: dominant kernel
     ev_rows, ev_meas, ev_cal = [], [], []
     if "roofline" in legs:
-        reps = max(5, args.steps)
+        reps = max(MIN_SAMPLES, args.steps)
         per = {}
         for grp in groups:
             def all_layers(grp=grp):
@@ -346,14 +446,16 @@ def main():
             ctx.sync()
             run = None if args.no_graph else capture(torch, stream, all_layers)
             run = run or all_layers
-            for _ in range(3):
+            for _ in range(MIN_WARMUP):
                 run()
             torch.cuda.synchronize()
             samples = [s / L * 1e3 for s in timer.samples_ms(run, reps)]   # us per launch, one sample per replay
-            ms = sum(samples) / len(samples) * 1e-3
+            st = summarize(samples)
+            ms = st["median"] * 1e-3
             nbytes = sum(gemv_bytes(lw_t, n, k) for nm, lw_t, n, k in LAYER_TENSORS if nm in grp[1]) \
                 - (len(grp[1]) - 1) * grp[2].numel() * 4      # the shared activation row is read once
-            per[grp[0]] = {"us_per_launch": ms * 1e3, "bytes_per_launch": nbytes,
+            per[grp[0]] = {"us_per_launch": ms * 1e3, "mad_us": st["mad"], "rel_mad": st["rel_mad"], "samples": st["n"],
+                           "bytes_per_launch": nbytes,
                            "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
             log(f"[bench] kernel {grp[0]:8s}: {ms * 1e3:7.2f} us  {per[grp[0]]['GBps']:6.0f} GB/s "
                 f"({100 * per[grp[0]]['frac_hbm_peak']:.1f}% of peak)")
@@ -363,7 +465,7 @@ def main():
                                                     flops=2.0 * rows * kk, bytes_moved=nbytes,
                                                     memory_kb=nbytes // 1024, device=props.name))
             ev_meas.append(evidence.measurement(f"decode.{grp[0]}.launch", "us", samples))
-            ev_cal.append(evidence.calibration_metric(qt0, False, nbytes, samples, launch_us=2.0))
+            ev_cal.append(evidence.calibration_metric(qt0, False, nbytes, samples, launch_us=launch_us))
         dom = per["gate_up"]
         traffic, traffic_source = measured_traffic()
         out["roofline"] = {"bound": "hbm", "achieved": dom["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -371,7 +473,13 @@ def main():
                            "kernel": "gemv_decode_kernel<Q4_K, M=1>: gate+up (2 x 4096->14336) in one launch, "
                                      "activation quantized in the prologue",
                            "bytes_per_launch": dom["bytes_per_launch"], "us_per_launch": dom["us_per_launch"],
-                           "launches_timed": reps * L, "other_kernels": {k: v for k, v in per.items() if k != "gate_up"}}
+                           "statistic": "median of one sample per graph replay of the 32 layers' launches",
+                           "mad_us": dom["mad_us"], "rel_mad": dom["rel_mad"], "samples": dom["samples"],
+                           "launches_timed": reps * L, "launch_us": launch_us,
+                           "other_kernels": {k: v for k, v in per.items() if k != "gate_up"}}
+        probe = recorded_streaming_probe()
+        if probe:
+            out["roofline"]["streaming_probe_us"] = probe
         if args.calib_copy:
             # a plain elementwise kernel of known traffic (reads 256 MiB, writes 256 MiB) to scale the
             # FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this same command
@@ -395,18 +503,35 @@ def main():
                 def all_layers(names=names, k=k):
                     for lw in layers:
                         ctx.mul_mat_multi([lw[n] for n in names], xs[k], ACT_GGML, outs=[ys[n] for n in names], sync=False)
-                all_layers()
-                ctx.sync()
-                run = (None if args.no_graph else capture(torch, stream, all_layers)) or all_layers
-                run()
-                torch.cuda.synchronize()
-                ms = timer.time_ms(run, max(5, args.steps)) / L
+                def timed_layers(fn):
+                    fn()
+                    ctx.sync()
+                    run = (None if args.no_graph else capture(torch, stream, fn)) or fn
+                    for _ in range(MIN_WARMUP):
+                        run()
+                    torch.cuda.synchronize()
+                    return summarize([s_ / L * 1e3 for s_ in timer.samples_ms(run, max(MIN_SAMPLES, args.steps))])
+                st = timed_layers(all_layers)
+                ms = st["median"] * 1e-3
+                # the same projections through the entry point a graph reaches them by when the rows were quantized by
+                # an earlier node (the norm in front writes the planes: qproj_rms_norm_quantize, then
+                # qproj_mul_mat_quantized): no quantizer launch inside the timed call
+                qt0 = {nm: t for nm, t, _, _ in LAYER_TENSORS}[names[0]]
+                qb = torch.empty(int(lib.qproj_act_bytes(ACT_GGML, qt0, m, k)), dtype=torch.uint8, device=dev)
+                ctx.quantize_activations_raw(xs[k], ACT_GGML, qt0, out=qb, sync=True)
+
+                def all_layers_q(names=names, qb=qb):
+                    for lw in layers:
+                        ctx.mul_mat_quantized([lw[n] for n in names], qb, ACT_GGML, m, [ys[n] for n in names], sync=False)
+                stq = timed_layers(all_layers_q)
                 nbytes = sum(gemv_bytes(t, n, kk, m) for nm, t, n, kk in LAYER_TENSORS if nm in names) \
                     - (len(names) - 1) * m * k * 4
-                res.append({"M": m, "group": gname, "us_per_launch": ms * 1e3, "GBps": nbytes / (ms * 1e-3) / 1e9,
+                res.append({"M": m, "group": gname, "us_per_launch": ms * 1e3, "mad_us": st["mad"], "samples": st["n"],
+                            "us_rows_quantized_earlier": stq["median"], "mad_us_rows_quantized_earlier": stq["mad"],
+                            "GBps": nbytes / (ms * 1e-3) / 1e9,
                             "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS})
                 log(f"[bench] verify M={m:2d} {gname:8s}: {ms * 1e3:7.2f} us  {res[-1]['GBps']:6.0f} GB/s "
-                    f"({100 * res[-1]['frac_hbm_peak']:.1f}% of peak)")
+                    f"({100 * res[-1]['frac_hbm_peak']:.1f}% of peak); rows quantized by an earlier call: {stq['median']:.2f} us")
         out["verify"] = {"note": "weights read once for all M rows; ggml activation mode", "shapes": res}
 
     # ------------------------------------------------------------------ Q8_0 leg (config 1)
@@ -425,11 +550,13 @@ def main():
         rot()
         ctx.sync()
         run = (None if args.no_graph else capture(torch, stream, rot)) or rot
-        run()
+        for _ in range(MIN_WARMUP):
+            run()
         torch.cuda.synchronize()
-        ms = timer.time_ms(run, max(5, args.steps)) / nrot
+        stq8 = summarize([s_ / nrot * 1e3 for s_ in timer.samples_ms(run, max(MIN_SAMPLES, args.steps))])
+        ms = stq8["median"] * 1e-3
         nbytes = gemv_bytes(Q8_0, D_MODEL, D_MODEL)
-        out["q8_0"] = {"shape": "4096x4096, M=1", "us_per_launch": ms * 1e3, "GBps": nbytes / (ms * 1e-3) / 1e9,
+        out["q8_0"] = {"shape": "4096x4096, M=1", "us_per_launch": ms * 1e3, "mad_us": stq8["mad"], "samples": stq8["n"], "GBps": nbytes / (ms * 1e-3) / 1e9,
                        "frac_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
         log(f"[bench] q8_0 4096x4096 M=1: {ms * 1e3:.2f} us  {out['q8_0']['GBps']:.0f} GB/s")
         for w in ws:
@@ -498,18 +625,20 @@ def main():
                 torch.cuda.synchronize()
                 fq = lambda: ctx.quantize_activations_raw(x, ACT_Q8X32, Q4_K, out=qb, sync=False)
                 fg = lambda: ctx.mul_mat_quantized([w], qb, ACT_Q8X32, m, [yb], sync=False)
-                fq(); fg(); ctx.sync()
-                it = 5 if m * n * k > 1e11 else 10
-                tq = timer.time_ms(fq, it)
-                sg = timer.samples_ms(fg, it)
-                tg = sum(sg) / len(sg)
+                for _ in range(MIN_WARMUP):
+                    fq(); fg()
+                ctx.sync()
+                tq = median(timer.samples_ms(fq, MIN_SAMPLES))
+                sg = timer.samples_ms(fg, MIN_SAMPLES)
+                stg = summarize(sg)
+                tg = stg["median"]
                 ops = 2.0 * m * n * k
                 ev_rows.append(evidence.backend_ops_row("MUL_MAT", evidence.mul_mat_params(Q4_K, n, m, k) + ",act=q8x32",
                                                         [s * 1e3 for s in sg], flops=ops,
                                                         bytes_moved=gguf_bytes(Q4_K, n, k) + m * k + m * n * 4,
                                                         memory_kb=(gguf_bytes(Q4_K, n, k) + m * n * 4) // 1024,
                                                         device=props.name))
-                res.append({"M": m, "K": k, "N": n, "gemm_ms": tg, "quantize_ms": tq,
+                res.append({"M": m, "K": k, "N": n, "gemm_ms": tg, "gemm_mad_ms": stg["mad"], "rel_mad": stg["rel_mad"], "quantize_ms": tq,
                             "gemm_tops": ops / (tg * 1e-3) / 1e12,
                             "end_to_end_tops": ops / ((tg + tq) * 1e-3) / 1e12,
                             "frac_int8_peak": ops / (tg * 1e-3) / 1e12 / INT8_PEAK_TOPS})
@@ -520,6 +649,15 @@ def main():
         head = [r for r in res if (r["M"], r["K"], r["N"]) == (4096, 4096, 14336)][0]
         out["prefill"] = {"act_format": "per-32 int8 + fp32 scale", "mfma": "v_mfma_i32_32x32x32_i8",
                           "headline_tops": head["gemm_tops"], "headline_frac_int8_peak": head["frac_int8_peak"],
+                          "headline_rel_mad": head["rel_mad"], "samples_per_shape": MIN_SAMPLES, "statistic": "median",
+                          # What bounds this format (not the matrix cores): both operands change scale every 32 weights, so
+                          # an int32 result is good for ONE matrix instruction and each of its 16 outputs a lane costs
+                          # convert + scale product + fma on the vector ALU: 48 vector instructions behind every
+                          # 32 x 32 x 32 product (52.8 measured with addresses and loads).  With a matrix instruction holding
+                          # the issue port 16 of its 32 cycles and a vector instruction 4, the floor is
+                          # 5000 TOPS x 32 / (16 + 4 x 52.8) = 704 TOPS (profiles/prefill_gemm_kernels.txt, section 2).
+                          "bound": "valu", "floor_tops": 704.0,
+                          "floor": "5000 x 32 / (16 + 4 x 52.8): 48 of 52.8 vector instr. per matrix instr. are the per-32 flush",
                           "peak_tops": INT8_PEAK_TOPS, "shapes": res}
         # the same shapes in the ggml activation format (Q8_K, one scale per 256): the reference's own arithmetic
         # (plus the layer's Q6_K down projection, which a Q4_K_M model runs through the same operator, and
@@ -537,11 +675,13 @@ def main():
                 torch.cuda.synchronize()
                 fq = lambda: ctx.quantize_activations_raw(x, ACT_GGML, qt, out=qb, sync=False)
                 fg = lambda: ctx.mul_mat_quantized([w], qb, ACT_GGML, m, [yb], sync=False)
-                fq(); fg(); ctx.sync()
-                it = 5 if m * n * k > 1e11 else 10
-                tq = timer.time_ms(fq, it)
-                sg = timer.samples_ms(fg, it)
-                tg = sum(sg) / len(sg)
+                for _ in range(MIN_WARMUP):
+                    fq(); fg()
+                ctx.sync()
+                tq = median(timer.samples_ms(fq, MIN_SAMPLES))
+                sg = timer.samples_ms(fg, MIN_SAMPLES)
+                stg = summarize(sg)
+                tg = stg["median"]
                 ops = 2.0 * m * n * k
                 ev_rows.append(evidence.backend_ops_row("MUL_MAT", evidence.mul_mat_params(qt, n, m, k),
                                                         [s * 1e3 for s in sg], flops=ops,
@@ -549,7 +689,7 @@ def main():
                                                         memory_kb=(gguf_bytes(qt, n, k) + m * n * 4) // 1024,
                                                         device=props.name))
                 tname = {Q4_K: "Q4_K", Q6_K: "Q6_K", Q8_0: "Q8_0"}[qt]
-                resg.append({"type": tname, "M": m, "K": k, "N": n, "gemm_ms": tg, "quantize_ms": tq,
+                resg.append({"type": tname, "M": m, "K": k, "N": n, "gemm_ms": tg, "gemm_mad_ms": stg["mad"], "rel_mad": stg["rel_mad"], "quantize_ms": tq,
                              "gemm_tops": ops / (tg * 1e-3) / 1e12,
                              "frac_int8_peak": ops / (tg * 1e-3) / 1e12 / INT8_PEAK_TOPS})
                 log(f"[bench] prefill(ggml acts) {tname} M={m} K={k} N={n}: gemm {tg:.3f} ms = {resg[-1]['gemm_tops']:.1f} TOPS "
@@ -562,6 +702,7 @@ def main():
                                             "Q6_K: v_mfma_i32_32x32x16_i8 per sub-block, integer scale on the vector ALU; "
                                             "Q8_0: v_mfma_i32_32x32x32_i8 per block, fp32 scales",
                                     "headline_tops": headg["gemm_tops"], "headline_frac_int8_peak": headg["frac_int8_peak"],
+                                    "headline_rel_mad": headg["rel_mad"], "samples_per_shape": MIN_SAMPLES, "statistic": "median",
                                     "shapes": resg}
 
     # ------------------------------------------------------------------ MoE leg (config 5)
@@ -607,9 +748,12 @@ def main():
             rotation(); ctx.sync()
             run = (None if args.no_graph else capture(torch, stream, rotation)) or rotation
             run(); torch.cuda.synchronize()
-            reps = max(2, 96 // len(calls))
-            sm_ = [s_ / len(calls) for s_ in timer.samples_ms(run, reps)]     # ms per call, one sample per rotation
-            ms = sum(sm_) / len(sm_)
+            for _ in range(MIN_WARMUP - 1):
+                run()
+            torch.cuda.synchronize()
+            sm_ = [s_ / len(calls) for s_ in timer.samples_ms(run, MIN_SAMPLES)]     # ms per call, one sample per rotation
+            stm = summarize(sm_)
+            ms = stm["median"]
             byts = sum(distinct) / len(calls) * per_expert + B * dm * 4 * 2  # mean distinct-expert bytes of a call
             run1 = (None if args.no_graph else capture(torch, stream, resident)) or resident
             run1(); torch.cuda.synchronize()
@@ -619,9 +763,10 @@ def main():
                                                     ",fused=moe_ffn(gate,up,swiglu,down,combine)", [s_ * 1e3 for s_ in sm_],
                                                     flops=2.0 * B * top * 3 * dm * dff, bytes_moved=byts,
                                                     memory_kb=int(byts) // 1024, device=props.name))
-            ev_cal.append(evidence.calibration_metric(Q4_K, True, byts, [s_ * 1e3 for s_ in sm_], launch_us=2.0))
+            ev_cal.append(evidence.calibration_metric(Q4_K, True, byts, [s_ * 1e3 for s_ in sm_], launch_us=launch_us))
             res.append({"B": B, "distinct_experts_mean": sum(distinct) / len(calls), "calls_in_rotation": len(calls),
-                        "bytes_cycled": cycled, "ms": ms, "GBps": byts / (ms * 1e-3) / 1e9,
+                        "bytes_cycled": cycled, "ms": ms, "mad_ms": stm["mad"], "rel_mad": stm["rel_mad"], "samples": stm["n"],
+                        "GBps": byts / (ms * 1e-3) / 1e9,
                         "frac_hbm_peak": byts / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                         "cache_resident": {"ms": ms1, "GBps": byts1 / (ms1 * 1e-3) / 1e9, "bytes": byts1}})
             log(f"[bench] moe B={B}: {ms * 1e3:.1f} us a call over a rotation of {len(calls)} calls cycling {cycled / 1e6:.0f} MB "
@@ -641,24 +786,28 @@ def main():
         from oracle import oracle as orc
         import numpy as np
         orc.build()
-        nl = min(4, L)
+        nl = L                       # every layer of the step: 4.4 GB of blocks on the host, far beyond its caches
         host = [[(qt, n, k, ctx.download(layers[l][name])) for name, qt, n, k in LAYER_TENSORS] for l in range(nl)]
         xs = {D_MODEL: x_attn.cpu().numpy(), D_FF: x_down.cpu().numpy()}
-        # every thread of the box's CPU share (16 for one GPU); the reference's own policy is one thread per physical
-        # core (inference/parity/profiles/pr.toml:41).  AVX2 dot products in the shape of ggml's x86 path when the
-        # oracle was built with them, the generic C loops otherwise.
-        threads = min(orc.max_threads(), 16)
+        # One thread a physical core, the reference's own policy (inference/parity/profiles/pr.toml:41), counted from
+        # /sys over the CPUs this process may run on and capped by the 16 CPUs a one-GPU box gives a job.  AVX2 dot
+        # products in the shape of ggml's x86 path when the oracle was built with them, the generic C loops otherwise.
+        phys, logical = physical_cores()
+        threads = max(1, min(phys, orc.max_threads(), 16))
         avx2 = orc.has_avx2()
         run_cpu = (lambda qt, blocks, k, th: orc.time_mul_mat_avx2(qt, blocks, k, xs[k], th, 1)) if avx2 else \
                   (lambda qt, blocks, k, th: orc.time_mul_mat(qt, blocks, k, xs[k], orc.ACT_GGML, th, 1))
         t_end = time.time() + args.cpu_seconds
-        passes, spent = 0, 0.0
-        while passes < 2 or time.time() < t_end:
+        pass_s = []                                # seconds of arithmetic per pass over the layers
+        while len(pass_s) < 2 or time.time() < t_end:
+            t_pass = 0.0
             for lw in host:
                 for qt, n, k, blocks in lw:
-                    spent += run_cpu(qt, blocks, k, threads)
-            passes += 1
-        cpu_gbs = passes * nl * LAYER_BYTES / spent / 1e9
+                    t_pass += run_cpu(qt, blocks, k, threads)
+            pass_s.append(t_pass)
+        passes, spent = len(pass_s), sum(pass_s)
+        stc = summarize(pass_s)
+        cpu_gbs = nl * LAYER_BYTES / stc["median"] / 1e9
         one = 0.0                                  # one thread, one layer
         for qt, n, k, blocks in host[0]:
             one += run_cpu(qt, blocks, k, 1)
@@ -666,19 +815,21 @@ def main():
         for qt, n, k, blocks in host[0]:
             scalar_one += orc.time_mul_mat(qt, blocks, k, xs[k], orc.ACT_GGML, 1, 1)
         out["cpu_baseline"] = {"value": cpu_gbs, "unit": "GB/s", "cores": threads, "kind": "port",
-                               "sample": f"{passes} passes over {nl} of the same layers (7 projections each, M=1, "
-                                         f"ggml activation mode), {spent:.1f} s on the host",
+                               "sample": f"{passes} passes over the same {nl} layers (7 projections each, M=1, ggml activation "
+                                         f"mode; median pass), {spent:.1f} s on the host",
+                               "rel_mad": stc["rel_mad"], "thread_policy": "physical-cores, at most the box's 16-CPU share",
+                               "host_physical_cores": phys, "host_logical_cpus": logical,
                                "isa": "AVX2 maddubs/madd dot products, OpenMP over rows" if avx2 else "generic C, OpenMP over rows",
                                "host_cpus": os.cpu_count(),
                                "one_thread_GBps": LAYER_BYTES / one / 1e9,
                                "one_thread_generic_c_GBps": LAYER_BYTES / scalar_one / 1e9}
-        log(f"[bench] cpu baseline: {cpu_gbs:.2f} GB/s on {threads} threads")
+        log(f"[bench] cpu baseline: {cpu_gbs:.2f} GB/s on {threads} threads ({phys} physical cores, {logical} logical CPUs usable)")
 
     # ------------------------------------------------------------------ llama-bench style leg
     # pp512 / tg128 over the projections of all layers (no attention, norms or sampling): the prompt
     # pass is one 512-token batch per layer tensor group, generation is 128 single-token steps.
     if "llama_bench" in legs:
-        n_prompt, n_gen, reps = 512, 128, 5
+        n_prompt, n_gen, reps = 512, 128, 10       # the reference's gate takes the median of 10 (generation-128.json:44-51)
         xs = {kk: torch.randn((n_prompt, kk), generator=g, device=dev) for kk in (D_MODEL, D_FF)}
         yp = {name: torch.empty((n_prompt, n), device=dev) for name, _, n, _ in LAYER_TENSORS}
 
@@ -708,7 +859,7 @@ def main():
         rec_pp = evidence.llama_bench_record("llama-bench.prompt-processing", n_prompt, 1, 0, 0, pp, cfg, devs)
         rec_tg = evidence.llama_bench_record("llama-bench.token-generation", 0, 0, n_gen, n_gen, tg, cfg, devs)
         out["llama_bench"] = [rec_pp, rec_tg]
-        med = lambda v: sorted(v)[len(v) // 2]
+        med = median
         log(f"[bench] llama-bench style, projections only: pp{n_prompt} {n_prompt * 1e9 / med(pp):.0f} tok/s "
             f"({med(pp) / 1e6:.2f} ms), tg{n_gen} {n_gen * 1e9 / med(tg):.0f} tok/s ({med(tg) / 1e6:.1f} ms)")
 

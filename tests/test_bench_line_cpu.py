@@ -26,24 +26,31 @@ def full_result(nshapes=9, nsamples=400):
                    "launch_route": "eager", "hip_graph": False},
         "ms_per_step_by_route": {"eager": 1.19, "hip_graph": 1.23}, "pct_hbm_peak": 46.4265, "tokens_per_s_projection_only": 839.51,
         "bytes_per_step": 4421000000,
+        "step_stats": bench.summarize([1.19 + 0.001 * (i % 5) for i in range(20)]),
+        "launch_us": bench.summarize([1.77, 1.78, 1.76]),
         "roofline": {"bound": "hbm", "achieved": 4520.123456, "peak": 8000.0, "unit": "GB/s", "frac": 0.565015432,
                      "traffic": 66509926, "traffic_source": "profiles/decode_gate_up_q4k.txt (" + "s" * 80 + ")",
                      "kernel": "gemv_decode_kernel<Q4_K, M=1>: " + "k" * 100, "bytes_per_launch": 66191360,
-                     "us_per_launch": 14.6434343, "launches_timed": 640, "other_kernels": per},
-        "verify": {"note": "n", "shapes": [{"M": m, "group": g, "us_per_launch": 20.912345, "GBps": 3200.5, "frac_hbm_peak": 0.4}
+                     "us_per_launch": 14.6434343, "mad_us": 0.0512345, "rel_mad": 0.0034987, "samples": 30, "launches_timed": 960,
+                     "launch_us": 1.7712345, "streaming_probe_us": [11.3, 12.5], "other_kernels": per},
+        "verify": {"note": "n", "shapes": [{"M": m, "group": g, "us_per_launch": 20.912345, "us_rows_quantized_earlier": 16.812345,
+                                            "GBps": 3200.5, "frac_hbm_peak": 0.4}
                                            for m in (2, 4, 8, 16) for g in ("gate_up", "down")]},
         "q8_0": {"shape": "4096x4096, M=1", "us_per_launch": 6.07123, "GBps": 2940.12, "frac_hbm_peak": 0.3675},
         "norm": {"M=1": {"separate_us": 17.9, "fused_us": 16.2, "fused_swiglu_us": 16.3}},
         "prefill": {"act_format": "per-32", "mfma": "m", "headline_tops": 520.123, "headline_frac_int8_peak": 0.104,
+                    "headline_rel_mad": 0.0041234, "samples_per_shape": 30, "bound": "valu", "floor_tops": 704.0,
+                    "floor": "5000 x 32 / (16 + 4 x 52.8): 48 of 52.8 vector instr. per matrix instr. are the per-32 flush",
                     "peak_tops": 5000.0, "shapes": shapes},
         "prefill_ggml_acts": {"act_format": "q8k", "mfma": "m" * 200, "headline_tops": 911.6, "headline_frac_int8_peak": 0.1823,
-                              "shapes": ggml_shapes},
+                              "headline_rel_mad": 0.0061234, "samples_per_shape": 30, "shapes": ggml_shapes},
         "moe": {"experts": 128, "batches": [{"B": b, "distinct_experts_mean": 51.5, "calls_in_rotation": 12, "bytes_cycled": 1019215872,
-                                             "ms": 0.0551234, "GBps": 2581.123, "frac_hbm_peak": 0.32,
+                                             "ms": 0.0551234, "rel_mad": 0.0071234, "GBps": 2581.123, "frac_hbm_peak": 0.32,
                                              "cache_resident": {"ms": 0.05, "GBps": 2800.0, "bytes": 137000000}} for b in (1, 8, 64)],
                 "note": "n" * 300},
         "cpu_baseline": {"value": 9.912345, "unit": "GB/s", "cores": 16, "kind": "port", "sample": "s" * 160, "host_cpus": 128,
-                         "one_thread_GBps": 0.68123, "isa": "AVX2"},
+                         "host_physical_cores": 64, "host_logical_cpus": 128, "thread_policy": "physical-cores, at most the box's 16-CPU share",
+                         "rel_mad": 0.0123456, "one_thread_GBps": 0.68123, "isa": "AVX2"},
         "llama_bench": [evidence.llama_bench_record("llama-bench.prompt-processing", 512, 1, 0, 0, [12.3e6] * 5, cfg, devs),
                         evidence.llama_bench_record("llama-bench.token-generation", 0, 0, 128, 128, [157e6] * 5, cfg, devs)],
     }
@@ -75,6 +82,20 @@ def test_final_line_is_compact_and_complete():
     assert line["llama_bench_projections_only"]["pp512_tok_s"] == round(512e9 / 12.3e6)
     assert line["moe_ffn"]["B64"]["us"] == 55.1
     assert "evidence" not in line and line["details"] == "gpurun_out/bench_details.json"
+    # the spread of every headline figure rides on the line: median + MAD over raw samples, as the reference's
+    # comparator summarizes a measurement (inference/crates/icn-parity/src/compare.rs:727-766)
+    vs = line["value_stats"]
+    assert vs["n"] == 20 and vs["median_ms"] == 1.192 and vs["mad_ms"] == 0.001 and 0 < vs["rel_mad"] < 0.01
+    assert rf["mad_us"] == 0.0512 and rf["rel_mad"] == 0.0035 and rf["samples"] == 30 and rf["launch_us"] == 1.7712
+    assert rf["streaming_probe_us"] == [11.3, 12.5]
+    assert line["prefill_q8x32"]["rel_mad"] == 0.0041 and line["prefill_q8k"]["rel_mad"] == 0.0061
+    assert line["prefill_q8x32"]["samples"] == 30 and line["prefill_q8k"]["samples"] == 30
+    # config 4's own format is bounded by the vector ALU: the line says so, with the floor, and keeps frac against 5 POPS
+    assert line["prefill_q8x32"]["bound"] == "valu" and line["prefill_q8x32"]["floor_tops"] == 704.0
+    assert "floor" in line["prefill_q8x32"] and line["prefill_q8x32"]["peak_tops"] == 5000.0
+    assert line["moe_ffn"]["B64"]["rel_mad"] == 0.0071
+    assert cb["host_physical_cores"] == 64 and cb["cores"] == 16 and "physical-cores" in cb["thread_policy"] and cb["rel_mad"] == 0.0123
+    assert line["verify_us_rows_quantized_earlier"]["M16_down"] == 16.81
 
 
 def test_final_line_sheds_tables_before_contract_fields():
@@ -86,6 +107,16 @@ def test_final_line_sheds_tables_before_contract_fields():
     assert len(text) <= bench.MAX_LINE_BYTES
     assert line["roofline"]["frac"] and line["cpu_baseline"]["value"] and line["value"]
     assert line["prefill_q8k"]["headline_tops"] == 911.6 and "tops" not in line["prefill_q8k"]
+
+
+def test_summary_statistics_are_the_reference_comparators():
+    # median: mean of the two middle samples of an even count; MAD: median of the absolute deviations from it
+    assert bench.median([3.0, 1.0, 2.0]) == 2.0 and bench.median([4.0, 1.0, 3.0, 2.0]) == 2.5
+    st = bench.summarize([10.0, 12.0, 11.0, 30.0, 9.0])
+    assert st == {"median": 11.0, "mad": 1.0, "rel_mad": 1.0 / 11.0, "n": 5}
+    assert bench.MIN_SAMPLES >= 30 and bench.MIN_WARMUP >= 5
+    phys, logical = bench.physical_cores()
+    assert 1 <= phys <= logical
 
 
 def test_only_the_step_leg():
