@@ -22,7 +22,14 @@
  *   - activations, ids and outputs are DEVICE pointers owned by the caller (ggml tensors
  *     living in backend buffers); all work is enqueued on the context's HIP stream.  Outputs
  *     are ordinary device memory (hipMalloc; not host-coherent or managed allocations): some
- *     launches add their partial results to them with the memory side's float adder;
+ *     launches add their partial results to them with the memory side's float adder (two addends
+ *     onto rows cleared beforehand: the sum does not depend on their order; sums below the
+ *     smallest normal float are flushed to zero by that adder).  Where that route is taken the
+ *     launch that quantizes the activation rows also clears the output rows, so it writes y
+ *     before the projection does: outputs must not overlap the activations of the same call.
+ *     (The library looks for an overlap where it matters and then takes the route that stores
+ *     its results instead; callers should not rely on aliasing all the same.)  The add route
+ *     needs 16-byte aligned outputs and is skipped for others;
  *   - a context is used by one thread at a time (the reference serialises native calls on one
  *     executor thread: /root/reference/design/inference/engine.md:49-50).
  *   - row-major, ggml element order: x is [M][K], y is [M][N], W is N rows of K weights.
@@ -154,7 +161,15 @@ int qproj_rms_norm_ffn_gate_up(qproj_ctx *ctx, const qproj_weight *gate, const q
  *     y_dev[M][N] = down . ( silu(gate . x') * (up . x') ),   x' = rms_norm(x) * gamma or x.
  * gate and up are [K -> d_ff], down is [d_ff -> N].  Bit-identical to qproj_(rms_norm_)ffn_gate_up followed by
  * qproj_mul_mat: two launches for M <= 2; for batches the swiglu is formed inside the quantizer of the down projection
- * (gate and up go to scratch of the context, the intermediate rows are never written as fp32). */
+ * (gate and up go to scratch of the context, the intermediate rows are never written as fp32).
+ * What is promised end to end in the ggml activation mode: each half agrees with ggml's arithmetic to the last bits
+ * of fp32 (the integer dot products are exact, only the order of the fp32 additions differs: 5e-5 relative at most
+ * in the tests), and so does the whole - EXCEPT where a code of the re-quantized intermediate sits on a rounding tie.
+ * The down projection quantizes h to int8 as ggml does; a value of h that lies within an fp32 rounding of the middle
+ * between two codes may round the other way than on the CPU, and one code moves every output of that row by
+ * 1/127 of the largest |h| of its 256-wide block times a weight.  Measured over thousands of random cases: none at
+ * d_ff = 14336; at d_ff = 256..768 about one case in 500, up to 2e-3 relative in 1 % of its outputs.  That is a
+ * property of quantizing twice, the same between any two correct implementations of ggml's arithmetic. */
 int qproj_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *up, const qproj_weight *down,
               const float *x_dev, const float *gamma_dev, float eps, int use_norm, int64_t M, float *y_dev, int act);
 
@@ -176,8 +191,12 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
  * the library (one copy per GPU, held until the process ends) instead of the context's growable workspace, and the
  * call issues no hipMalloc / hipFree.  A call that needs more answers QPROJ_ERR_INVALID_ARG and launches nothing
  * (qproj_workspace_bytes tells the need beforehand; M <= 2 needs none; the 8B-class shapes fit up to M = 512).
- * All contexts on one GPU share that buffer, which keeps the last call's contents (every byte a kernel reads
- * was written earlier in the same call): calls that overlap in time on one GPU race. */
+ * The buffer keeps the last call's contents (every byte a kernel reads was written earlier in the same call), so
+ * two calls that overlap in time on one GPU would overwrite each other's scratch.  One context cannot do that (its
+ * calls are ordered on its stream); a second context could, unseen by either, so the buffer of a GPU belongs to the
+ * first context that calls this entry point on it until that context is destroyed, and calls from any other context
+ * are refused with QPROJ_ERR_UNSUPPORTED.  A call recorded into a HIP graph must not be replayed while other work of
+ * the same context that uses the buffer is in flight on another stream. */
 #define QPROJ_NOALLOC_SCRATCH_BYTES (64u << 20)
 int qproj_mul_mat_multi_noalloc(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev,
                                 int64_t M, float *const *y_dev, int act);
@@ -185,7 +204,10 @@ int qproj_mul_mat_multi_noalloc(qproj_ctx *ctx, int n, const qproj_weight *const
 /* Scratch bytes qproj_mul_mat_multi reserves for n tensors of `type` with rows N[0..n) sharing K, M activation
  * rows and activation mode `act` (0 for the decode regime, which needs none).  Needs no device: it walks the
  * library's own dispatch for that shape without launching, and checks on the way that every kernel launcher it
- * picks accepts a buffer of exactly that size and refuses a smaller one; *status (may be null) is QPROJ_OK then. */
+ * picks accepts what it is handed out of a buffer of exactly that size (each launcher works out its own demand and
+ * refuses less), that the reservation refuses a buffer one byte smaller, and that no launcher which cuts K goes
+ * ahead when it is handed no scratch at all; *status (may be null) is QPROJ_OK then.  The figure is an upper bound:
+ * matrices that ride in one launch with K whole leave the part reserved for their partial tiles unused. */
 size_t qproj_workspace_bytes(int type, int64_t K, int n, const int64_t *N, int64_t M, int act, int *status);
 
 /* The second half of a MUL_MAT on its own: `act_dev` holds M rows already quantized by
@@ -203,7 +225,10 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w_exps, const float *x_
 /* The MoE feed-forward of llama.cpp's build_moe_ffn, fused:
  *   y[b] = sum_j weights[b][j] * down_e( silu(gate_e x_b) * (up_e x_b) ),  e = ids[b][j]
  * x_dev f32 [B][d_model]; ids_dev int32 [B][n_used]; weights_dev f32 [B][n_used];
- * y_dev f32 [B][d_model].  gate/up are [d_model -> d_ff], down is [d_ff -> d_model]. */
+ * y_dev f32 [B][d_model].  gate/up are [d_model -> d_ff], down is [d_ff -> d_model].
+ * The same end-to-end promise as qproj_ffn: gate/up products, swiglu and the weighted sum follow ggml's arithmetic
+ * (halves within 5e-5 relative of it), the whole within 1e-3 except where a re-quantized code of the intermediate sits
+ * on a rounding tie (see qproj_ffn). */
 int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate_exps, const qproj_weight *up_exps,
                   const qproj_weight *down_exps, const float *x_dev, const int32_t *ids_dev,
                   const float *weights_dev, int64_t n_used, int64_t B, float *y_dev, int act);
@@ -234,6 +259,19 @@ typedef struct qproj_eligibility {
     char diagnostic[244];                                /* absent / failed: why                  */
 } qproj_eligibility;
 int qproj_probe_eligibility(qproj_eligibility *out);
+
+/* The routing table of the dispatch (no counterpart in the reference: ggml keeps its kernel selection inside each
+ * backend's supports_op / graph_compute; here it can be read and pinned by a test).  Writes into buf, one line a
+ * launch, the kernels that qproj_mul_mat_multi (with_norm = 0) or qproj_rms_norm_mul_mat (with_norm = 1) would launch
+ * for n matrices of `type` with K columns and N[i] rows against M activation rows in mode `act` - kernel, template
+ * instance, tile, grid, cuts of K - and a last line "scratch: <bytes> bytes".  The lines are written by the launchers
+ * themselves during a dry run of the code that serves the call; no device is touched.  Returns QPROJ_OK, the status
+ * the call would be refused with, or QPROJ_ERR_INVALID_ARG when buf is too small (the text is then cut). */
+int qproj_plan_mul_mat(int type, int64_t K, int n, const int64_t *N, int64_t M, int act, int with_norm, char *buf, size_t buf_bytes);
+/* The same for qproj_moe_ffn: gate/up experts [n_expert][d_ff][d_model] of gate_type, down experts of down_type,
+ * B tokens with n_used experts each. */
+int qproj_plan_moe_ffn(int gate_type, int down_type, int64_t d_model, int64_t d_ff, int64_t n_expert, int64_t n_used,
+                       int64_t B, char *buf, size_t buf_bytes);
 
 /* library build tag: "qproj-<version>-gfx950" */
 const char *qproj_version(void);

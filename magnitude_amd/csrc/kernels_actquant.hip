@@ -139,7 +139,10 @@ hipError_t launch_minterm_rows(int kind, const float *d, const int16_t *bsums, c
                                uint16_t *msum, float *rs, hipStream_t s) {
     if (M == 0) return hipSuccess;
     if (K % 256 != 0 || !msum || !rs || (kind != kActKindQ8_K && kind != kActKindQ8X32)) return hipErrorInvalidValue;
-    if (dry_run()) return hipSuccess;
+    if (dry_run()) {
+        plan_note("minterm_rows_kernel: min-term plane of %lld rows, grid %lld x 256", (long long)M, (long long)((M + 3) / 4));
+        return hipSuccess;
+    }
     const dim3 grid((unsigned)((M + 3) / 4)), block(256);
     if (kind == kActKindQ8_K)
         hipLaunchKernelGGL(minterm_rows_kernel<false>, grid, block, 0, s, d, bsums, isum, M, (int)(K / 256), msum, rs);
@@ -162,7 +165,13 @@ hipError_t launch_quantize_act(int kind, const float *x, int64_t M, int64_t K, i
         for (int i = 0; i < zj.count; ++i)
             if (zj.n[i] % 4 != 0 || (reinterpret_cast<uintptr_t>(zj.p[i]) & 15) != 0) return hipErrorInvalidValue;
     }
-    if (dry_run()) return hipSuccess;
+    if (dry_run()) {
+        plan_note("quantizer: %lld x %lld -> %s%s%s%s", (long long)M, (long long)K,
+                  kind == kActKindQ8_K ? "Q8_K" : kind == kActKindQ8_0 ? "Q8_0 blocks" : "per-32 int8",
+                  msum && rs ? " + min-term plane" : "", u ? ", rows = silu(x) * u" : "",
+                  zj.count ? ", clears the output rows of a projection that adds its two K parts" : "");
+        return hipSuccess;
+    }
     // with the min-term plane wanted: one launch, a workgroup per row (measured against the quantizer followed by
     // the min-term launch: 4.6 against 7.1 us at 128 x 4096, 9.3 against 10.6 at 512 x 14336; many short rows are
     // the exception, 22.8 against 18.8 us at 4096 x 4096, where a workgroup has one chunk a wave and two barriers)

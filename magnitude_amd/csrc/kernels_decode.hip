@@ -9,6 +9,7 @@
 // does a handful of operations per step and the vector unit only the dot products.
 #include "actquant_device.h"
 #include "gemv_frags.h"
+#include <stdio.h>
 
 namespace qproj {
 
@@ -379,7 +380,15 @@ hipError_t launch_decode(const GemvArgs &args, hipStream_t s) {
     const int kpad = (int)((K + CH - 1) / CH * CH);
     const size_t smem = (size_t)MT * kpad + (size_t)MT * (kpad / BLK) * 4 + (!is_q8_0<QT> ? (size_t)MT * (kpad / 16) * 2 : 0);
     if (PAIR) a.n_targets = 2;
-    if (dry_run()) return hipSuccess;
+    if (dry_run()) {
+        char rows[96] = "";
+        for (int i = 0, o = 0; i < (PAIR ? 1 : a.n_targets) && o < 80; ++i)
+            o += snprintf(rows + o, sizeof rows - o, "%s%lld rows/%d a wave pair", i ? ", " : "", (long long)a.t[i].w.N, a.t[i].rows_per_pair);
+        plan_note("gemv_decode_kernel<%s, %d activation rows, %d weight rows a step, activations in %s, %s%s>: grid %lld x %d, %s, LDS %zu B",
+                  plan_type_name(QT), MT, R, XREG ? "registers" : "LDS", FUSE ? "quantizer in the prologue" : "rows quantized earlier",
+                  PAIR ? ", gate/up paired + swiglu" : "", (long long)grid, kDecodeThreads, rows, smem);
+        return hipSuccess;
+    }
     auto kern = &gemv_decode_kernel<QT, MT, R, XREG, FUSE, PAIR>;
     if (smem > 48 * 1024) {
         static size_t allowed = 0;

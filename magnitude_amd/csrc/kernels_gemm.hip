@@ -893,7 +893,12 @@ hipError_t launch_per32(const WeightView &w, const ActView &a, int64_t M, float 
     if (w.K > (1 << 24)) return hipErrorInvalidValue;   // 32-bit lane offsets: 128 rows of K bytes
     const int n_split = sc.p ? per32_splits(w.K, M, w.N) : 1;
     if (n_split > 1 && (size_t)n_split * M * w.N * 4 > sc.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
-    if (dry_run()) return hipSuccess;
+    if (dry_run()) {
+        if (n_split > 1) plan_note_cut();
+        plan_note("gemm_per32_kernel<%s>: tile 128 tokens x 128 rows, %lld tiles x %d K stretches%s", plan_type_name(QT),
+                  (long long)(((w.N + BN - 1) / BN) * ((M + BM - 1) / BM)), n_split, n_split > 1 ? " + sum_parts_kernel" : "");
+        return hipSuccess;
+    }
     const auto kern = &gemm_per32_kernel<QT>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(GemmSmem));
@@ -909,7 +914,10 @@ hipError_t launch_per32(const WeightView &w, const ActView &a, int64_t M, float 
 }  // namespace
 
 hipError_t launch_sum_parts(const float *part, int n_split, size_t n, float *y, hipStream_t s) {
-    if (dry_run()) return hipSuccess;
+    if (dry_run()) {
+        plan_note("sum_parts_kernel: adds %d partial results of %zu outputs in order", n_split, n);
+        return hipSuccess;
+    }
     const size_t n4 = n / 4;   // callers only split when n is a multiple of 4
     hipLaunchKernelGGL(sum_parts_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, part, n_split, n4, y);
     return hipGetLastError();
@@ -1014,7 +1022,15 @@ hipError_t launch_gemm_q8k(const WeightView &w, const ActView &a, int64_t M, flo
     const bool add = zeroed && p.n_split == 2;   // both stretches add to the cleared rows: no partial tiles
     if (zeroed && !add) p = q4k_plan(w.K, M, w.N, scratch.p != nullptr);
     if (p.n_split > 1 && !add && (size_t)p.n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
-    if (dry_run()) return hipSuccess;
+    if (dry_run()) {
+        if (p.n_split > 1 && !add) plan_note_cut();
+        const long long tiles = p.wide ? (long long)(((w.N + 255) / 256) * ((M + 127) / 128)) : (long long)(((w.N + 127) / 128) * ((M + 63) / 64));
+        plan_note("%s: tile %s, %lld tiles x %d K stretches%s, partial tiles %zu B", p.wide ? "gemm_q4k_q8k_wide_kernel" : "gemm_q4k_q8k_direct_kernel",
+                  p.wide ? "128 tokens x 256 rows" : "64 tokens x 128 rows", tiles, p.n_split,
+                  p.n_split == 1 ? "" : add ? ", the two stretches add themselves to cleared rows" : " + sum_parts_kernel",
+                  p.n_split > 1 && !add ? (size_t)p.n_split * M * w.N * 4 : (size_t)0);
+        return hipSuccess;
+    }
     float *const part = add ? nullptr : scratch.p;
     if (p.wide) {   // 128 tokens x 256 weight rows per workgroup, one workgroup per compute unit
         using Smem = WideSmem<8>;
@@ -1089,7 +1105,16 @@ hipError_t launch_gemm_q8k_multi(int n, const WeightView *w, const ActView &a, i
         hipError_t e = launch_gemm_q8k(w[i], a, M, y[i], scratch.for_target(i), s);
         if (e != hipSuccess) return e;
     }
-    if (n_joined == 0 || dry_run()) return hipSuccess;
+    if (n_joined == 0) return hipSuccess;
+    if (dry_run()) {
+        long long wgs = 0;
+        for (int j = 0; j < n_joined; ++j) {
+            wgs += (long long)(((w[joined[j]].N + 32 * NW - 1) / (32 * NW)) * ((M + 63) / 64));
+            wgs = (wgs + 7) / 8 * 8;
+        }
+        plan_note("gemm_q4k_q8k_direct_kernel: %d matrices in one launch, tile 64 tokens x 128 rows, %lld workgroups, K whole", n_joined, wgs);
+        return hipSuccess;
+    }
     using Smem = DirectSmem<NW>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8k_direct_kernel<NW>),
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem));

@@ -460,7 +460,12 @@ __global__ __launch_bounds__(512, 1) void gemm_q6k_q8k_wide_kernel(const WeightV
 namespace {
 template <int NW, int JT>
 hipError_t launch_q6k(const WeightView &w, const ActView &a, int64_t M, float *y, float *scratch, int n_split, hipStream_t s) {
-    if (dry_run()) return hipSuccess;
+    if (dry_run()) {
+        if (n_split > 1) plan_note_cut();
+        plan_note("gemm_q6k_q8k_kernel<%d waves, %d token tiles>: tile %d tokens x %d rows, %lld tiles x %d K stretches%s", NW, JT, 32 * JT, 32 * NW,
+                  (long long)(((w.N + 32 * NW - 1) / (32 * NW)) * ((M + 32 * JT - 1) / (32 * JT))), n_split, n_split > 1 ? " + sum_parts_kernel" : "");
+        return hipSuccess;
+    }
     using Smem = Q6Smem<NW, JT>;
     const auto kern = &gemm_q6k_q8k_kernel<NW, JT>;
     static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
@@ -523,7 +528,13 @@ hipError_t launch_gemm_q6k_q8k(const WeightView &w, const ActView &a, int64_t M,
     const Q6Plan p = q6k_plan(w.K, M, w.N, scratch.p != nullptr);
     if (p.n_split > 1 && (size_t)p.n_split * M * w.N * 4 > scratch.bytes) return hipErrorInvalidValue;   // partial tiles would not fit
     if (p.wide) {
-        if (dry_run()) return hipSuccess;
+        if (dry_run()) {
+            if (p.n_split > 1) plan_note_cut();
+            plan_note("gemm_q6k_q8k_wide_kernel: tile 128 tokens x 256 rows, %lld tiles x %d K stretches%s, partial tiles %zu B",
+                      (long long)(((w.N + 255) / 256) * ((M + 127) / 128)), p.n_split, p.n_split > 1 ? " + sum_parts_kernel" : "",
+                      p.n_split > 1 ? (size_t)p.n_split * M * w.N * 4 : (size_t)0);
+            return hipSuccess;
+        }
         static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q6k_q8k_wide_kernel),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Q6WideSmem));
         if (attr != hipSuccess) return attr;

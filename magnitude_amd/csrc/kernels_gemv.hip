@@ -200,7 +200,12 @@ hipError_t launch_one(const GemvArgs &args, int n_experts_grid, hipStream_t s) {
         a.t[i].first_block = total_blocks;
         total_blocks += (int)((a.t[i].w.N + 4 * R - 1) / (4 * R));
     }
-    if (total_blocks == 0 || dry_run()) return hipSuccess;
+    if (total_blocks == 0) return hipSuccess;
+    if (dry_run()) {
+        plan_note("gemv_q8act_kernel<%s, %d rows, %d weight rows a wave%s%s>: grid %d x %d", plan_type_name(QT), MT, R, GROUPED ? ", expert-grouped" : "",
+                  SWIGLU ? ", swiglu" : "", total_blocks, GROUPED ? n_experts_grid : 1);
+        return hipSuccess;
+    }
     const dim3 grid((unsigned)total_blocks, (unsigned)(GROUPED ? n_experts_grid : 1));
     constexpr size_t smem = gemv_smem_bytes(QT, MT);
     if (smem > 48 * 1024) {  // above the default dynamic-LDS allowance: opt in once per kernel

@@ -199,7 +199,11 @@ hipError_t launch_f32(const GemvArgs &args, hipStream_t s) {
         a.t[i].first_block = total;
         total += (int)((a.t[i].w.N + 4 * R - 1) / (4 * R));
     }
-    if (total == 0 || dry_run()) return hipSuccess;
+    if (total == 0) return hipSuccess;
+    if (dry_run()) {
+        plan_note("gemv_f32_kernel<%s, %d rows>: fp32 activations x dequantized weights, grid %d x 256", plan_type_name(QT), MT, total);
+        return hipSuccess;
+    }
     hipLaunchKernelGGL((gemv_f32_kernel<QT, MT, R>), dim3((unsigned)total), dim3(256), (size_t)MT * tile_kf(MT) * 4, s, a);
     return hipGetLastError();
 }

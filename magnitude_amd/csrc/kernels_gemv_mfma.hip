@@ -905,7 +905,15 @@ hipError_t launch_one(const MfmaArgs &g, hipStream_t s) {
     }
     // K parts of a row group are summed through the waves' regions: a wave's partial tile must fit its region
     if (g.kw > 1 && (MODE == kGroupedSwiglu ? 2 : 1) * (8 * NI) * 32 * 4 > Cfg<QT>::kRegion) return hipErrorInvalidValue;
-    if (dry_run()) return hipSuccess;
+    if (dry_run()) {
+        if (g.n_chunks > 1 && !g.add_out) plan_note_cut();
+        plan_note("gemv_mfma_kernel<%s, %d staged rows, %d waves, %s%s>: %d workgroups, K in %d chunk(s) of %d super-blocks x %d parts a row group%s",
+                  plan_type_name(QT), 8 * NI, W, MODE == kDense ? "dense" : MODE == kGroupedSwiglu ? "expert-grouped + swiglu" : "expert-grouped",
+                  FLAT ? ", one item stream a wave" : "", g.n_wgs, g.n_chunks, g.chunk_sb, g.kw,
+                  g.n_chunks == 1 ? "" : g.add_out ? ", the two chunks add themselves to cleared rows"
+                                   : MODE == kDense ? " + sum_chunks_kernel" : " + sum_parts_kernel");
+        return hipSuccess;
+    }
     const Layout L = layout<QT, 8 * NI, W>(g.chunk_sb);
     auto kern = gemv_mfma_kernel<QT, NI, W, MODE, FLAT>;
     static int allowed = 0;

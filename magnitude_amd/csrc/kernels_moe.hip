@@ -248,6 +248,12 @@ hipError_t launch_moe_group(const int32_t *ids, int64_t n_pairs, int64_t n_exper
     const size_t table = (size_t)((n_pairs + 63) / 64) * (size_t)n_expert;
     const bool by_block = n_pairs <= 64 * 16 * kBlocksPerWave && table <= 24 * 1024;   // at most 96 KB of LDS
     const size_t lds = ((size_t)n_expert + 48 + (by_block ? table : n_pairs <= kGroupLdsIds ? (size_t)n_pairs : 0)) * sizeof(int32_t);
+    if (dry_run()) {
+        plan_note("moe_group_kernel: %lld pairs over %lld experts (%s)%s", (long long)n_pairs, (long long)n_expert,
+                  by_block ? "ballot per bit of the id, prefix over 64-pair blocks" : "ballot sweeps per expert",
+                  quantize ? ", spare workgroups quantize the token rows" : "");
+        return hipSuccess;
+    }
     static size_t allowed = 48 * 1024;
     if (lds > allowed) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(moe_group_kernel),
@@ -289,7 +295,11 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const float *__restrict__ g
 }
 
 hipError_t launch_swiglu(const float *g, const float *u, size_t n, float *h, hipStream_t s) {
-    if (n == 0 || dry_run()) return hipSuccess;
+    if (n == 0) return hipSuccess;
+    if (dry_run()) {
+        plan_note("swiglu_kernel: %zu elements", n);
+        return hipSuccess;
+    }
     hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, g, u, n, h);
     return hipGetLastError();
 }
@@ -298,6 +308,10 @@ hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, i
                               float *y, hipStream_t s) {
     const int64_t n = B * N;
     if (n == 0) return hipSuccess;
+    if (dry_run()) {
+        plan_note("moe_combine_kernel: %lld tokens x %lld, %lld experts a token in slot order", (long long)B, (long long)N, (long long)n_used);
+        return hipSuccess;
+    }
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, e, weights, B,
                        (int)n_used, N, y);
     return hipGetLastError();

@@ -282,10 +282,14 @@ size_t staged_bytes(int64_t K, int64_t group) {
 }
 }  // namespace
 
-bool moe_decode_fits(int type, int64_t K, int64_t n_pairs, int64_t group) {
+// Every condition on the SHAPE that launch_moe_decode refuses a call for (the dispatch asks this before it picks the
+// route, the launcher asserts the same predicate: one rule, so a shape the launcher would turn down never reaches it
+// and takes the grouped route instead).  With it the launcher's LDS never exceeds the budget: the staged rows leave
+// room for 64 result rows a pair, and the results a workgroup keeps are cut to what is left.
+bool moe_decode_fits(int type, int64_t K, int64_t N, int64_t n_pairs, int64_t group, int64_t n_expert) {
     return (type == kTypeQ4_K || type == kTypeQ6_K) && K % 256 == 0 && K >= 256 && K <= (1 << 20) && n_pairs >= 1 &&
-           n_pairs <= (1 << 20) && group >= 1 && group <= kMaxGroup && n_pairs % group == 0 &&
-           staged_bytes(K, group) + (size_t)group * 4 * 64 + 64 <= kLdsBudget;   // room for 64 result rows a pair at least
+           n_pairs <= (1 << 20) && group >= 1 && group <= kMaxGroup && n_pairs % group == 0 && N >= 1 && N <= (1 << 24) &&
+           n_expert >= 1 && staged_bytes(K, group) + (size_t)group * 4 * 64 + 64 <= kLdsBudget;
 }
 
 // args: t[0] (and t[1] = up when swiglu) expert stacks, x fp32 rows, x_div, ids, n_pairs, error_flag as for the
@@ -329,8 +333,8 @@ hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, co
         }
     }
     const bool x_shared = !combine_weights && group > 1;
-    if (!moe_decode_fits(w.type, w.K, args.n_pairs, x_shared ? 1 : group) || args.n_pairs % group != 0 || !args.x || !args.ids ||
-        !args.error_flag || n_expert < 1 || w.N < 1 || w.N > (1 << 24) || (swiglu && combine_weights))
+    if (!moe_decode_fits(w.type, w.K, w.N, args.n_pairs, x_shared ? 1 : group, n_expert) || args.n_pairs % group != 0 || !args.x ||
+        !args.ids || !args.error_flag || (swiglu && combine_weights))
         return hipErrorInvalidValue;
     if (swiglu && (args.n_targets != 2 || args.t[1].w.type != w.type || args.t[1].w.K != w.K || args.t[1].w.N != w.N))
         return hipErrorInvalidValue;
@@ -359,8 +363,13 @@ hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, co
     g.rows_per_wg = (int)(steps_per_wg * S);
     g.wgs_per_group = (int)((w.N + g.rows_per_wg - 1) / g.rows_per_wg);
     const size_t lds = staged + (combine_weights ? (size_t)group * (g.rows_per_wg + 1) * 4 : 0);
-    if (lds > 160 * 1024) return hipErrorInvalidValue;
-    if (dry_run()) return hipSuccess;
+    if (lds > 160 * 1024) return hipErrorInvalidValue;   // (cannot happen for a shape moe_decode_fits accepts; kept as a guard)
+    if (dry_run()) {
+        plan_note("moe_decode_kernel<%s%s%s>: an expert read per pair, %d pairs, %d pairs share a workgroup set%s, %d workgroups, LDS %zu B",
+                  plan_type_name(w.type), swiglu ? ", gate/up + swiglu" : "", combine_weights ? ", weighted sum over a token's experts" : "",
+                  args.n_pairs, group, x_shared ? " (one staged token row)" : "", n_groups * g.wgs_per_group, lds);
+        return hipSuccess;
+    }
     const unsigned grid = (unsigned)(n_groups * g.wgs_per_group);
     // two row steps a unit where a wave would otherwise walk four or more units of rows that fill under 4 KB a step
     static const int two_env = tuning_int("QPROJ_MOE_DECODE_TWO_STEPS", -1);

@@ -102,7 +102,12 @@ hipError_t launch_rms_norm(int kind, const float *x, const float *gamma, float e
     if (K <= 0 || K % 32 != 0) return hipErrorInvalidValue;
     if ((kind == kActKindQ8_K || kind == kActKindQ8X32) && K % 256 != 0) return hipErrorInvalidValue;
     if (kind >= 0 && kind != kActKindQ8_K && kind != kActKindQ8_0 && kind != kActKindQ8X32) return hipErrorInvalidValue;
-    if (dry_run()) return hipSuccess;
+    if (dry_run()) {
+        plan_note("rms_norm_kernel: %lld x %lld -> %s%s, grid %lld x %d", (long long)M, (long long)K,
+                  kind < 0 ? "fp32 rows" : kind == kActKindQ8_K ? "Q8_K" : kind == kActKindQ8_0 ? "Q8_0 blocks" : "per-32 int8",
+                  msum && rs ? " + min-term plane" : "", (long long)M, kNormThreads);
+        return hipSuccess;
+    }
     const dim3 grid((unsigned)M), block(kNormThreads);
     const bool mt = msum && rs && (kind == kActKindQ8_K || kind == kActKindQ8X32) &&
                     row_minterm_lds_bytes(kind == kActKindQ8X32, (int)(K / 256)) <= kRowLdsMax;

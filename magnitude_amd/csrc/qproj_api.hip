@@ -2,11 +2,13 @@
 #include "../../include/qproj.h"
 
 #include <dlfcn.h>
+#include <stdarg.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
+#include <mutex>
 #include <new>
 #include <string>
 
@@ -17,9 +19,29 @@ using namespace qproj;
 namespace qproj {
 namespace {
 thread_local bool g_dry_run = false;
+thread_local size_t g_scratch_shave = 0;    // dry runs only: bytes withheld from what the launchers are told they have
+thread_local int g_plan_cuts = 0;           // dry runs only: launches noted that cut K into parts kept in scratch
+thread_local std::string *g_plan = nullptr;   // where plan_note writes; null: nobody is listening
 }
 bool dry_run() { return g_dry_run; }
+size_t scratch_shave() { return g_dry_run ? g_scratch_shave : 0; }
 void set_dry_run(bool on) { g_dry_run = on; }
+
+void plan_note_cut() { ++g_plan_cuts; }
+
+void plan_note(const char *fmt, ...) {
+    if (!g_plan) return;
+    char line[384];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(line, sizeof line, fmt, ap);
+    va_end(ap);
+    g_plan->append(line);
+    g_plan->push_back('\n');
+}
+const char *plan_type_name(int type) {
+    return type == kTypeQ4_K ? "Q4_K" : type == kTypeQ6_K ? "Q6_K" : type == kTypeQ8_0 || type == 1008 ? "Q8_0" : "?";
+}
 
 int tuning_int(const char *name, int dflt) {
 #ifdef QPROJ_TUNING
@@ -40,7 +62,12 @@ static __device__ __align__(256) unsigned char scratch[QPROJ_NOALLOC_SCRATCH_BYT
 
 namespace {
 constexpr int kMaxDevices = 64;
+std::mutex g_noalloc_mu;                    // guards the two tables below
 uint8_t *g_noalloc_ptr[kMaxDevices] = {};   // device address of `scratch` on each device, null until looked up
+// The context that uses a device's fixed scratch: the first one to call the allocation-free entry point on the device,
+// until it is destroyed.  Two contexts launch on two streams, and their calls would overwrite each other's activation
+// planes and partial tiles in the one buffer with no error anywhere; a second context is refused instead.
+qproj_ctx *g_noalloc_owner[kMaxDevices] = {};
 }  // namespace
 
 struct qproj_ctx {
@@ -122,6 +149,7 @@ int reserve(qproj_ctx *ctx, Workspace &ws, size_t bytes) {
     if (dry_run() && !ws.fixed) {   // sizes only: any non-null base will do, nothing is dereferenced
         ws.base = reinterpret_cast<uint8_t *>(uintptr_t(256));
         ws.cap = bytes;
+        if (ctx) ctx->ws_bytes = std::max(ctx->ws_bytes, bytes);   // (a stand-in context: what the call would have asked for)
         return QPROJ_OK;
     }
     if (ws.fixed) {
@@ -423,7 +451,15 @@ bool dense_fuses_quantizer(const qproj_weight *w, int64_t M) {
 // The quantizer launch in front of the small-batch kernel clears the output rows where a pass of that kernel cuts K
 // in two chunks: the chunks then add themselves to the output and the launch that summed them goes (8B down
 // projection, 14336 -> 4096 Q6_K, at 4 and 8 rows).  Fills `z` and answers true when that is the case.
-bool dense_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *const *y, ZeroJob &z) {
+// true when [a, a + na) and [b, b + nb) (floats) share an address
+bool overlaps(const float *a, int64_t na, const float *b, int64_t nb) {
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), a1 = a0 + (uintptr_t)na * 4, b0 = reinterpret_cast<uintptr_t>(b), b1 = b0 + (uintptr_t)nb * 4;
+    return a0 < b1 && b0 < a1;
+}
+
+// (x: the rows the quantizer launch reads, M x K floats.  Output rows that overlap them cannot be cleared by that launch -
+// some workgroups would zero what others have yet to read - so such a call keeps the route that stores.)
+bool dense_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *const *y, const float *x, ZeroJob &z) {
     if (takes_tiled(w[0], M) || !use_mfma_kernel(w[0]->type, M, w[0]->K)) return false;
     int64_t rgs = 0;
     for (int i = 0; i < n; ++i) rgs += (w[i]->N + 31) / 32;
@@ -436,6 +472,7 @@ bool dense_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *co
         z.p[i] = y[i];
         z.n[i] = M * w[i]->N;
         if (z.n[i] % 4 != 0 || (reinterpret_cast<uintptr_t>(y[i]) & 15) != 0) return false;
+        if (overlaps(y[i], z.n[i], x, M * w[0]->K)) return false;
     }
     return true;
 }
@@ -443,7 +480,7 @@ bool dense_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *co
 // The same for the tiled Q4_K kernels: the matrices of the call whose launch cuts K in exactly two stretches get their
 // output rows cleared by the quantizer launch, and the stretches add themselves (no partial tiles, no adding pass).
 // Returns the mask of those matrices and fills `z` with their rows.
-uint32_t tiled_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *const *y, bool have_scratch, ZeroJob &z) {
+uint32_t tiled_clears_rows(int n, const qproj_weight *const *w, int64_t M, float *const *y, const float *x, bool have_scratch, ZeroJob &z) {
     WeightView views[kMaxTargets];
     for (int i = 0; i < n; ++i) views[i] = w[i]->view;
     uint32_t mask = q4k_multi_adds(n, views, M, have_scratch);
@@ -451,7 +488,7 @@ uint32_t tiled_clears_rows(int n, const qproj_weight *const *w, int64_t M, float
     for (int i = 0; i < n; ++i) {
         if (!((mask >> i) & 1u)) continue;
         const int64_t cnt = M * w[i]->N;
-        if (cnt % 4 != 0 || (reinterpret_cast<uintptr_t>(y[i]) & 15) != 0) {
+        if (cnt % 4 != 0 || (reinterpret_cast<uintptr_t>(y[i]) & 15) != 0 || overlaps(y[i], cnt, x, M * w[0]->K)) {
             mask &= ~(1u << i);
             continue;
         }
@@ -565,7 +602,7 @@ bool moe_decode_route(int type, int64_t K, int64_t N, int64_t n_pairs, int64_t g
     const bool small_expert = K * N <= ((int64_t)2 << 20);
     const bool few = n_pairs <= 16 && small_expert;
     const int64_t per4 = per_4_experts + (small_expert ? per_4_experts / 2 : 0);
-    return on && (few || (n_pairs <= max_pairs && 4 * n_pairs <= per4 * E)) && moe_decode_fits(type, K, n_pairs, group);
+    return on && (few || (n_pairs <= max_pairs && 4 * n_pairs <= per4 * E)) && moe_decode_fits(type, K, N, n_pairs, group, E);
 }
 
 // Expert rows too long for the staged rows of the grouped matrix-core kernel (K > 4096): from `min_mt` pairs an expert
@@ -692,15 +729,18 @@ int qproj_ctx_create(int device, void *stream, qproj_ctx **out) {
         ctx->own_stream = true;
     }
     // the fixed scratch of the allocation-free entry point: each device holds its own copy at its own address
-    if (device < kMaxDevices && !g_noalloc_ptr[device]) {
-        void *ptr = nullptr;
-        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
-            (void)hipGetLastError();
-            if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
-            delete ctx;
-            return QPROJ_ERR_HIP;
+    if (device < kMaxDevices) {
+        std::lock_guard<std::mutex> lock(g_noalloc_mu);
+        if (!g_noalloc_ptr[device]) {
+            void *ptr = nullptr;
+            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+                (void)hipGetLastError();
+                if (ctx->own_stream) (void)hipStreamDestroy(ctx->stream);
+                delete ctx;
+                return QPROJ_ERR_HIP;
+            }
+            g_noalloc_ptr[device] = static_cast<uint8_t *>(ptr);
         }
-        g_noalloc_ptr[device] = static_cast<uint8_t *>(ptr);
     }
     if (hipMalloc((void **)&ctx->flag_dev, 256) != hipSuccess ||
         hipMemsetAsync(ctx->flag_dev, 0, 256, ctx->stream) != hipSuccess ||
@@ -717,6 +757,10 @@ int qproj_ctx_destroy(qproj_ctx *ctx) {
     if (!ctx) return QPROJ_OK;
     (void)hipSetDevice(ctx->device);
     (void)hipStreamSynchronize(ctx->stream);
+    if (ctx->device >= 0 && ctx->device < kMaxDevices) {   // the device's fixed scratch is free for another context again
+        std::lock_guard<std::mutex> lock(g_noalloc_mu);
+        if (g_noalloc_owner[ctx->device] == ctx) g_noalloc_owner[ctx->device] = nullptr;
+    }
     if (ctx->ws) (void)hipFree(ctx->ws);
     if (ctx->ws2) (void)hipFree(ctx->ws2);
     if (ctx->flag_dev) (void)hipFree(ctx->flag_dev);
@@ -926,7 +970,7 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
             ActView a{};
             a.kind = act_kind_for(act, w[0]->type);
             a.K = K;
-            return run_dense_q8act(ctx, n, w, a, M, y_dev, Scratch{reinterpret_cast<float *>(wsp.base), extra}, x_dev);
+            return run_dense_q8act(ctx, n, w, a, M, y_dev, Scratch{reinterpret_cast<float *>(wsp.base), extra - std::min(extra, scratch_shave())}, x_dev);
         }
         const ActPlanes p = act_planes(act_kind_for(act, w[0]->type), M, K);
         const size_t extra = act == kActGGML ? dense_scratch_bytes(n, w, M) : per32_scratch_max(n, w, M);
@@ -948,14 +992,14 @@ static int mul_mat_multi_impl(qproj_ctx *ctx, int n, const qproj_weight *const *
                                         reinterpret_cast<int32_t *>(ws + p.off_aux),
                                         minterm ? reinterpret_cast<float *>(ws + p.off_rs) : nullptr, ctx->stream));
         } else {
-            y_zeroed = act == kActGGML && !minterm && dense_clears_rows(n, w, M, y_dev, zero);
+            y_zeroed = act == kActGGML && !minterm && dense_clears_rows(n, w, M, y_dev, x_dev, zero);
             if (act == kActGGML && w[0]->type == kTypeQ4_K && takes_tiled(w[0], M))
-                tile_adds = tiled_clears_rows(n, w, M, y_dev, extra > 0, zero);
+                tile_adds = tiled_clears_rows(n, w, M, y_dev, x_dev, extra > 0, zero);
             QP_HIP(ctx, run_quantize(ctx, p, ws, x_dev, M, K, minterm, swiglu_u, y_zeroed || tile_adds ? &zero : nullptr));
         }
         const ActView a = act_view(p, ws, K);
         // the partial results lie behind the activation planes; `extra` is all a launcher may use of it
-        const Scratch sc{extra ? reinterpret_cast<float *>(ws + p.total) : nullptr, extra, tile_adds};
+        const Scratch sc{extra ? reinterpret_cast<float *>(ws + p.total) : nullptr, extra - std::min(extra, scratch_shave()), tile_adds};
         if (act == kActGGML) return run_dense_q8act(ctx, n, w, a, M, y_dev, sc, nullptr, y_zeroed);
         for (int i = 0; i < n; ++i) QP_HIP(ctx, launch_gemm_q8x32(w[i]->view, a, M, y_dev[i], sc, ctx->stream));
         return QPROJ_OK;
@@ -997,9 +1041,21 @@ int qproj_mul_mat_multi(qproj_ctx *ctx, int n, const qproj_weight *const *w, con
 int qproj_mul_mat_multi_noalloc(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, int64_t M,
                                 float *const *y_dev, int act) {
     if (!ctx) return QPROJ_ERR_INVALID_ARG;
-    if (ctx->device < 0 || ctx->device >= kMaxDevices || !g_noalloc_ptr[ctx->device])
+    uint8_t *fixed = nullptr;
+    if (ctx->device >= 0 && ctx->device < kMaxDevices) {
+        std::lock_guard<std::mutex> lock(g_noalloc_mu);
+        fixed = g_noalloc_ptr[ctx->device];
+        if (fixed) {
+            if (!g_noalloc_owner[ctx->device]) g_noalloc_owner[ctx->device] = ctx;
+            if (g_noalloc_owner[ctx->device] != ctx)
+                return fail(ctx, QPROJ_ERR_UNSUPPORTED,
+                            "qproj_mul_mat_multi_noalloc: the fixed scratch of this GPU is in use by another context "
+                            "(calls from two contexts would overwrite each other's scratch)");
+        }
+    }
+    if (!fixed)
         return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat_multi_noalloc: the fixed scratch was not set up for this device");
-    Workspace wsp{g_noalloc_ptr[ctx->device], (size_t)QPROJ_NOALLOC_SCRATCH_BYTES, true};
+    Workspace wsp{fixed, (size_t)QPROJ_NOALLOC_SCRATCH_BYTES, true};
     return mul_mat_multi_impl(ctx, n, w, x_dev, M, y_dev, act, nullptr, wsp);
 }
 
@@ -1022,7 +1078,7 @@ size_t qproj_workspace_bytes(int type, int64_t K, int n, const int64_t *N, int64
         ws[i].dev = reinterpret_cast<uint8_t *>(uintptr_t(256));
         make_view(&ws[i]);
         wp[i] = &ws[i];
-        yp[i] = reinterpret_cast<float *>(uintptr_t(256));
+        yp[i] = reinterpret_cast<float *>((uintptr_t(1) << 40) + (uintptr_t(i) << 36));   // stand-ins, apart from x and from each other
     }
     const float *fake_x = reinterpret_cast<const float *>(uintptr_t(256));
     set_dry_run(true);
@@ -1033,13 +1089,102 @@ size_t qproj_workspace_bytes(int type, int64_t K, int n, const int64_t *N, int64
         Workspace exact{reinterpret_cast<uint8_t *>(uintptr_t(256)), total, true};
         rc = mul_mat_multi_impl(&ctx, n, wp, fake_x, M, yp, act, nullptr, exact);
     }
-    if (rc == QPROJ_OK && total > 0) {   // ... and one byte less must be refused, not overrun
+    if (rc == QPROJ_OK && total > 0) {   // ... one byte less must be refused by the reservation ...
         Workspace less{reinterpret_cast<uint8_t *>(uintptr_t(256)), total - 1, true};
         if (mul_mat_multi_impl(&ctx, n, wp, fake_x, M, yp, act, nullptr, less) == QPROJ_OK) rc = QPROJ_ERR_HIP;
+    }
+    if (rc == QPROJ_OK && act == kActGGML && dense_scratch_bytes(n, wp, M) > 0) {
+        // ... and the launchers' own capacity checks are exercised too: the reservation succeeds, but every launcher is
+        // told it has NO scratch beyond the activation planes (and no cleared output rows to add into).  A launcher
+        // that cuts K must then refuse; the only calls that may still pass are those whose launchers need none (the
+        // reservation is an upper bound: matrices that ride in one launch with K whole use none of it).
+        Workspace exact{reinterpret_cast<uint8_t *>(uintptr_t(256)), total, true};
+        float *odd[kMaxTargets];   // misaligned outputs: no route that adds into cleared rows instead of using scratch
+        for (int i = 0; i < n; ++i) odd[i] = reinterpret_cast<float *>(uintptr_t(260));
+        g_plan_cuts = 0;
+        g_scratch_shave = ~(size_t)0;
+        const int starved = mul_mat_multi_impl(&ctx, n, wp, fake_x, M, odd, act, nullptr, exact);
+        g_scratch_shave = 0;
+        if (starved == QPROJ_OK && g_plan_cuts > 0) rc = QPROJ_ERR_HIP;   // a K cut went through without scratch
     }
     set_dry_run(false);
     if (status) *status = rc;
     return rc == QPROJ_OK ? total : 0;
+}
+
+// The routing table: the launches a call of this shape makes, one line each, written by the launchers themselves
+// during a dry run of the dispatch code that serves the call (nothing touches a device).
+namespace {
+int finish_plan(const std::string &text, int rc, size_t scratch, char *buf, size_t buf_bytes) {
+    std::string out = text;
+    char tail[96];
+    snprintf(tail, sizeof tail, "scratch: %zu bytes\n", scratch);
+    out += tail;
+    if (rc != QPROJ_OK) out += "(the call is refused with status " + std::to_string(rc) + ")\n";
+    if (!buf || buf_bytes == 0) return QPROJ_ERR_INVALID_ARG;
+    const size_t n = std::min(out.size(), buf_bytes - 1);
+    memcpy(buf, out.data(), n);
+    buf[n] = 0;
+    return out.size() < buf_bytes ? rc : QPROJ_ERR_INVALID_ARG;
+}
+void fake_weight(qproj_weight &w, int type, int64_t K, int64_t N, int64_t E) {
+    w.type = type;
+    w.K = K;
+    w.N = N;
+    w.E = E;
+    w.dev = reinterpret_cast<uint8_t *>(uintptr_t(256));
+    make_view(&w);
+}
+}  // namespace
+
+int qproj_plan_mul_mat(int type, int64_t K, int n, const int64_t *N, int64_t M, int act, int with_norm, char *buf, size_t buf_bytes) {
+    if (!type_ok(type) || n <= 0 || n > kMaxTargets || !N || M < 0 || K <= 0 || K % block_elems(type) != 0) return QPROJ_ERR_INVALID_ARG;
+    qproj_ctx ctx;
+    qproj_weight ws[kMaxTargets];
+    const qproj_weight *wp[kMaxTargets];
+    float *yp[kMaxTargets];
+    for (int i = 0; i < n; ++i) {
+        if (N[i] <= 0) return QPROJ_ERR_INVALID_ARG;
+        fake_weight(ws[i], type, K, N[i], 1);
+        wp[i] = &ws[i];
+        yp[i] = reinterpret_cast<float *>((uintptr_t(1) << 40) + (uintptr_t(i) << 36));   // stand-ins, apart from x and from each other
+    }
+    const float *fake_x = reinterpret_cast<const float *>(uintptr_t(256));
+    const NormSpec norm{fake_x, 1e-5f};
+    std::string text;
+    set_dry_run(true);
+    g_plan = &text;
+    Workspace sized{nullptr, 0, false};
+    const int rc = mul_mat_multi_impl(&ctx, n, wp, fake_x, M, yp, act, with_norm ? &norm : nullptr, sized);
+    g_plan = nullptr;
+    set_dry_run(false);
+    return finish_plan(text, rc, sized.reserved, buf, buf_bytes);
+}
+
+int qproj_plan_moe_ffn(int gate_type, int down_type, int64_t d_model, int64_t d_ff, int64_t n_expert, int64_t n_used, int64_t B,
+                       char *buf, size_t buf_bytes) {
+    if (!type_ok(gate_type) || !type_ok(down_type) || d_model <= 0 || d_ff <= 0 || n_expert <= 0 || n_used <= 0 || B < 0 ||
+        d_model % block_elems(gate_type) != 0 || d_ff % block_elems(down_type) != 0)
+        return QPROJ_ERR_INVALID_ARG;
+    qproj_ctx ctx;
+    qproj_weight gate, up, down;
+    fake_weight(gate, gate_type, d_model, d_ff, n_expert);
+    fake_weight(up, gate_type, d_model, d_ff, n_expert);
+    fake_weight(down, down_type, d_ff, d_model, n_expert);
+    const float *fx = reinterpret_cast<const float *>(uintptr_t(256));
+    std::string text;
+    set_dry_run(true);
+    g_plan = &text;
+    ctx.ws_bytes = 0;
+    ctx.flag_dev = reinterpret_cast<int32_t *>(uintptr_t(256));   // never dereferenced in a dry run
+    const int rc = qproj_moe_ffn(&ctx, &gate, &up, &down, fx, reinterpret_cast<const int32_t *>(uintptr_t(256)), fx, n_used, B,
+                                 reinterpret_cast<float *>(uintptr_t(256)), kActGGML);
+    g_plan = nullptr;
+    set_dry_run(false);
+    const size_t scratch_bytes = ctx.ws_bytes;
+    ctx.ws_bytes = 0;
+    ctx.flag_dev = nullptr;
+    return finish_plan(text, rc, scratch_bytes, buf, buf_bytes);
 }
 
 int qproj_rms_norm_mul_mat(qproj_ctx *ctx, int n, const qproj_weight *const *w, const float *x_dev, const float *gamma_dev,
@@ -1178,7 +1323,7 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
         return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_mul_mat_id: nb1 must be 1 or n_used");
     if (act != kActGGML) return fail(ctx, QPROJ_ERR_UNSUPPORTED, "qproj_mul_mat_id: only the ggml activation mode");
     if (B == 0) return QPROJ_OK;
-    QP_HIP(ctx, hipSetDevice(ctx->device));
+    if (!dry_run()) QP_HIP(ctx, hipSetDevice(ctx->device));
     const int64_t K = w->K, n_pairs = B * n_used, rows = B * nb1;
     if (moe_decode_route(w->type, K, w->N, n_pairs, 1, w->E)) {
         GemvArgs g{};
@@ -1201,18 +1346,19 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
     const bool long_rows = grouped_long_rows(w, n_pairs);
     const size_t parts_bytes = long_rows ? mfma_grouped_scratch_bytes(K, w->N, n_pairs, w->E) : 0;
     const size_t total = off_parts + align_up(parts_bytes);
-    int rc = ensure_ws(ctx, total);
+    Workspace wsp = ctx_workspace(ctx);
+    int rc = reserve(ctx, wsp, total);
     if (rc) return rc;
     // few pairs an expert: the grouped kernel quantizes the rows it needs in its prologue
     const bool fuse = grouped_fuses_quantizer(w->type, K, n_pairs, w->E);
-    int32_t *order = reinterpret_cast<int32_t *>(ctx->ws + off_order);
-    int32_t *offsets = reinterpret_cast<int32_t *>(ctx->ws + off_offsets);
-    int32_t *active = reinterpret_cast<int32_t *>(ctx->ws + off_active);
+    int32_t *order = reinterpret_cast<int32_t *>(wsp.base + off_order);
+    int32_t *offsets = reinterpret_cast<int32_t *>(wsp.base + off_offsets);
+    int32_t *active = reinterpret_cast<int32_t *>(wsp.base + off_active);
     const bool pair_mode = grouped_pair_mode(w->type, K, n_pairs, w->E);
     // the quantizer and the grouping pass read only the call's inputs: one launch carries both
     const bool joined = !fuse && !pair_mode && p.kind == kActKindQ8_K;
-    const RowQuantJob job = quantize_job(p, ctx->ws, x_dev, rows, K);
-    if (!fuse && !joined) QP_HIP(ctx, run_quantize(ctx, p, ctx->ws, x_dev, rows, K, false));
+    const RowQuantJob job = quantize_job(p, wsp.base, x_dev, rows, K);
+    if (!fuse && !joined) QP_HIP(ctx, run_quantize(ctx, p, wsp.base, x_dev, rows, K, false));
     if (!pair_mode)
         QP_HIP(ctx, launch_moe_group(ids_dev, n_pairs, w->E, order, offsets, active, ctx->flag_dev,
                                      joined ? &job : nullptr, ctx->stream));
@@ -1225,7 +1371,7 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
         g.n_pairs = (int)n_pairs;
         g.error_flag = ctx->flag_dev;
     }
-    g.a = act_view(p, ctx->ws, K);
+    g.a = act_view(p, wsp.base, K);
     g.x = fuse ? x_dev : nullptr;
     g.order = order;
     g.offsets = offsets;
@@ -1235,7 +1381,7 @@ int qproj_mul_mat_id(qproj_ctx *ctx, const qproj_weight *w, const float *x_dev, 
         QP_HIP(ctx, launch_gemv_mfma_grouped(g, n_pairs, false, ctx->stream));
     else if (long_rows)
         QP_HIP(ctx, launch_gemv_mfma_grouped(g, n_pairs, false, ctx->stream,
-                                             Scratch{reinterpret_cast<float *>(ctx->ws + off_parts), parts_bytes}));
+                                             Scratch{reinterpret_cast<float *>(wsp.base + off_parts), parts_bytes}));
     else
         QP_HIP(ctx, launch_gemv_q8act(g, grouped_mt(n_pairs, w->E), (int)w->E, ctx->stream));
     return QPROJ_OK;
@@ -1255,7 +1401,7 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     if (d_ff % block_elems(down->type) != 0 || (down->type != kTypeQ8_0 && d_ff % 256 != 0))
         return fail(ctx, QPROJ_ERR_INVALID_ARG, "qproj_moe_ffn: d_ff must be a multiple of the block size");
     if (B == 0) return QPROJ_OK;
-    QP_HIP(ctx, hipSetDevice(ctx->device));
+    if (!dry_run()) QP_HIP(ctx, hipSetDevice(ctx->device));
     const int64_t n_pairs = B * n_used;
     const ActPlanes px = act_planes(act_kind_for(act, gate->type), B, d_model);
     const ActPlanes ph = act_planes(act_kind_for(act, down->type), n_pairs, d_ff);
@@ -1281,9 +1427,10 @@ int qproj_moe_ffn(qproj_ctx *ctx, const qproj_weight *gate, const qproj_weight *
     off += align_up(parts_bytes);
     const size_t off_h2 = off;
     if (long_gate) off += align_up((size_t)(n_pairs * d_ff) * 4);
-    int rc = ensure_ws(ctx, off);
+    Workspace wsp = ctx_workspace(ctx);
+    int rc = reserve(ctx, wsp, off);
     if (rc) return rc;
-    uint8_t *ws = ctx->ws;
+    uint8_t *ws = wsp.base;
     int32_t *order = reinterpret_cast<int32_t *>(ws + off_order);
     int32_t *offsets = reinterpret_cast<int32_t *>(ws + off_offsets);
     int32_t *active = reinterpret_cast<int32_t *>(ws + off_active);

@@ -104,6 +104,14 @@ struct Scratch {
 // library reserves covers what the launchers it picks ask for.  Thread-local, off by default.
 bool dry_run();
 void set_dry_run(bool on);
+size_t scratch_shave();   // dry runs: bytes withheld from the scratch the launchers are told they have (capacity-check tests)
+
+// Plan recorder: while one is installed on the calling thread (qproj_plan does that around a dry run of the
+// dispatch), every launcher writes down the launch it would make - kernel, tile, grid, cuts of K, scratch - as one
+// line.  The lines ARE the routing table: they come from the very code that serves a call.
+void plan_note(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+const char *plan_type_name(int type);
+void plan_note_cut();     // a launcher in a dry run: this launch keeps partial results of a cut K in scratch
 
 // Into how many stretches K is cut for a grid of `tiles` 128-token tiles (one workgroup a compute unit) that would
 // not fill the chip by itself: the cut that minimises rounds x (stretch + fixed cost) + the pass that adds the
@@ -201,7 +209,7 @@ hipError_t launch_moe_swiglu_gemv(const GemvArgs &gate_up, int mt, int n_experts
 // ALU: args as for the pair mode of the grouped kernel (t[0], and t[1] = up when `swiglu`; x fp32 rows, x_div, ids,
 // n_pairs, error_flag).  combine_weights null: t[0].y is [n_pairs][N]; otherwise the n_used consecutive pairs of a
 // token are added with their routing weights in slot order and t[0].y is [n_pairs / n_used][N].
-bool moe_decode_fits(int type, int64_t K, int64_t n_pairs, int64_t group);
+bool moe_decode_fits(int type, int64_t K, int64_t N, int64_t n_pairs, int64_t group, int64_t n_expert);
 hipError_t launch_moe_decode(const GemvArgs &args, int n_expert, bool swiglu, const float *combine_weights, int n_used,
                              hipStream_t s);
 hipError_t launch_moe_combine(const float *e, const float *weights, int64_t B, int64_t n_used, int64_t N,

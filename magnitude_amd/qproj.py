@@ -60,6 +60,8 @@ SYMBOLS = {
     "qproj_mul_mat_quantized": (_i32, [_vp, _i32, C.POINTER(_vp), _vp, _i32, _i64, C.POINTER(_vp)]),
     "qproj_mul_mat_id": (_i32, [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _vp, _i32]),
     "qproj_moe_ffn": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _i32]),
+    "qproj_plan_mul_mat": (_i32, [_i32, _i64, _i32, C.POINTER(_i64), _i64, _i32, _i32, C.c_char_p, _sz]),
+    "qproj_plan_moe_ffn": (_i32, [_i32, _i32, _i64, _i64, _i64, _i64, _i64, C.c_char_p, _sz]),
     "qproj_version": (C.c_char_p, []),
     "qproj_probe_eligibility": (_i32, [_vp]),
 }
@@ -149,6 +151,26 @@ def workspace_bytes(qtype: int, k: int, ns: Sequence[int], m: int, act: int = AC
     return nbytes
 
 
+def plan_mul_mat(qtype: int, k: int, ns: Sequence[int], m: int, act: int = ACT_GGML, with_norm: bool = False) -> str:
+    """The launches mul_mat_multi (or rms_norm_mul_mat) makes for this shape, one line each, as the launchers
+    themselves describe them in a dry run of the dispatch; the last line is the scratch reserved.  Needs no GPU."""
+    arr = (_i64 * len(ns))(*ns)
+    buf = C.create_string_buffer(8192)
+    st = load_library().qproj_plan_mul_mat(qtype, k, len(ns), arr, m, act, 1 if with_norm else 0, buf, len(buf))
+    if st:
+        raise QprojError(st, f"qproj_plan_mul_mat(type {qtype}, K {k}, N {list(ns)}, M {m}, act {act}): " + buf.value.decode())
+    return buf.value.decode()
+
+
+def plan_moe_ffn(gate_type: int, down_type: int, d_model: int, d_ff: int, n_expert: int, n_used: int, batch: int) -> str:
+    """The launches moe_ffn makes for this shape (see plan_mul_mat)."""
+    buf = C.create_string_buffer(8192)
+    st = load_library().qproj_plan_moe_ffn(gate_type, down_type, d_model, d_ff, n_expert, n_used, batch, buf, len(buf))
+    if st:
+        raise QprojError(st, f"qproj_plan_moe_ffn({gate_type}, {down_type}, {d_model}, {d_ff}, {n_expert}, {n_used}, {batch}): " + buf.value.decode())
+    return buf.value.decode()
+
+
 def row_bytes(qtype: int, k: int) -> int:
     return int(load_library().qproj_row_bytes(qtype, k))
 
@@ -194,6 +216,7 @@ class Context:
             raise QprojError(st, "qproj_ctx_create failed (is a gfx950 device visible?)")
         self.handle = h.value
         self.device = device
+        self._held = []     # contiguous copies handed to launches that may still be pending (dropped in sync())
 
     def close(self) -> None:
         if getattr(self, "handle", 0):
@@ -216,6 +239,16 @@ class Context:
 
     def sync(self) -> None:
         self._check(self.lib.qproj_sync(self.handle))
+        self._held.clear()
+
+    def _cptr(self, t: torch.Tensor) -> int:
+        """Device address of t made contiguous.  A copy made for that is kept alive until the next sync(): the launch
+        that reads it runs on the context's own stream, which torch's allocator does not track, so a temporary freed
+        when the ctypes call returns could be handed out again while the kernel is still reading it."""
+        c = t.contiguous()
+        if c is not t:
+            self._held.append(c)
+        return _ptr(c)
 
     # ---- weights -------------------------------------------------------------------------
     def upload(self, qtype: int, k: int, n: int, gguf: np.ndarray, n_expert: int = 1) -> Weight:
@@ -295,7 +328,7 @@ class Context:
         y = out if out is not None else torch.empty((m, w.N), dtype=torch.float32, device=x.device)
         if sync:
             torch.cuda.current_stream().synchronize()
-        self._check(self.lib.qproj_mul_mat(self.handle, w.handle, _ptr(x2.contiguous()), m, _ptr(y), act))
+        self._check(self.lib.qproj_mul_mat(self.handle, w.handle, self._cptr(x2), m, _ptr(y), act))
         if sync:
             self.sync()
         return y
@@ -328,7 +361,7 @@ class Context:
         y = out if out is not None else torch.empty_like(x)
         if sync:
             torch.cuda.current_stream().synchronize()
-        self._check(self.lib.qproj_rms_norm(self.handle, _ptr(x), 0 if gamma is None else _ptr(gamma.contiguous()),
+        self._check(self.lib.qproj_rms_norm(self.handle, _ptr(x), 0 if gamma is None else self._cptr(gamma),
                                             C.c_float(eps), m, k, _ptr(y)))
         if sync:
             self.sync()
@@ -346,7 +379,7 @@ class Context:
         if sync:
             torch.cuda.current_stream().synchronize()
         self._check(self.lib.qproj_rms_norm_quantize(self.handle, kind, wtype, _ptr(x),
-                                                     0 if gamma is None else _ptr(gamma.contiguous()),
+                                                     0 if gamma is None else self._cptr(gamma),
                                                      C.c_float(eps), m, k, _ptr(buf)))
         if sync:
             self.sync()
@@ -365,7 +398,7 @@ class Context:
         if sync:
             torch.cuda.current_stream().synchronize()
         self._check(self.lib.qproj_rms_norm_mul_mat(self.handle, n, wa, _ptr(x2),
-                                                    0 if gamma is None else _ptr(gamma.contiguous()),
+                                                    0 if gamma is None else self._cptr(gamma),
                                                     C.c_float(eps), m, ya, act))
         if sync:
             self.sync()
@@ -384,7 +417,7 @@ class Context:
             self._check(self.lib.qproj_ffn_gate_up(self.handle, gate.handle, up.handle, _ptr(x2), m, _ptr(h), act))
         else:
             self._check(self.lib.qproj_rms_norm_ffn_gate_up(self.handle, gate.handle, up.handle, _ptr(x2),
-                                                            0 if gamma is None else _ptr(gamma.contiguous()),
+                                                            0 if gamma is None else self._cptr(gamma),
                                                             C.c_float(eps), m, _ptr(h), act))
         if sync:
             self.sync()
@@ -429,7 +462,7 @@ class Context:
         if sync:
             torch.cuda.current_stream().synchronize()
         self._check(self.lib.qproj_ffn(self.handle, gate.handle, up.handle, down.handle, _ptr(x),
-                                       0 if gamma is None else _ptr(gamma.contiguous()),
+                                       0 if gamma is None else self._cptr(gamma),
                                        C.c_float(0.0 if eps is None else eps), 0 if eps is None else 1, m, _ptr(y), act))
         if sync:
             self.sync()
@@ -446,8 +479,8 @@ class Context:
         y = torch.empty((b, n_used, w.N), dtype=torch.float32, device=x.device)
         if sync:
             torch.cuda.current_stream().synchronize()
-        self._check(self.lib.qproj_mul_mat_id(self.handle, w.handle, _ptr(x.contiguous()), nb1,
-                                              _ptr(ids.contiguous()), n_used, b, _ptr(y), act))
+        self._check(self.lib.qproj_mul_mat_id(self.handle, w.handle, self._cptr(x), nb1,
+                                              self._cptr(ids), n_used, b, _ptr(y), act))
         if sync:
             self.sync()
         return y
@@ -465,8 +498,8 @@ class Context:
         if sync:
             torch.cuda.current_stream().synchronize()
         self._check(self.lib.qproj_moe_ffn(self.handle, gate.handle, up.handle, down.handle,
-                                           _ptr(x.contiguous()), _ptr(ids.contiguous()),
-                                           _ptr(weights.contiguous()), n_used, b, _ptr(y), act))
+                                           self._cptr(x), self._cptr(ids),
+                                           self._cptr(weights), n_used, b, _ptr(y), act))
         if sync:
             self.sync()
         return y

@@ -77,6 +77,10 @@ extern "C" {
                                        x_dev: *const f32, m: i64, y_dev: *const *mut f32, act: c_int) -> c_int;
     pub fn qproj_workspace_bytes(ty: c_int, k: i64, n: c_int, rows: *const i64, m: i64, act: c_int,
                                  status: *mut c_int) -> usize;
+    pub fn qproj_plan_mul_mat(ty: c_int, k: i64, n: c_int, rows: *const i64, m: i64, act: c_int, with_norm: c_int,
+                              buf: *mut c_char, buf_bytes: usize) -> c_int;
+    pub fn qproj_plan_moe_ffn(gate_ty: c_int, down_ty: c_int, d_model: i64, d_ff: i64, n_expert: i64, n_used: i64,
+                              b: i64, buf: *mut c_char, buf_bytes: usize) -> c_int;
     pub fn qproj_mul_mat_quantized(ctx: *mut qproj_ctx, n: c_int, w: *const *const qproj_weight,
                                    act_dev: *const c_void, kind: c_int, m: i64, y_dev: *const *mut f32) -> c_int;
     pub fn qproj_mul_mat_id(ctx: *mut qproj_ctx, w: *const qproj_weight, x_dev: *const f32, nb1: i64,

@@ -78,3 +78,61 @@ def test_the_8b_layer_fits_the_fixed_scratch_up_to_512_tokens():
         for qt, k, ns in groups:
             assert qproj.workspace_bytes(qt, k, ns, m, GGML) <= qproj.NOALLOC_SCRATCH_BYTES, (m, qt, k, ns)
     assert qproj.workspace_bytes(Q6_K, 14336, (4096,), 4096, GGML) > qproj.NOALLOC_SCRATCH_BYTES   # and larger ones are refused
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# The routing table: which kernel, tile, grid and cuts of K serve every shape of the benchmark configurations.  The
+# lines are written by the launchers themselves in a dry run of the dispatch (qproj_plan_mul_mat / qproj_plan_moe_ffn),
+# so an edit of a routing threshold shows up as a diff of tests/golden/dispatch_plan.txt.
+# Regenerate after a deliberate change with:  QPROJ_UPDATE_PLAN=1 python -m pytest tests/test_dispatch_cpu.py -k routing_table
+def routing_table() -> str:
+    out = []
+
+    def dense(title, qtype, k, ns, m, act=GGML, with_norm=False):
+        out.append(f"## {title}: {'Q8_0' if qtype == Q8_0 else 'Q4_K' if qtype == Q4_K else 'Q6_K'} K={k} N={list(ns)} M={m} "
+                   f"act={'ggml' if act == GGML else 'f32' if act == F32 else 'q8x32'}{' +rms_norm' if with_norm else ''}")
+        out.append(qproj.plan_mul_mat(qtype, k, ns, m, act, with_norm).rstrip())
+
+    layer = [("q/k/v", Q4_K, 4096, (4096, 1024, 1024)), ("o", Q4_K, 4096, (4096,)), ("gate/up", Q4_K, 4096, (14336, 14336)),
+             ("down", Q6_K, 14336, (4096,))]
+    dense("config 1", Q8_0, 4096, (4096,), 1)
+    for name, qt, k, ns in layer:
+        dense(f"config 2 {name}", qt, k, ns, 1)
+    dense("config 2 norm + q/k/v", Q4_K, 4096, (4096, 1024, 1024), 1, with_norm=True)
+    dense("config 2 norm + gate/up", Q4_K, 4096, (14336, 14336), 1, with_norm=True)
+    for m in (2, 4, 8, 16):
+        for name, qt, k, ns in layer:
+            dense(f"config 3 {name}", qt, k, ns, m)
+    for m in (512, 2048, 4096):
+        for k, n in ((4096, 14336), (14336, 4096), (4096, 4096)):
+            dense("config 4 (per-32 activations)", Q4_K, k, (n,), m, Q8X32)
+            dense("config 4 (ggml activations)", Q4_K, k, (n,), m)
+        dense("config 4 (ggml activations) down", Q6_K, 14336, (4096,), m)
+        dense("config 4 (ggml activations) config 1's matrix", Q8_0, 4096, (4096,), m)
+    for name, qt, k, ns in layer:
+        dense(f"prompt batch of the engine (512 tokens) {name}", qt, k, ns, 512)
+    for b in (1, 8, 64):
+        out.append(f"## config 5: 128 experts, top-8, d_model 2048, d_ff 768, Q4_K, B={b}")
+        out.append(qproj.plan_moe_ffn(Q4_K, Q4_K, 2048, 768, 128, 8, b).rstrip())
+    return "\n".join(out) + "\n"
+
+
+def test_routing_table_of_the_benchmark_configurations_is_pinned():
+    import os
+    path = os.path.join(os.path.dirname(__file__), "golden", "dispatch_plan.txt")
+    table = routing_table()
+    if os.environ.get("QPROJ_UPDATE_PLAN"):
+        with open(path, "w") as f:
+            f.write(table)
+    with open(path) as f:
+        pinned = f.read()
+    assert table == pinned, "the dispatch changed: review the diff, then regenerate tests/golden/dispatch_plan.txt"
+    # every shape is served (no refusal) and the decode regime stays one launch
+    assert "refused" not in table
+    first = table.split("## config 2 q/k/v")[1].split("##")[0]
+    assert first.count("gemv_decode_kernel") == 1 and "quantizer:" not in first
+
+
+def test_plan_reports_a_refused_call():
+    with pytest.raises(qproj.QprojError):
+        qproj.plan_mul_mat(Q6_K, 4096, (4096,), 64, Q8X32)

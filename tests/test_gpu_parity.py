@@ -385,6 +385,32 @@ def test_two_k_chunks_add_themselves_like_the_summing_launch(ctx, qtype, k, n, m
     w.free()
 
 
+def test_outputs_that_overlap_the_activations_keep_the_storing_route(ctx):
+    """Where two K parts add themselves to the output, the launch that quantizes x also clears y - so y would be
+    written while x is still being read.  A call whose output overlaps its input must therefore not take that route:
+    the quantizer reads all of x first, the projection stores y afterwards, and the result is that of a call with
+    separate buffers.  (8 rows of the 14336 -> 4096 Q6_K matrix: the small-batch kernel with two K chunks; 192 rows of
+    4096 x 4096 Q4_K: two K stretches of a tile.)"""
+    from magnitude_amd import ACT_GGML, synth
+    for qtype, k, n, m in ((Q6_K, 14336, 4096, 8), (Q4_K, 4096, 4096, 192)):
+        w = ctx.upload_from_device(qtype, k, n, synth.random_weight(qtype, n, k, seed=8300 + m, device="cuda"))
+        g = torch.Generator(device="cuda")
+        g.manual_seed(m)
+        x = torch.randn((m, k), generator=g, device="cuda")
+        want = ctx.mul_mat(w, x, ACT_GGML)
+        buf = torch.empty(max(m * k, m * n) + 64, device="cuda")
+        xa = buf[: m * k].view(m, k)
+        xa.copy_(x)
+        ya = buf[: m * n].view(m, n)                      # the output starts where the input starts
+        ctx.mul_mat(w, xa, ACT_GGML, out=ya)
+        assert torch.allclose(ya, want, rtol=1e-5, atol=1e-6), (qtype, m)   # (the two routes differ in fp32 order only)
+        xa.copy_(x)
+        yt = buf[64: 64 + m * n].view(m, n)               # ... and a shifted overlap
+        ctx.mul_mat(w, xa, ACT_GGML, out=yt)
+        assert torch.allclose(yt, want, rtol=1e-5, atol=1e-6), (qtype, m, "shifted")
+        w.free()
+
+
 @pytest.mark.parametrize("m,k,ns", [(192, 4096, (4096,)), (64, 4096, (14336,)), (256, 14336, (4096,)),
                                      (192, 4096, (4096, 1024, 1024)), (130, 4096, (14336, 14336))])
 def test_two_k_stretches_of_a_tile_add_themselves(ctx, m, k, ns):
@@ -965,7 +991,8 @@ def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):
         ys = {"dec": torch.empty((1, n), device="cuda"), "small": torch.empty((8, n6), device="cuda"),
               "tiled6": torch.empty((200, n6), device="cuda"), "tiled4": torch.empty((200, n6), device="cuda"),
               "per32": torch.empty((200, n6), device="cuda"), "moe": torch.empty((B, d_model), device="cuda"),
-              "small_add": torch.empty((8, 4096), device="cuda"), "tiled_add": torch.empty((192, 4096), device="cuda")}
+              "small_add": torch.empty((8, 4096), device="cuda"), "tiled_add": torch.empty((192, 4096), device="cuda"),
+              "small_noalloc": torch.empty((8, n6), device="cuda"), "tiled_noalloc": torch.empty((200, n6), device="cuda")}
 
         def fill(seed):
             gen = torch.Generator(device="cuda").manual_seed(seed)
@@ -982,6 +1009,10 @@ def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):
             c.moe_ffn(g, u, d, xs["moe"], ids_d, wts_d, ACT_GGML, out=ys["moe"], sync=False)
             c.mul_mat(w6big, xs["small"], ACT_GGML, out=ys["small_add"], sync=False)
             c.mul_mat(w4sq, xs["mid"], ACT_GGML, out=ys["tiled_add"], sync=False)
+            # the allocation-free entry point is what a caller under capture is meant to use: chunks of K and partial
+            # tiles in the library's fixed buffer
+            c.mul_mat_multi([w6], xs["small"], ACT_GGML, outs=[ys["small_noalloc"]], sync=False, noalloc=True)
+            c.mul_mat_multi([w4l], xs["tiled"], ACT_GGML, outs=[ys["tiled_noalloc"]], sync=False, noalloc=True)
 
         def eager(seed):
             fill(seed)
@@ -1004,6 +1035,7 @@ def test_calls_replayed_from_a_hip_graph_give_the_eager_results(orc, moe):
             for name, t in ys.items():
                 assert torch.equal(t, want[name]), f"replay with inputs {seed}: {name} differs from the eager call"
             assert float(ys["moe"].abs().sum()) > 0
+            assert torch.equal(ys["small_noalloc"], ys["small"]) and torch.equal(ys["tiled_noalloc"], ys["tiled4"])
     finally:
         c.close()
 

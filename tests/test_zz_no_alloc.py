@@ -95,3 +95,27 @@ def test_noalloc_refuses_what_does_not_fit(ctx):
     want = ctx.mul_mat_multi([w], x[:64], ACT_GGML)[0]
     assert torch.equal(got.view(torch.int32), want.view(torch.int32))
     w.free()
+
+
+def test_noalloc_scratch_belongs_to_one_context_at_a_time(ctx):
+    """Two contexts launch on two streams; their calls would overwrite each other's scratch in the one fixed buffer
+    of the GPU with no error anywhere.  The buffer belongs to the first context that uses it until that context is
+    destroyed: a second context is refused, and served once the first is gone."""
+    from magnitude_amd import ACT_GGML, Context, QprojError
+    w = upload(ctx, Q4_K, 512, 4096, seed=8)
+    x = torch.randn((8, 4096), device="cuda")
+    want = ctx.mul_mat_multi([w], x, ACT_GGML, noalloc=True)[0]           # this module's context owns the buffer
+    other = Context(0)
+    try:
+        w2 = upload(other, Q4_K, 512, 4096, seed=8)
+        with pytest.raises(QprojError) as e:
+            other.mul_mat_multi([w2], x, ACT_GGML, noalloc=True)
+        assert e.value.status == 4 and "another context" in str(e.value)
+        got = other.mul_mat_multi([w2], x, ACT_GGML)[0]                    # its allocating route is untouched
+        assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+        w2.free()
+    finally:
+        other.close()
+    again = ctx.mul_mat_multi([w], x, ACT_GGML, noalloc=True)[0]
+    assert torch.equal(again.view(torch.int32), want.view(torch.int32))
+    w.free()
