@@ -140,6 +140,60 @@ impl Context {
                                y.0.cast(), Activation::Ggml as c_int)
         })
     }
+
+    /// RMS norm (llama.cpp's `build_norm`, `LLM_NORM_RMS`) followed by the projections that read the normalised rows.
+    #[allow(clippy::too_many_arguments)]
+    pub fn rms_norm_mul_mat(&self, w: &[&Weight<'_>], x: DevicePtr, gamma: DevicePtr, eps: f32, m: i64, y: &[DevicePtr],
+                            act: Activation) -> Result<()> {
+        if w.is_empty() || w.len() > 4 || w.len() != y.len() {
+            return Err(QprojError { status: sys::QPROJ_ERR_INVALID_ARG, message: "one to four tensors, one output each".into() });
+        }
+        let ws: Vec<*const sys::qproj_weight> = w.iter().map(|t| t.raw as *const _).collect();
+        let ys: Vec<*mut f32> = y.iter().map(|p| p.0.cast()).collect();
+        self.check(unsafe {
+            sys::qproj_rms_norm_mul_mat(self.raw, ws.len() as c_int, ws.as_ptr(), x.0.cast(), gamma.0.cast(), eps, m, ys.as_ptr(),
+                                        act as c_int)
+        })
+    }
+
+    /// llama.cpp's `build_ffn` of a dense layer: (norm,) gate, up, swiglu, down.  `gamma`: the norm weights, or `None`
+    /// for rows that are already normalised.
+    #[allow(clippy::too_many_arguments)]
+    pub fn ffn(&self, gate: &Weight<'_>, up: &Weight<'_>, down: &Weight<'_>, x: DevicePtr, gamma: Option<DevicePtr>, eps: f32,
+               m: i64, y: DevicePtr) -> Result<()> {
+        let (g, use_norm) = match gamma {
+            Some(p) => (p.0 as *const f32, 1),
+            None => (ptr::null(), 0),
+        };
+        self.check(unsafe {
+            sys::qproj_ffn(self.raw, gate.raw, up.raw, down.raw, x.0.cast(), g, eps, use_norm, m, y.0.cast(),
+                           Activation::Ggml as c_int)
+        })
+    }
+}
+
+/// Scratch bytes a `mul_mat` of this shape needs at most (what `mul_mat_noalloc` holds against its fixed buffer).
+pub fn workspace_bytes(ty: WeightType, k: i64, rows: &[i64], m: i64, act: Activation) -> Result<usize> {
+    let mut st: c_int = sys::QPROJ_OK;
+    let bytes = unsafe { sys::qproj_workspace_bytes(ty as c_int, k, rows.len() as c_int, rows.as_ptr(), m, act as c_int, &mut st) };
+    if st != sys::QPROJ_OK {
+        return Err(QprojError { status: st, message: "qproj_workspace_bytes".into() });
+    }
+    Ok(bytes)
+}
+
+/// Which kernels a `mul_mat` of this shape would launch, one launch a line; needs no GPU.
+pub fn plan_mul_mat(ty: WeightType, k: i64, rows: &[i64], m: i64, act: Activation, with_norm: bool) -> Result<String> {
+    let mut buf = vec![0u8; 4096];
+    let st = unsafe {
+        sys::qproj_plan_mul_mat(ty as c_int, k, rows.len() as c_int, rows.as_ptr(), m, act as c_int, with_norm as c_int,
+                                buf.as_mut_ptr().cast(), buf.len())
+    };
+    let text = CStr::from_bytes_until_nul(&buf).map(|c| c.to_string_lossy().into_owned()).unwrap_or_default();
+    if st != sys::QPROJ_OK {
+        return Err(QprojError { status: st, message: text });
+    }
+    Ok(text)
 }
 
 impl Drop for Context {
