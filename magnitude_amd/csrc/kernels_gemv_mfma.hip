@@ -56,6 +56,7 @@ struct MfmaArgs {
     ActView a;
     const float *x;        // non-null: fp32 activation rows [rows][K], quantized by every workgroup in its prologue
     int M, n_chunks, chunk_sb, kw, rw, n_wgs;
+    int rpg;               // weight rows a row group (32 fill the matrix instruction; dense launches may take fewer, below)
     int add_out;           // dense mode, two chunks, output rows cleared before the launch: both chunks add to y
     int64_t part_plane;    // expert-grouped mode with K in chunks: floats of one chunk's results, [n_pairs][N], in t[0].part
     // expert-grouped mode (MUL_MAT_ID): activation rows of expert e are the pairs order[offsets[e]..offsets[e+1])
@@ -652,7 +653,7 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
     Stager<QT> sa, sb_;
     // the wave's rg-th row group: rows, how much of K, where its blocks start
     auto set_rowgroup = [&](int rg) {
-        row0 = ((rs * (GROUPED ? g.rg_loop : 1) + rg) * g.rw + rgl) * 32;
+        row0 = ((rs * (GROUPED ? g.rg_loop : 1) + rg) * g.rw + rgl) * (GROUPED ? 32 : g.rpg);
         rows_ok = row0 < N;
         steps = rows_ok ? s1 - s0 : 0;
         items = NT * steps;                       // (tensor, super-block) pairs this wave streams
@@ -660,10 +661,11 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
         const int64_t row = (int64_t)expert * N + (rows_ok ? row0 : 0);
         sa.rebase(0, w, row);
         sa.rebase(1, SWIGLU ? g.t[1].w : w, row);
-        sa.init(w, rows_ok ? min(31, N - 1 - row0) : 0, lane);
+        const int last_row = rows_ok ? min((GROUPED ? 32 : g.rpg) - 1, N - 1 - row0) : 0;   // rows past it repeat it
+        sa.init(w, last_row, lane);
         sb_.rebase(0, w, row);
         sb_.rebase(1, SWIGLU ? g.t[1].w : w, row);
-        sb_.init(w, rows_ok ? min(31, N - 1 - row0) : 0, lane);
+        sb_.init(w, last_row, lane);
     };
     // item i -> tensor i / steps, super-block c0 + s0 + i % steps (clamped: harmless repeats past the end)
     auto issue = [&](Stager<QT> &st, int i) {
@@ -873,7 +875,7 @@ __global__ __launch_bounds__(W * 64) void gemv_mfma_kernel(const MfmaArgs g) {
                 const int m = 8 * (v >> 2) + 4 * h + (v & 3);
                 float r = out[0][v];
                 if constexpr (SWIGLU) r = (r / (1.0f + expf(-r))) * out[NT - 1][v];
-                if (m < m_cnt && n < N) {
+                if (m < m_cnt && n < N && (GROUPED || nl < g.rpg)) {
                     float *o = dst + (size_t)(GROUPED ? map[m] : m0 + m) * N + n;
                     // two addends on zero: the sum does not depend on which chunk arrives first
                     if (add) unsafeAtomicAdd(o, r);
@@ -907,9 +909,9 @@ hipError_t launch_one(const MfmaArgs &g, hipStream_t s) {
     if (g.kw > 1 && (MODE == kGroupedSwiglu ? 2 : 1) * (8 * NI) * 32 * 4 > Cfg<QT>::kRegion) return hipErrorInvalidValue;
     if (dry_run()) {
         if (g.n_chunks > 1 && !g.add_out) plan_note_cut();
-        plan_note("gemv_mfma_kernel<%s, %d staged rows, %d waves, %s%s>: %d workgroups, K in %d chunk(s) of %d super-blocks x %d parts a row group%s",
+        plan_note("gemv_mfma_kernel<%s, %d staged rows, %d waves, %s%s>: %d workgroups, K in %d chunk(s) of %d super-blocks x %d parts a row group of %d rows%s",
                   plan_type_name(QT), 8 * NI, W, MODE == kDense ? "dense" : MODE == kGroupedSwiglu ? "expert-grouped + swiglu" : "expert-grouped",
-                  FLAT ? ", one item stream a wave" : "", g.n_wgs, g.n_chunks, g.chunk_sb, g.kw,
+                  FLAT ? ", one item stream a wave" : "", g.n_wgs, g.n_chunks, g.chunk_sb, g.kw, MODE == kDense ? g.rpg : 32,
                   g.n_chunks == 1 ? "" : g.add_out ? ", the two chunks add themselves to cleared rows"
                                    : MODE == kDense ? " + sum_chunks_kernel" : " + sum_parts_kernel");
         return hipSuccess;
@@ -1064,6 +1066,19 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStr
     g.rw = W / p.kw;
     g.rg_loop = 1;
     g.add_out = args.y_zeroed && mfma_gemv_two_chunks(args.t[0].w.type, args.a.K, args.M, total_rg);
+    // Rows a row group.  The kernel streams weights and the matrix cores idle, so a grid that leaves compute units
+    // without a workgroup is evened out with row groups of fewer than the instruction's 32 rows (the spare columns
+    // repeat the group's last row and are not stored): the fewest rows, 24 at least, whose grid is still one round.
+    // Gate + up of 14336 rows each are 896 groups of 32 = 224 workgroups, and 1024 groups of 28 = 256.
+    const auto wgs_with = [&](int rpg) {
+        int64_t n = 0;
+        for (int i = 0; i < args.n_targets; ++i) n += ((args.t[i].w.N + rpg - 1) / rpg + g.rw - 1) / g.rw;
+        return n * g.n_chunks;
+    };
+    g.rpg = 32;
+    static const bool even_out = tuning_int("QPROJ_MFMA_NO_SHORT_GROUPS", 0) == 0;
+    if (even_out && wgs_with(32) < cu_count())
+        for (int r = 31; r >= 24 && wgs_with(r) <= cu_count(); --r) g.rpg = r;
     int wg = 0;
     size_t part_off = 0;
     for (int i = 0; i < args.n_targets; ++i) {
@@ -1071,7 +1086,7 @@ hipError_t launch_gemv_mfma(const GemvArgs &args, const Scratch &scratch, hipStr
         g.t[i].y = args.t[i].y;
         g.t[i].part = scratch.p ? scratch.p + part_off : nullptr;
         part_off += (size_t)g.n_chunks * args.M * args.t[i].w.N;
-        const int n_rg = (int)((args.t[i].w.N + 31) / 32);
+        const int n_rg = (int)((args.t[i].w.N + g.rpg - 1) / g.rpg);
         g.t[i].n_rowsets = (n_rg + g.rw - 1) / g.rw;
         g.t[i].first_wg = wg;
         wg += g.t[i].n_rowsets * g.n_chunks;

@@ -252,6 +252,37 @@ def test_mul_mat_ggml_mode_matches_oracle(ctx, orc, qtype, m):
         w.free()
 
 
+@pytest.mark.parametrize("qtype,k,ns", [(Q4_K, 4096, (4097,)), (Q4_K, 2048, (3001, 1000)), (Q6_K, 2048, (3000,)),
+                                        (Q8_0, 4096, (5000,)), (Q4_K, 4096, (6143, 6145))])
+def test_small_batch_row_groups_of_fewer_than_32_rows(ctx, orc, qtype, k, ns):
+    """A grid of the small-batch kernel that would leave compute units without a workgroup is evened out with row
+    groups of 24..31 rows (the spare columns of the matrix instruction repeat a row and are not stored).  Shapes whose
+    plan says so, with ragged last groups and two matrices in one launch, against the oracle; rows past the end of a
+    matrix stay untouched."""
+    import re
+    from magnitude_amd import ACT_GGML, qproj
+    for m in (5, 8, 16, 27):
+        plan = qproj.plan_mul_mat(qtype, k, list(ns), m, ACT_GGML)
+        rows = [int(r) for r in re.findall(r"a row group of (\d+) rows", plan)]
+        assert rows and all(24 <= r < 32 for r in rows), plan
+        ws, blocks = [], []
+        for i, n in enumerate(ns):
+            blocks.append(make_weight(orc, qtype, n, k, seed=2400 + k + n + i))
+            ws.append(ctx.upload(qtype, k, n, blocks[-1]))
+        rng = np.random.default_rng(m + k + ns[0])
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        # outputs inside larger buffers: what lies behind them must not change
+        bufs = [torch.full((m * n + 64,), 7.0, dtype=torch.float32, device="cuda") for n in ns]
+        outs = [b[: m * n].view(m, n) for b, n in zip(bufs, ns)]
+        ctx.mul_mat_multi(ws, dev(x), ACT_GGML, outs=outs)
+        for b, o, n, blk in zip(bufs, outs, ns, blocks):
+            want = orc.mul_mat(qtype, blk, k, x, orc.ACT_GGML)
+            close(o.cpu().numpy(), want, 2e-5)
+            assert bool((b[m * n:] == 7.0).all())
+        for w in ws:
+            w.free()
+
+
 @pytest.mark.parametrize("qtype,k,n", [(Q4_K, 4096, 512), (Q4_K, 14336, 203), (Q4_K, 256, 9), (Q8_0, 4096, 384),
                                        (Q8_0, 14336, 77), (Q6_K, 4096, 130), (Q6_K, 14336, 256)])
 def test_rows_17_to_32_on_the_small_batch_kernel(ctx, orc, qtype, k, n):
