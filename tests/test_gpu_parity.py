@@ -263,7 +263,7 @@ def test_small_batch_row_groups_of_fewer_than_32_rows(ctx, orc, qtype, k, ns):
     from magnitude_amd import ACT_GGML, qproj
     for m in (5, 8, 16, 27):
         plan = qproj.plan_mul_mat(qtype, k, list(ns), m, ACT_GGML)
-        rows = [int(r) for r in re.findall(r"a row group of (\d+) rows", plan)]
+        rows = [int(r) for r in re.findall(r"row group(?:\(s\))? of (\d+) rows", plan)]
         assert rows and all(24 <= r < 32 for r in rows), plan
         ws, blocks = [], []
         for i, n in enumerate(ns):
