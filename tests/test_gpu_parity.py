@@ -135,6 +135,33 @@ def test_upload_rejects_bad_arguments(ctx, orc):
         ctx.upload(Q4_K, 100, 4, blocks)
 
 
+def test_empty_batches_are_accepted_and_touch_nothing(ctx, orc):
+    """A scheduler step may carry no rows for a layer (ggml computes a MUL_MAT with ne1 = 0 as a no-op): M = 0 and
+    B = 0 return success without writing; negative counts are refused."""
+    import ctypes as C
+    from magnitude_amd import ACT_GGML
+    QPROJ_ERR_INVALID_ARG = 1   # include/qproj.h
+    k, n, e = 256, 64, 4
+    w = ctx.upload(Q4_K, k, n, make_weight(orc, Q4_K, n, k, seed=3))
+    we = ctx.upload(Q4_K, k, n, make_weight(orc, Q4_K, n * e, k, seed=4), n_expert=e)
+    x = torch.ones((4, k), device="cuda")
+    y = torch.full((4, n), 7.0, device="cuda")
+    ids = torch.zeros((4, 2), dtype=torch.int32, device="cuda")
+    wa = (C.c_void_p * 1)(w.handle)
+    ya = (C.c_void_p * 1)(y.data_ptr())
+    lib, h = ctx.lib, ctx.handle
+    assert lib.qproj_mul_mat(h, w.handle, x.data_ptr(), 0, y.data_ptr(), ACT_GGML) == 0
+    assert lib.qproj_mul_mat_multi(h, 1, wa, x.data_ptr(), 0, ya, ACT_GGML) == 0
+    assert lib.qproj_mul_mat_id(h, we.handle, x.data_ptr(), 1, ids.data_ptr(), 2, 0, y.data_ptr(), ACT_GGML) == 0
+    ctx.sync()
+    assert bool((y == 7.0).all())
+    assert lib.qproj_mul_mat(h, w.handle, x.data_ptr(), -1, y.data_ptr(), ACT_GGML) == QPROJ_ERR_INVALID_ARG
+    assert lib.qproj_mul_mat_id(h, we.handle, x.data_ptr(), 1, ids.data_ptr(), 2, -1, y.data_ptr(), ACT_GGML) == QPROJ_ERR_INVALID_ARG
+    assert bool((y == 7.0).all())
+    w.free()
+    we.free()
+
+
 # ---------------------------------------------------------------- activation quantizers
 
 def activation_cases(rng, m, k):
